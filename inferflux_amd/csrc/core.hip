@@ -1,0 +1,240 @@
+// Row-wise kernels of the decoder: embedding gather, residual add + RMSNorm, bias + rotary
+// position encoding + append to the paged cache, SwiGLU.  All math in float; the residual
+// stream is float in every mode.
+//
+// Formulas follow the reference's dense path:
+//   embedding  runtime/backends/cuda/native/cuda_kernels.cu:255-270, 674-689
+//   RMSNorm    cuda_kernels.cu:15-48 (eps inside the square root, line 41)
+//   residual add + norm  cuda_kernels.cu:193-249, 617-671
+//   bias       cuda_kernels.cu:518-527
+//   RoPE       cuda_kernels.cu:71-117 (split-half pairing 102-105), fused with the cache write
+//              as in runtime/backends/cuda/native/kernels/fused_rope_kv_append.cuh:26-166
+//   SwiGLU     cuda_kernels.cu:139-151
+#include "common.h"
+
+IFX_DEFINE_LAST_ERROR()
+
+// ---------------------------------------------------------------------------------------
+// out[t, :] = float(table[ids[t], :])
+template <typename T>
+__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  const T* src = table + (size_t)ids[t] * H;
+  float* dst = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f(src[i]);
+}
+
+extern "C" int ifx_embedding(const int* ids, const void* table, int table_dtype, float* out, int T,
+                             int H, void* stream) {
+  IFX_REQUIRE(T >= 0 && H > 0, "embedding: bad sizes T=%d H=%d", T, H);
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (table_dtype == DT_F32)
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T), dim3(256), 0, s, ids, (const float*)table, out, H);
+  else if (table_dtype == DT_BF16)
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids, (const bf16_t*)table, out, H);
+  else
+    IFX_FAIL("embedding: unknown dtype %d", table_dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// x = residual[src] (+ delta[src]);  if write_back: residual[src] = x
+// out[r, :] = x * rsqrt(mean(x^2) + eps) * weight         src = rows ? rows[r] : r
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                   const void* __restrict__ weight, int weight_dtype,
+                                   TO* __restrict__ out, const int* __restrict__ rows, int H, float eps,
+                                   int write_back) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* res = residual + src * H;
+  const TD* dl = delta ? delta + src * H : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x = res[i];
+    if (dl) {
+      x += to_f(dl[i]);
+      if (write_back) res[i] = x;
+    }
+    ss += x * x;
+  }
+  ss = block_sum(ss, red);
+  const float rms = rsqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x = res[i];
+    if (dl && !write_back) x += to_f(dl[i]);
+    o[i] = from_f<TO>(x * rms * load_dyn(weight, weight_dtype, i));
+  }
+}
+
+extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* weight,
+                               int weight_dtype, void* out, int out_dtype, const int* rows, int n_rows,
+                               int H, float eps, int write_back, void* stream) {
+  IFX_REQUIRE(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  IFX_REQUIRE(!(rows && write_back), "add_rmsnorm: a row gather cannot write the residual back");
+  if (n_rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = H >= 2048 ? 512 : 256;
+#define LAUNCH(TD, TO)                                                                              \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(threads), 0, s, residual,     \
+                     (const TD*)delta, weight, weight_dtype, (TO*)out, rows, H, eps, write_back)
+  const int dd = delta ? delta_dtype : out_dtype;
+  if (dd == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
+  else if (dd == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (dd == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
+  else if (dd == DT_BF16 && out_dtype == DT_F32) LAUNCH(bf16_t, float);
+  else IFX_FAIL("add_rmsnorm: unknown dtypes delta=%d out=%d", delta_dtype, out_dtype);
+#undef LAUNCH
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// Per token t: qkv[t] = [q (nH*d) | k (nKV*d) | v (nKV*d)].  Adds the bias, rotates q and k by
+// the token's position, writes q to q_out[t] and k, v into the paged cache at slot[t]
+// (slot = page * page_size + offset; slot < 0: nothing is written to the cache).
+// Cache layouts: K [page][kv head][offset][d], V [page][kv head][d][offset].
+// rope_style: 0 none, 1 split-half pairs (p, p + rot/2), 2 consecutive pairs (2p, 2p+1);
+// angle = float(position) * inv_freq[p]; elements at or beyond rotary_dim are copied.
+struct RopeArgs {
+  const void* qkv;
+  const void* bias;
+  int bias_dtype;
+  const int* positions;
+  const int* slots;
+  const float* inv_freq;
+  int rope_style;
+  int rotary_dim;
+  int nH, nKV, d, page_size;
+  void* q_out;
+  void* k_cache;
+  void* v_cache;
+};
+
+template <typename T>
+__global__ void rope_append_kernel(RopeArgs a) {
+  const int t = blockIdx.x;
+  const int d = a.d, half = d / 2, rot_half = a.rotary_dim / 2;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
+  const T* row = (const T*)a.qkv + (size_t)t * row_width;
+  const float pos = (float)a.positions[t];
+  const int slot = a.slots ? a.slots[t] : -1;
+  const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
+  T* qo = (T*)a.q_out + (size_t)t * q_width;
+
+  const int n_rot_items = (a.nH + a.nKV) * half;
+  for (int it = threadIdx.x; it < n_rot_items; it += blockDim.x) {
+    const int head = it / half, p = it % half;
+    const bool is_q = head < a.nH;
+    if (!is_q && slot < 0) continue;
+    int i0, i1;
+    bool rotate = a.rope_style != 0 && p < rot_half;
+    if (rotate) {
+      if (a.rope_style == 1) { i0 = p; i1 = p + rot_half; }
+      else { i0 = 2 * p; i1 = 2 * p + 1; }
+    } else {
+      const int base = a.rope_style != 0 ? a.rotary_dim + 2 * (p - rot_half) : 2 * p;
+      i0 = base; i1 = base + 1;
+    }
+    const int col = head * d;  // q heads first, then k heads: the same offset rule
+    float x0 = to_f(row[col + i0]), x1 = to_f(row[col + i1]);
+    if (a.bias) {
+      x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
+      x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
+    }
+    float y0 = x0, y1 = x1;
+    if (rotate) {
+      float sn, cs;
+      sincosf(pos * a.inv_freq[p], &sn, &cs);
+      y0 = x0 * cs - x1 * sn;
+      y1 = x0 * sn + x1 * cs;
+    }
+    if (is_q) {
+      qo[col + i0] = from_f<T>(y0);
+      qo[col + i1] = from_f<T>(y1);
+    } else {
+      const int kh = head - a.nH;
+      T* kc = (T*)a.k_cache + (((size_t)page * a.nKV + kh) * a.page_size + off) * d;
+      kc[i0] = from_f<T>(y0);
+      kc[i1] = from_f<T>(y1);
+    }
+  }
+  if (slot >= 0) {
+    for (int it = threadIdx.x; it < kv_width; it += blockDim.x) {
+      const int kh = it / d, e = it % d;
+      const int col = q_width + kv_width + it;
+      float x = to_f(row[col]);
+      if (a.bias) x += load_dyn(a.bias, a.bias_dtype, col);
+      T* vc = (T*)a.v_cache + (((size_t)page * a.nKV + kh) * d + e) * a.page_size + off;
+      *vc = from_f<T>(x);
+    }
+  }
+}
+
+extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype,
+                               const int* positions, const int* slots, const float* inv_freq,
+                               int rope_style, int rotary_dim, int T, int nH, int nKV, int d,
+                               int page_size, void* q_out, void* k_cache, void* v_cache, void* stream) {
+  IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
+  IFX_REQUIRE(rope_style >= 0 && rope_style <= 2, "rope_append: unknown rope style %d", rope_style);
+  IFX_REQUIRE(rope_style == 0 || (rotary_dim > 0 && rotary_dim <= d && rotary_dim % 2 == 0 && inv_freq),
+              "rope_append: rotary_dim %d must be even, within head_dim %d, with a frequency table", rotary_dim, d);
+  IFX_REQUIRE(!slots || (page_size > 0 && k_cache && v_cache), "rope_append: cache write without cache");
+  if (T == 0) return 0;
+  RopeArgs a{qkv, bias, bias_dtype, positions, slots, inv_freq, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32) hipLaunchKernelGGL(rope_append_kernel<float>, dim3(T), dim3(256), 0, s, a);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(rope_append_kernel<bf16_t>, dim3(T), dim3(256), 0, s, a);
+  else IFX_FAIL("rope_append: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// gu[t] = [gate (I) | up (I)];  out[t, i] = gate / (1 + exp(-gate)) * up
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const size_t t = idx / I;
+  const int i = (int)(idx % I);
+  const float g = to_f(gu[t * 2 * I + i]);
+  const float u = to_f(gu[t * 2 * I + I + i]);
+  out[idx] = from_f<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, void* stream) {
+  IFX_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  if (T == 0) return 0;
+  const size_t n = (size_t)T * I;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n);
+  else IFX_FAIL("swiglu: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// out = float(in) or bf16(in), elementwise: the only cast the engine needs outside a kernel's
+// own epilogue (a bf16 activation in front of a matrix that the file stores in 32-bit).
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < n) out[idx] = from_f<TO>(to_f(in[idx]));
+}
+
+extern "C" int ifx_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n, void* stream) {
+  IFX_REQUIRE(n >= 0, "cast: bad size");
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (in_dtype == DT_F32 && out_dtype == DT_BF16)
+    hipLaunchKernelGGL((cast_kernel<float, bf16_t>), dim3(blocks), dim3(256), 0, s, (const float*)in, (bf16_t*)out, (size_t)n);
+  else if (in_dtype == DT_BF16 && out_dtype == DT_F32)
+    hipLaunchKernelGGL((cast_kernel<bf16_t, float>), dim3(blocks), dim3(256), 0, s, (const bf16_t*)in, (float*)out, (size_t)n);
+  else IFX_FAIL("cast: unsupported %d -> %d", in_dtype, out_dtype);
+  IFX_LAUNCH_CHECK();
+}

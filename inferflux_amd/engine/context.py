@@ -1,0 +1,126 @@
+"""What one step looks like to the parts: the flattened rows of a batch and their metadata.
+
+A step is a list of (request, its next tokens).  All rows are laid end to end; the rows of one
+request are contiguous and in position order.  For every row the context gives its token,
+its absolute position and its request's index in the batch; for every request its row range,
+its length after the step and its state slot; for every cache group the block tables and the
+slot each row's key and value are written to.  Everything is built on the host as int32 and
+uploaded in one copy.
+
+The reference passes a list of UnifiedBatchInput{sequence_id, n_past, tokens, request_logits}
+(runtime/backends/common/backend_types.h:22-34) and splits it into one batched decode forward
+plus one forward per prefill item (runtime/backends/cuda/inferflux_cuda_executor.cpp:3231-3263,
+3289-3345, 3539-3625); here the whole list is one forward.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Callable, Dict, Hashable, List, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclasses.dataclass
+class StepEntry:
+    """A request's share of a step: its next ``tokens`` and the places among them (indices into
+    ``tokens``) whose logits are wanted."""
+    rid: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class StepContext:
+    def __init__(self, entries: Sequence[StepEntry], manager, act_dtype: torch.dtype, device):
+        self.act_dtype, self.device = act_dtype, device
+        self.entries = list(entries)
+        R = self.n_requests = len(self.entries)
+        P = manager.page_size
+        q_len = np.array([len(e.tokens) for e in self.entries], dtype=np.int32)
+        start = np.array([manager.length(e.rid) for e in self.entries], dtype=np.int32)
+        q_start = np.zeros(R, dtype=np.int32)
+        if R > 1:
+            q_start[1:] = np.cumsum(q_len)[:-1]
+        T = self.n_tokens = int(q_len.sum())
+        self.h_q_len, self.h_q_start, self.h_start_pos = q_len, q_start, start
+        self.h_kv_len = start + q_len
+        self.h_token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in self.entries]) if R else np.zeros(0, np.int32)
+        self.h_row_req = np.repeat(np.arange(R, dtype=np.int32), q_len)
+        self.h_positions = (np.arange(T, dtype=np.int32) - np.repeat(q_start, q_len) + np.repeat(start, q_len)).astype(np.int32)
+        rows: List[int] = []
+        for i, e in enumerate(self.entries):
+            rows.extend(int(q_start[i]) + int(w) for w in e.want)
+        self.h_logit_rows = np.asarray(rows, dtype=np.int32)
+        self.n_logit_rows = len(rows)
+        self.h_state_slots = np.array([manager.state_slot(e.rid) for e in self.entries], dtype=np.int32)
+
+        n_groups = len(manager.groups)
+        self.h_block_tables: List[np.ndarray] = []
+        self.h_write_slots: List[np.ndarray] = []
+        for g in range(n_groups):
+            tables = [manager.block_table(e.rid, g) for e in self.entries]
+            width = max(8, -(-max((len(t) for t in tables), default=1) // 8) * 8)
+            bt = np.full((R, width), -1, dtype=np.int32)
+            for i, t in enumerate(tables):
+                bt[i, :len(t)] = t
+            self.h_block_tables.append(bt)
+            blk = self.h_positions // P
+            pages = bt[self.h_row_req, blk] if T else np.zeros(0, np.int32)
+            if T and (pages < 0).any():
+                raise RuntimeError(f"cache group {g}: a row of this step has no page (reserve before building the step)")
+            self.h_write_slots.append((pages * P + self.h_positions % P).astype(np.int32))
+
+        # One upload: every array above, end to end, each start aligned to 4 ints.
+        named = [("token_ids", self.h_token_ids), ("positions", self.h_positions), ("row_req", self.h_row_req),
+                 ("q_start", q_start), ("q_len", q_len), ("kv_len", self.h_kv_len),
+                 ("logit_rows", self.h_logit_rows), ("state_slots", self.h_state_slots)]
+        for g in range(n_groups):
+            named.append((f"block_table{g}", self.h_block_tables[g]))
+            named.append((f"write_slots{g}", self.h_write_slots[g]))
+        offs, total = {}, 0
+        for name, a in named:
+            offs[name] = (total, a.size, a.shape)
+            total += (a.size + 3) // 4 * 4
+        slab = np.zeros(max(total, 4), dtype=np.int32)
+        for name, a in named:
+            o, n, _ = offs[name]
+            slab[o:o + n] = a.reshape(-1)
+        self._slab = torch.from_numpy(slab).to(device)
+        self._views: Dict[str, torch.Tensor] = {}
+        for name, _ in named:
+            o, n, shape = offs[name]
+            self._views[name] = self._slab[o:o + n].view(shape)
+        self._derived: Dict[object, object] = {}
+
+    # ---- device views -------------------------------------------------------------
+    @property
+    def token_ids(self) -> torch.Tensor: return self._views["token_ids"]
+    @property
+    def positions(self) -> torch.Tensor: return self._views["positions"]
+    @property
+    def row_req(self) -> torch.Tensor: return self._views["row_req"]
+    @property
+    def q_start(self) -> torch.Tensor: return self._views["q_start"]
+    @property
+    def q_len(self) -> torch.Tensor: return self._views["q_len"]
+    @property
+    def kv_len(self) -> torch.Tensor: return self._views["kv_len"]
+    @property
+    def logit_rows(self) -> torch.Tensor: return self._views["logit_rows"]
+    @property
+    def state_slots(self) -> torch.Tensor: return self._views["state_slots"]
+
+    def block_table(self, group: int) -> torch.Tensor:
+        return self._views[f"block_table{group}"]
+
+    def write_slots(self, group: int) -> torch.Tensor:
+        return self._views[f"write_slots{group}"]
+
+    def derived(self, key, make: Callable[[], object]):
+        """A value computed once per step and shared by every layer that asks (kernel work lists)."""
+        if key not in self._derived:
+            self._derived[key] = make()
+        return self._derived[key]
+
+    def upload(self, array: np.ndarray) -> torch.Tensor:
+        return torch.from_numpy(np.ascontiguousarray(array)).to(self.device)

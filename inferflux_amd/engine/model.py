@@ -1,0 +1,96 @@
+"""The generic model: parts built from a plan, weights bound by name, one forward over a step.
+
+Nothing here is specific to an architecture.  The plan says which parts make each layer and
+in which order layers run; the model builds them, collects the tensors they declare, hands
+each part its tensors, and runs a step's rows through embedding, the scheduled layers, the
+final norm on the wanted rows and the head.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Mapping, Optional
+
+import torch
+
+from .. import architectures  # noqa: F401  (registers the known architectures)
+from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
+from ..config.registry import plan_for
+from ..parts.base import build_part
+from ..parts.plan import ModelPlan, ParamSpec
+from ..weights.loader import load_weights, random_tensor
+
+
+def _walk(part):
+    yield part
+    for c in part.children():
+        yield from _walk(c)
+
+
+class Model:
+    def __init__(self, config=None, plan: Optional[ModelPlan] = None):
+        if plan is None:
+            plan = plan_for(config)
+        plan.validate()
+        self.config, self.plan = config, plan
+        H = plan.hidden_size
+        self.embedding = build_part("embedding", plan.embedding, hidden_size=H)
+        self.blocks = [build_part("block", l.block, layer=l, hidden_size=H) for l in plan.layers]
+        self.final_norm = build_part("norm", plan.final_norm, hidden_size=H)
+        self.head = build_part("head", plan.lm_head, hidden_size=H)
+        self.dtype: Optional[torch.dtype] = None
+        self.device = None
+
+    # ---- structure ----------------------------------------------------------------
+    def parts(self):
+        yield from _walk(self.embedding)
+        for b in self.blocks:
+            yield from _walk(b)
+        yield from _walk(self.final_norm)
+        yield from _walk(self.head)
+
+    def schedule_mixers(self) -> List:
+        return [self.blocks[e.layer].mixer for e in self.plan.schedule]
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        out: Dict[str, ParamSpec] = {}
+        for p in self.parts():
+            for n, s in p.param_specs().items():
+                if n in out and out[n] != s:
+                    raise ValueError(f"tensor '{n}' is declared twice with different specs")
+                out[n] = s
+        return out
+
+    @staticmethod
+    def param_specs_for(config) -> Dict[str, ParamSpec]:
+        return Model(config).param_specs()
+
+    # ---- weights ------------------------------------------------------------------
+    def bind(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device) -> "Model":
+        for p in self.parts():
+            p.load(tensors)
+        self.dtype, self.device = dtype, torch.device(device)
+        return self
+
+    def load_folder(self, folder: str, dtype: torch.dtype, device) -> "Model":
+        return self.bind(load_weights(folder, self.param_specs(), dtype, device), dtype, device)
+
+    def init_random(self, seed: int, dtype: torch.dtype, device) -> "Model":
+        """Random weights made on the device, tensor by tensor (for sizes whose folder would take
+        long to write).  Values follow each spec's rule, rounded to bfloat16 in both modes so the
+        two modes see the same numbers."""
+        tensors = {}
+        for n, s in self.param_specs().items():
+            t = random_tensor(n, s, seed, torch.bfloat16, device=device)
+            tensors[n] = t if (dtype == torch.bfloat16 or s.integer) else t.float()
+        return self.bind(tensors, dtype, device)
+
+    # ---- forward ------------------------------------------------------------------
+    def forward(self, ctx, storage) -> torch.Tensor:
+        """float32 logits [len(ctx.logit_rows), vocab] for the step ``ctx`` describes."""
+        residual = self.embedding.forward(ctx.token_ids)
+        pending = None
+        for i, e in enumerate(self.plan.schedule):
+            residual, pending = self.blocks[e.layer].forward(residual, pending, ctx, storage.binding(i))
+        if ctx.n_logit_rows == 0:
+            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=residual.device)
+        h = self.final_norm.forward(residual, pending, ctx.act_dtype, rows=ctx.logit_rows)
+        return self.head.forward(h)

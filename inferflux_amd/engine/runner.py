@@ -1,0 +1,99 @@
+"""The step function: run a batch of (request, next tokens) from the cache and return logits.
+
+``ModelRunner.step`` takes any mix of prompt portions and single decoded tokens, cut anywhere.
+It checks the whole step first (known requests, token ids, positions, pages), reserves pages
+for every row or raises before anything has changed, runs all rows as one batch, commits the
+new positions and returns float32 logits at the wanted places, in the order of the entries
+and of their ``want`` lists.  It samples nothing.
+
+The reference's step (InferfluxCudaExecutor::ExecuteUnifiedBatch,
+runtime/backends/cuda/inferflux_cuda_executor.cpp:3165-3769) samples inside the step and
+reports failures per item (3234-3253, 3545-3560); here a step succeeds for every entry or
+raises before it touches the cache.
+"""
+from __future__ import annotations
+
+from typing import Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import OutOfPages
+from ..cache.storage import CacheStorage
+from .context import StepContext, StepEntry
+from .model import Model
+
+
+class StepError(ValueError):
+    """A step that cannot run; the cache is unchanged."""
+
+
+class ModelRunner:
+    def __init__(self, model: Model, num_pages: int, page_size: int = 16, max_requests: int = 64):
+        if model.device is None:
+            raise ValueError("the model has no weights yet (load_folder / init_random first)")
+        if model.device.type != "cuda":
+            raise RuntimeError(f"the engine runs on the GPU only, the model is on {model.device}")
+        self.model = model
+        self.device, self.dtype = model.device, model.dtype
+        self.storage = CacheStorage(model.plan.schedule, model.schedule_mixers(), page_size, num_pages,
+                                    max_requests, model.dtype, model.device)
+        self.manager = self.storage.manager
+        self.page_size = page_size
+        self.vocab_size = model.plan.vocab_size
+        self.max_position = model.plan.max_position
+
+    # ---- requests -----------------------------------------------------------------
+    def add_request(self, rid: Hashable) -> None:
+        slot = self.manager.add(rid)
+        self.storage.reset_state(slot)
+
+    def free_request(self, rid: Hashable) -> None:
+        self.manager.free(rid)
+
+    def has_request(self, rid: Hashable) -> bool:
+        return self.manager.has(rid)
+
+    def length(self, rid: Hashable) -> int:
+        return self.manager.length(rid)
+
+    # ---- the step -----------------------------------------------------------------
+    def validate(self, entries: Sequence[StepEntry]) -> None:
+        seen = set()
+        for e in entries:
+            if e.rid in seen:
+                raise StepError(f"request {e.rid!r} appears twice in one step")
+            seen.add(e.rid)
+            if not self.manager.has(e.rid):
+                raise StepError(f"request {e.rid!r} is not live (add_request first)")
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.rid!r} brings no tokens")
+            bad = [t for t in e.tokens if not (0 <= int(t) < self.vocab_size)]
+            if bad:
+                raise StepError(f"request {e.rid!r}: token ids {bad[:8]} outside [0, {self.vocab_size})")
+            if self.manager.length(e.rid) + n > self.max_position:
+                raise StepError(f"request {e.rid!r}: {self.manager.length(e.rid)} + {n} tokens exceed max_position {self.max_position}")
+            badw = [w for w in e.want if not (0 <= int(w) < n)]
+            if badw:
+                raise StepError(f"request {e.rid!r}: wanted places {badw[:8]} outside its {n} tokens")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        entries = list(entries)
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        self.validate(entries)
+        needs = [(e.rid, len(e.tokens)) for e in entries]
+        if not self.manager.can_reserve(needs):
+            tot = [0] * len(self.manager.groups)
+            for rid, n in needs:
+                for g, k in enumerate(self.manager.pages_needed(rid, n)):
+                    tot[g] += k
+            g = next(g for g, t in enumerate(tot) if t > self.manager.pools[g].num_free)
+            raise OutOfPages(g, tot[g], self.manager.pools[g].num_free)
+        for rid, n in needs:
+            self.manager.reserve(rid, n)
+        ctx = StepContext(entries, self.manager, self.dtype, self.device)
+        logits = self.model.forward(ctx, self.storage)
+        for rid, n in needs:
+            self.manager.commit(rid, n)
+        return logits

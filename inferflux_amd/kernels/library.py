@@ -1,0 +1,188 @@
+"""Builds and loads the HIP kernel modules.
+
+Each ``csrc/<name>.hip`` is compiled by hipcc for gfx950 into one shared library
+``<name>[-variant].<hash>.so`` and loaded through ctypes.  The hash covers the source, the
+shared header, the flags and the variant's defines, so a library on disk always matches the
+source beside it: a stale one is simply not found and the module is compiled again.  A module
+is compiled when it is first used, which means a run compiles what its model needs and no
+more.  Libraries are written next to the sources when that folder is writable (so they travel
+with the tree) and to a per-user folder under the temporary directory otherwise.
+
+There is no fallback: if hipcc is missing or a module does not compile, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import fcntl
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import Dict, Iterable, Optional, Sequence, Tuple
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "csrc")
+CSRC = os.path.normpath(CSRC)
+ARCH = "gfx950"
+# -packed-fp32-ops is switched off for device code: some packed float forms have given wrong
+# results on this hardware.  The host pass of hipcc does not know the feature and says so.
+FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
+
+Variant = Tuple[Tuple[str, int], ...]
+
+
+class KernelBuildError(RuntimeError):
+    pass
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise KernelBuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): the HIP kernels cannot be built")
+
+
+def _variant_tag(variant: Variant) -> str:
+    return "".join(f"-{k.lower()}{v}" for k, v in variant)
+
+
+def _digest(name: str, variant: Variant) -> str:
+    h = hashlib.sha256()
+    for fn in (f"{name}.hip", "common.h"):
+        with open(os.path.join(CSRC, fn), "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(FLAGS).encode())
+    h.update(repr(variant).encode())
+    return h.hexdigest()[:12]
+
+
+def _fallback_dir() -> str:
+    d = os.path.join(tempfile.gettempdir(), f"inferflux_amd-{os.getuid()}")
+    os.makedirs(d, mode=0o700, exist_ok=True)
+    return d
+
+
+def _lib_filename(name: str, variant: Variant) -> str:
+    return f"{name}{_variant_tag(variant)}.{_digest(name, variant)}.so"
+
+
+def find_library(name: str, variant: Variant = ()) -> Optional[str]:
+    fn = _lib_filename(name, variant)
+    for d in (CSRC, _fallback_dir()):
+        p = os.path.join(d, fn)
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def _progress(msg: str) -> None:
+    print(f"[inferflux_amd] {msg}", file=sys.stderr, flush=True)
+
+
+def compile_module(name: str, variant: Variant = (), force: bool = False) -> str:
+    """Compile one module (unless an up-to-date library exists) and return the library's path."""
+    if not force:
+        hit = find_library(name, variant)
+        if hit:
+            return hit
+    src = os.path.join(CSRC, f"{name}.hip")
+    if not os.path.isfile(src):
+        raise KernelBuildError(f"no kernel source {src}")
+    out_dir = CSRC if os.access(CSRC, os.W_OK) else _fallback_dir()
+    fn = _lib_filename(name, variant)
+    out = os.path.join(out_dir, fn)
+    lock_path = os.path.join(out_dir, f".{name}{_variant_tag(variant)}.lock")
+    with open(lock_path, "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        try:
+            if not force and os.path.isfile(out):
+                return out
+            tmp = f"{out}.{os.getpid()}.tmp"
+            cmd = [_hipcc(), *FLAGS, *[f"-D{k}={v}" for k, v in variant], src, "-o", tmp]
+            label = f"{name}{_variant_tag(variant)}"
+            _progress(f"compiling {label} for {ARCH} ...")
+            t0 = time.time()
+            proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=out_dir)
+            done = threading.Event()
+
+            def tick():
+                while not done.wait(20.0):
+                    _progress(f"still compiling {label} ({time.time() - t0:.0f} s)")
+
+            th = threading.Thread(target=tick, daemon=True)
+            th.start()
+            log, _ = proc.communicate()
+            done.set()
+            if proc.returncode != 0 or not os.path.isfile(tmp):
+                if os.path.exists(tmp):
+                    os.unlink(tmp)
+                raise KernelBuildError(f"hipcc failed for {label} (exit {proc.returncode}):\n{' '.join(cmd)}\n{log}")
+            os.replace(tmp, out)
+            # Drop libraries of the same module built from older sources.
+            prefix = f"{name}{_variant_tag(variant)}."
+            for old in os.listdir(out_dir):
+                if old.startswith(prefix) and old.endswith(".so") and old != fn:
+                    try:
+                        os.unlink(os.path.join(out_dir, old))
+                    except OSError:
+                        pass
+            _progress(f"compiled {label} in {time.time() - t0:.1f} s")
+            return out
+        finally:
+            fcntl.flock(lock, fcntl.LOCK_UN)
+
+
+class KernelModule:
+    """A loaded library; functions are looked up by name, with their argument types set once."""
+
+    def __init__(self, name: str, variant: Variant, path: str):
+        self.name, self.variant, self.path = name, variant, path
+        self.lib = ctypes.CDLL(path)
+        self.lib.ifx_last_error.restype = ctypes.c_char_p
+        self._fns: Dict[str, ctypes._CFuncPtr] = {}
+
+    def fn(self, fname: str, argtypes: Sequence) -> "ctypes._CFuncPtr":
+        f = self._fns.get(fname)
+        if f is None:
+            f = getattr(self.lib, fname)
+            f.argtypes = list(argtypes)
+            f.restype = ctypes.c_int
+            self._fns[fname] = f
+        return f
+
+    def last_error(self) -> str:
+        return (self.lib.ifx_last_error() or b"").decode(errors="replace")
+
+
+_MODULES: Dict[Tuple[str, Variant], KernelModule] = {}
+_LOCK = threading.Lock()
+
+
+def load_module(name: str, variant: Variant = ()) -> KernelModule:
+    key = (name, variant)
+    m = _MODULES.get(key)
+    if m is not None:
+        return m
+    with _LOCK:
+        m = _MODULES.get(key)
+        if m is None:
+            m = KernelModule(name, variant, compile_module(name, variant))
+            _MODULES[key] = m
+    return m
+
+
+def all_module_variants() -> Iterable[Tuple[str, Variant]]:
+    """Every module and variant the package can ask for: what ``build_all`` compiles."""
+    from . import ops
+    return ops.module_variants()
+
+
+def build_all(force: bool = True, jobs: int = 8) -> None:
+    todo = list(all_module_variants())
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as ex:
+        list(ex.map(lambda nv: compile_module(nv[0], nv[1], force=force), todo))

@@ -1,0 +1,273 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that the operands are on the GPU, contiguous, of the
+expected type and of shapes that fit what the kernel and its grid assume, and only then
+launches on torch's current stream.  Nothing here falls back to another implementation: a
+missing library or a refused size raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Iterable, Optional, Tuple
+
+import torch
+
+from .library import KernelModule, Variant, load_module
+
+P = ctypes.c_void_p
+I = ctypes.c_int
+F = ctypes.c_float
+LL = ctypes.c_longlong
+
+DT_F32, DT_BF16 = 0, 1
+_DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
+
+ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def module_variants() -> Iterable[Tuple[str, Variant]]:
+    yield ("core", ())
+    yield ("gemm_f32", ())
+    yield ("attn_plain", ())
+    yield ("sampling", ())
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported element type {t.dtype} (float32 or bfloat16)") from None
+
+
+def _check(t: torch.Tensor, name: str, shape=None, dtype=None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: not a tensor")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}; the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: element type {t.dtype}, expected {dtype}")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != ts for s, ts in zip(shape, t.shape)):
+            raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _call(mod: KernelModule, fname: str, argtypes, *args) -> None:
+    rc = mod.fn(fname, argtypes)(*args)
+    if rc != 0:
+        raise KernelError(f"{fname}: {mod.last_error()} (code {rc})")
+
+
+# ----------------------------------------------------------------------------------------
+def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """float32 [T, H] rows of ``table`` [V, H] named by int32 ``ids`` [T] (ids are checked by the caller)."""
+    _check(ids, "ids", (None,), torch.int32)
+    _check(table, "table", (None, None))
+    T, H = ids.shape[0], table.shape[1]
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _call(load_module("core"), "ifx_embedding", (P, P, I, P, I, I, P),
+          ids.data_ptr(), table.data_ptr(), _dt(table), out.data_ptr(), T, H, _stream())
+    return out
+
+
+def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``residual`` [T, H] float32 (+= ``delta`` in place when given and no ``rows``), then RMSNorm.
+
+    With ``rows`` (int32 [R]) only those rows are normalised, into [R, H], and the residual is
+    left untouched.
+    """
+    _check(residual, "residual", (None, None), torch.float32)
+    T, H = residual.shape
+    _check(weight, "weight", (H,))
+    if delta is not None:
+        _check(delta, "delta", (T, H))
+    n = T
+    if rows is not None:
+        _check(rows, "rows", (None,), torch.int32)
+        n = rows.shape[0]
+    out = torch.empty((n, H), dtype=out_dtype, device=residual.device)
+    _call(load_module("core"), "ifx_add_rmsnorm", (P, P, I, P, I, P, I, P, I, I, F, I, P),
+          residual.data_ptr(), _ptr(delta), _dt(delta) if delta is not None else 0, weight.data_ptr(),
+          _dt(weight), out.data_ptr(), _DT[out_dtype], _ptr(rows), n, H, float(eps),
+          1 if (delta is not None and rows is None) else 0, _stream())
+    return out
+
+
+def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                slots: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], rope_style: int,
+                rotary_dim: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
+    """Bias, rotation and cache write of one step's projections; returns q [T, n_heads, head_dim].
+
+    ``qkv`` is [T, (n_heads + 2 n_kv_heads) head_dim] when the keys and values are written
+    (``slots`` int32 [T] = page * page_size + offset), or [T, n_heads head_dim] with
+    ``n_kv_heads`` = 0 for a mixer that only reads another's cache.
+    """
+    T = qkv.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    _check(qkv, "qkv", (T, width))
+    _check(positions, "positions", (T,), torch.int32)
+    if bias is not None:
+        _check(bias, "bias", (width,))
+    if inv_freq is not None:
+        _check(inv_freq, "inv_freq", (None,), torch.float32)
+        if rope_style != ROPE_NONE and inv_freq.shape[0] < rotary_dim // 2:
+            raise KernelError("inv_freq shorter than rotary_dim / 2")
+    if slots is not None:
+        _check(slots, "slots", (T,), torch.int32)
+        _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), qkv.dtype)
+        _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, head_dim, page_size), qkv.dtype)
+    elif n_kv_heads != 0:
+        raise KernelError("rope_append: keys and values given but no slots to write them to")
+    q = torch.empty((T, n_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, P),
+          qkv.data_ptr(), _dt(qkv), _ptr(bias), _dt(bias) if bias is not None else 0, positions.data_ptr(),
+          _ptr(slots), _ptr(inv_freq), rope_style, rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size,
+          q.data_ptr(), _ptr(k_cache), _ptr(v_cache), _stream())
+    return q
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """[T, 2I] = [gate | up]  ->  silu(gate) * up  [T, I]."""
+    _check(gate_up, "gate_up", (None, None))
+    T, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError("swiglu: odd width")
+    out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, P),
+          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, _stream())
+    return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    if x.dtype == dtype:
+        return x
+    _check(x, "x")
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _call(load_module("core"), "ifx_cast", (P, I, P, I, LL, P),
+          x.data_ptr(), _dt(x), out.data_ptr(), _DT[dtype], x.numel(), _stream())
+    return out
+
+
+# ----------------------------------------------------------------------------------------
+def gemm_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x [M, K] (float32 or bfloat16) times float32 ``weight`` [N, K] transposed, true 32-bit math."""
+    _check(x, "x", (None, None))
+    M, K = x.shape
+    _check(weight, "weight", (None, K), torch.float32)
+    N = weight.shape[0]
+    if bias is not None:
+        _check(bias, "bias", (N,), torch.float32)
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _call(load_module("gemm_f32"), "ifx_gemm_f32", (P, I, P, P, P, I, I, I, I, P),
+          x.data_ptr(), _dt(x), weight.data_ptr(), _ptr(bias), out.data_ptr(), _DT[out_dtype], M, N, K, _stream())
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x [M, K] times ``weight`` [N, K] transposed, chosen by the weight's type.
+
+    A float32 weight takes the true 32-bit kernel whatever the activation's type.  A bfloat16
+    weight with bfloat16 activations takes the library product with float accumulation, as
+    the reference does for every dense projection
+    (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).
+    """
+    if weight.dtype == torch.float32:
+        return gemm_f32(x, weight, None, out_dtype or x.dtype)
+    if weight.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+        raise KernelError(f"linear: weight {weight.dtype} with activation {x.dtype} is not supported")
+    _check(x, "x", (None, weight.shape[1]))
+    _check(weight, "weight", (None, None))
+    out = torch.matmul(x, weight.t())
+    if out_dtype is not None and out_dtype != out.dtype:
+        out = cast(out, out_dtype)
+    return out
+
+
+# ----------------------------------------------------------------------------------------
+def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_req: torch.Tensor,
+                    positions: torch.Tensor, block_table: torch.Tensor, window: Optional[int],
+                    scale: float) -> torch.Tensor:
+    """Causal (optionally windowed) attention of q [T, nH, d] over the paged cache; returns [T, nH*d]."""
+    _check(q, "q", (None, None, None))
+    T, nH, d = q.shape
+    _check(k_cache, "k_cache", (None, None, None, d), q.dtype)
+    n_pages, nKV, page_size, _ = k_cache.shape
+    _check(v_cache, "v_cache", (n_pages, nKV, d, page_size), q.dtype)
+    _check(row_req, "row_req", (T,), torch.int32)
+    _check(positions, "positions", (T,), torch.int32)
+    _check(block_table, "block_table", (None, None), torch.int32)
+    out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
+    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P),
+          q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q), row_req.data_ptr(),
+          positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, page_size,
+          int(window or 0), float(scale), _stream())
+    return out
+
+
+# ----------------------------------------------------------------------------------------
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Lowest index of the maximum of each row of float32 ``logits`` [R, V]; int32 [R]."""
+    _check(logits, "logits", (None, None), torch.float32)
+    R, V = logits.shape
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _call(load_module("sampling"), "ifx_argmax", (P, I, I, P, P), logits.data_ptr(), R, V, out.data_ptr(), _stream())
+    return out
+
+
+def apply_penalties(logits: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, counts: torch.Tensor,
+                    rep: torch.Tensor, freq: torch.Tensor, pres: torch.Tensor) -> None:
+    _check(logits, "logits", (None, None), torch.float32)
+    R, V = logits.shape
+    n = rows.shape[0]
+    for t, nm in ((rows, "rows"), (ids, "ids"), (counts, "counts")):
+        _check(t, nm, (n,), torch.int32)
+    for t, nm in ((rep, "rep"), (freq, "freq"), (pres, "pres")):
+        _check(t, nm, (R,), torch.float32)
+    _call(load_module("sampling"), "ifx_apply_penalties", (P, I, P, P, P, I, P, P, P, P),
+          logits.data_ptr(), V, rows.data_ptr(), ids.data_ptr(), counts.data_ptr(), n, rep.data_ptr(),
+          freq.data_ptr(), pres.data_ptr(), _stream())
+
+
+def add_logit_bias(logits: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, bias: torch.Tensor) -> None:
+    _check(logits, "logits", (None, None), torch.float32)
+    n = rows.shape[0]
+    _check(rows, "rows", (n,), torch.int32)
+    _check(ids, "ids", (n,), torch.int32)
+    _check(bias, "bias", (n,), torch.float32)
+    _call(load_module("sampling"), "ifx_add_logit_bias", (P, I, P, P, P, I, P),
+          logits.data_ptr(), logits.shape[1], rows.data_ptr(), ids.data_ptr(), bias.data_ptr(), n, _stream())
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    """One token per row of float32 ``logits`` [R, V]; rows with temperature <= 0 take the argmax."""
+    _check(logits, "logits", (None, None), torch.float32)
+    R, V = logits.shape
+    _check(temperature, "temperature", (R,), torch.float32)
+    _check(top_k, "top_k", (R,), torch.int32)
+    _check(top_p, "top_p", (R,), torch.float32)
+    _check(min_p, "min_p", (R,), torch.float32)
+    _check(uniform, "uniform", (R,), torch.float32)
+    weights = torch.empty_like(logits)
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _call(load_module("sampling"), "ifx_sample", (P, P, P, P, P, P, P, P, I, I, P),
+          logits.data_ptr(), weights.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
+          min_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), R, V, _stream())
+    return out

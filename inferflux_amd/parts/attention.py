@@ -1,0 +1,97 @@
+"""Grouped-query attention over the paged cache, with q/k/v bias, a position part and an
+optional window.
+
+Reference order (runtime/backends/cuda/native/transformer_forward.cu:1944-2135, 2145-2241):
+q, k, v = h Wq^T + bq, h Wk^T + bk, h Wv^T + bv; position encoding of q and k; k and v are
+written to the cache at the token's position; causal attention of head h over kv head
+h / (nH / nKV) with scale 1/sqrt(d) applied after the dot product; delta = attn Wo^T.
+The three projections are concatenated at load time into one [(nH + 2 nKV) d, H] product;
+the bias is added in float inside the rotary kernel (the reference rounds the product to the
+activation type first and adds the bias afterwards, cuda_kernels.cu:518-527).
+
+An execution that reads another entry's cache (binding.writes_cache False) projects and
+encodes only its queries.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from ..kernels.attention import paged_attention
+from .base import Mixer, MixerBinding, build_part, register_part
+from .ffn import concat_weights
+from .plan import CacheSpec, ParamSpec, PartSpec
+
+
+@register_part("mixer", "paged_attention")
+class PagedAttention(Mixer):
+    def __init__(self, name: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                 position: PartSpec, bias: bool = True, window: Optional[int] = None,
+                 scale: Optional[float] = None, init_std: float = 0.02):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{name}: {n_heads} query heads are not a multiple of {n_kv_heads} kv heads")
+        self.name, self.hidden_size = name, int(hidden_size)
+        self.n_heads, self.n_kv_heads, self.head_dim = int(n_heads), int(n_kv_heads), int(head_dim)
+        self.bias, self.window, self.init_std = bool(bias), (int(window) if window else None), init_std
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.position = build_part("position", position)
+        self.w_qkv = self.b_qkv = self.w_o = None
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.n_kv_heads, self.head_dim, self.window)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        H, d, s = self.hidden_size, self.head_dim, ("normal", self.init_std)
+        out = {
+            f"{self.name}.q_proj.weight": ParamSpec((self.n_heads * d, H), s),
+            f"{self.name}.k_proj.weight": ParamSpec((self.n_kv_heads * d, H), s),
+            f"{self.name}.v_proj.weight": ParamSpec((self.n_kv_heads * d, H), s),
+            f"{self.name}.o_proj.weight": ParamSpec((H, self.n_heads * d), s),
+        }
+        if self.bias:
+            out[f"{self.name}.q_proj.bias"] = ParamSpec((self.n_heads * d,), s)
+            out[f"{self.name}.k_proj.bias"] = ParamSpec((self.n_kv_heads * d,), s)
+            out[f"{self.name}.v_proj.bias"] = ParamSpec((self.n_kv_heads * d,), s)
+        return out
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        n = self.name
+        self.w_qkv = concat_weights([tensors[f"{n}.{p}_proj.weight"] for p in "qkv"])
+        self.b_qkv = concat_weights([tensors[f"{n}.{p}_proj.bias"] for p in "qkv"]) if self.bias else None
+        self.w_o = tensors[f"{n}.o_proj.weight"]
+
+    def forward(self, h: torch.Tensor, ctx, binding: MixerBinding) -> torch.Tensor:
+        cache = binding.cache
+        nH, d = self.n_heads, self.head_dim
+        nKV = self.n_kv_heads if binding.writes_cache else 0
+        width = (nH + 2 * nKV) * d
+        style, rotary_dim, inv_freq = self.position.kernel_args(h.device)
+        w, b = self.w_qkv, self.b_qkv
+        if not binding.writes_cache:  # only the queries: the first nH*d rows of the fused matrix
+            w, b = w[:width], (b[:width] if b is not None else None)
+        qkv = ops.linear(h, w)
+        if self.position.needs_apply:
+            qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
+        slots = ctx.write_slots(cache.group) if binding.writes_cache else None
+        q = ops.rope_append(qkv, b, ctx.positions, slots, inv_freq, style, rotary_dim, nH, nKV, d,
+                            cache.k if slots is not None else None, cache.v if slots is not None else None,
+                            cache.page_size)
+        out = paged_attention(q, cache, ctx, self.window, self.scale)
+        return ops.linear(out, self.w_o)
+
+    def _encode_outside(self, qkv, bias, ctx, nKV):
+        """For a position part that transforms q and k itself: add the bias, let the part encode,
+        and hand the kernel rows it only has to copy."""
+        nH, d, T = self.n_heads, self.head_dim, qkv.shape[0]
+        if bias is not None:
+            qkv = (qkv.float() + bias.float()).to(qkv.dtype)
+        q = qkv[:, : nH * d].reshape(T, nH, d)
+        k = qkv[:, nH * d: (nH + nKV) * d].reshape(T, nKV, d) if nKV else None
+        q, k = self.position.apply(q, k, ctx.positions)
+        cols = [q.reshape(T, nH * d)]
+        if nKV:
+            cols += [k.reshape(T, nKV * d), qkv[:, (nH + nKV) * d:]]
+        return torch.cat(cols, dim=1).contiguous()

@@ -1,0 +1,126 @@
+"""Interfaces of the parts a layer is made of, and the registry that finds them by name.
+
+A part is built from its sizes and constants alone; it never sees the model's config and does
+not know which model it is in.  It declares the tensors it expects under its weight prefix
+(``param_specs``), receives them once (``load``), and then runs on a step's rows.
+
+Categories and what each must provide beyond ``param_specs`` / ``load``:
+
+  norm      forward(residual, delta, rows=None) -> normalised rows in the activation type.
+            ``residual`` is the float32 stream [T, H]; ``delta`` (or None) is first added to it
+            in place.  With ``rows`` only those rows are returned and nothing is written.
+  position  prepares what the mixer's kernels need to encode positions (see parts/position.py);
+            a position part may also transform q and k itself through ``apply(q, k, positions)``.
+  mixer     forward(h, ctx, binding) -> delta [T, H].  ``cache_spec()`` says what it keeps per
+            token (or None), ``state_spec()`` what fixed-size state it keeps per request (or
+            None).  ``binding`` carries the cache tensors / state tensor the model allocated for
+            this execution of the layer.
+  ffn       forward(h, ctx) -> delta [T, H].
+  block     the arrangement: forward(residual, pending, ctx, binding) -> (residual, pending),
+            where ``pending`` is a delta not yet added to the stream (the next norm adds it).
+  embedding forward(token_ids) -> float32 stream [T, H].
+  head      forward(normalised rows) -> float32 logits [R, V].
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Callable, Dict, Mapping, Optional
+
+import torch
+
+from .plan import CacheSpec, ParamSpec, PartSpec, StateSpec
+
+_REGISTRY: Dict[str, Dict[str, Callable]] = {}
+CATEGORIES = ("norm", "position", "mixer", "ffn", "block", "embedding", "head")
+
+
+def register_part(category: str, name: str):
+    """Class decorator: make ``cls`` buildable from ``PartSpec(kind=name)`` in ``category``."""
+    if category not in CATEGORIES:
+        raise ValueError(f"unknown part category '{category}' (one of {CATEGORIES})")
+
+    def deco(cls):
+        table = _REGISTRY.setdefault(category, {})
+        if name in table and table[name] is not cls:
+            raise ValueError(f"{category} part '{name}' is already registered")
+        table[name] = cls
+        return cls
+
+    return deco
+
+
+def build_part(category: str, spec: PartSpec, **context) -> "Part":
+    """Build the part ``spec`` names.  ``context`` holds what the surrounding structure knows
+    (``prefix`` of the weight names, ``hidden_size``); the part's own sizes are in ``spec.args``."""
+    table = _REGISTRY.get(category, {})
+    if spec.kind not in table:
+        raise KeyError(f"no {category} part named '{spec.kind}'; registered: {sorted(table)}")
+    return table[spec.kind](**context, **spec.args)
+
+
+def registered_parts(category: str):
+    return sorted(_REGISTRY.get(category, {}))
+
+
+class Part:
+    """Base of all parts."""
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        """Full tensor names this part reads from the model file."""
+        return {}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Take the part's tensors (already on the device, stored by the loader's rule)."""
+
+    def children(self):
+        return ()
+
+
+@dataclasses.dataclass
+class LayerCache:
+    """The cache tensors of one schedule entry: K [pages, kv heads, page_size, d] and
+    V [pages, kv heads, d, page_size], and the cache group whose block tables index them."""
+    k: torch.Tensor
+    v: torch.Tensor
+    group: int
+    page_size: int
+
+
+@dataclasses.dataclass
+class MixerBinding:
+    """What one execution of a layer's mixer works on.
+
+    ``cache`` is None for a mixer without cache.  ``writes_cache`` is False when the entry
+    reads the cache another entry owns.  ``state`` is the [slots, *shape] tensor of the
+    mixer's per-request state, or None.
+    """
+    cache: Optional[LayerCache] = None
+    writes_cache: bool = True
+    state: Optional[torch.Tensor] = None
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, h: torch.Tensor, ctx, binding: MixerBinding) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    def forward(self, residual, pending, ctx, binding: MixerBinding):
+        raise NotImplementedError

@@ -1,0 +1,54 @@
+"""Token embedding and the output head.
+
+Embedding: x[t] = E[id[t]], no scaling, widened to the float32 stream
+(runtime/backends/cuda/native/cuda_kernels.cu:674-689).  Head: logits = h Wlm^T in float; the
+reference rounds logits to the activation type before widening them
+(transformer_forward.cu:2686-2699), which is not copied: logits are produced in float32.
+A tied head uses the embedding table (the reference ties when lm_head.weight is absent,
+weight_map.cpp:33-37; here the configuration says so and the file is checked against it).
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Part, register_part
+from .plan import ParamSpec
+
+
+@register_part("embedding", "token_embedding")
+class TokenEmbedding(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02):
+        self.name, self.vocab_size, self.hidden_size, self.init_std = name, int(vocab_size), int(hidden_size), init_std
+        self.table: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {f"{self.name}.weight": ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.table = tensors[f"{self.name}.weight"]
+
+    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        return ops.embedding(token_ids, self.table)
+
+
+@register_part("head", "linear_head")
+class LinearHead(Part):
+    """``tied_to`` names the tensor (the embedding table) a tied head shares; None for its own."""
+
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, init_std: float = 0.02):
+        self.name, self.vocab_size, self.hidden_size, self.tied_to, self.init_std = name, int(vocab_size), int(hidden_size), tied_to, init_std
+        self.weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        if self.tied_to:
+            return {}
+        return {f"{self.name}.weight": ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.tied_to or f"{self.name}.weight"]
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return ops.linear(h, self.weight, out_dtype=torch.float32)

@@ -1,0 +1,49 @@
+"""SwiGLU feed-forward: down( silu(gate(x)) * up(x) ), no biases.
+
+g = h Wg^T, u = h Wu^T, a = g / (1 + exp(-g)) * u in float, delta = a Wd^T
+(runtime/backends/cuda/native/transformer_forward.cu:2383-2419, 2487-2494, 2528-2547;
+cuda_kernels.cu:139-151).  The reference runs gate and up as two products; here the two
+matrices are concatenated at load time into one [2I, H] product, which changes nothing in
+the arithmetic of any output element.
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, register_part
+from .plan import ParamSpec
+
+
+def concat_weights(parts):
+    """Stack matrices along the output axis; mixed storage types are widened to float32."""
+    if len({p.dtype for p in parts}) > 1:
+        parts = [p.float() for p in parts]
+    return torch.cat(list(parts), dim=0).contiguous()
+
+
+@register_part("ffn", "swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, name: str, hidden_size: int, intermediate_size: int, init_std: float = 0.02):
+        self.name, self.hidden_size, self.intermediate_size = name, int(hidden_size), int(intermediate_size)
+        self.init_std = init_std
+        self.w_gate_up = None
+        self.w_down = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        H, I, s = self.hidden_size, self.intermediate_size, ("normal", self.init_std)
+        return {
+            f"{self.name}.gate_proj.weight": ParamSpec((I, H), s),
+            f"{self.name}.up_proj.weight": ParamSpec((I, H), s),
+            f"{self.name}.down_proj.weight": ParamSpec((H, I), s),
+        }
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_gate_up = concat_weights([tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]])
+        self.w_down = tensors[f"{self.name}.down_proj.weight"]
+
+    def forward(self, h, ctx):
+        gu = ops.linear(h, self.w_gate_up)
+        return ops.linear(ops.swiglu(gu), self.w_down)
