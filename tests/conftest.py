@@ -57,3 +57,85 @@ def model_folders(tmp_path_factory):
 
 def has_gpu():
     return torch.cuda.is_available()
+
+
+def sharpen(src_folder, dst_folder, seed, qk_gain=10.0):
+    """Rewrite a random model so that faults show: attention that is peaked (larger q/k matrices), a
+    feed-forward that matters (larger gate/up), norm weights and biases that are not 1 and 0-like.
+    Values stay bfloat16-representable."""
+    import shutil
+    from safetensors.torch import load_file
+    from inferflux_amd.weights import write_safetensors
+    os.makedirs(dst_folder, exist_ok=True)
+    shutil.copy(os.path.join(src_folder, "config.json"), os.path.join(dst_folder, "config.json"))
+    t = load_file(os.path.join(src_folder, "model.safetensors"))
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, w in t.items():
+        w = w.float()
+        if name.endswith(("q_proj.weight", "k_proj.weight")):
+            w = w * qk_gain
+        elif name.endswith(("gate_proj.weight", "up_proj.weight")):
+            w = w * 4.0
+        elif name.endswith(("layernorm.weight", "norm.weight")):
+            w = w + 0.2 * torch.randn(w.shape, generator=g)
+        elif name.endswith(".bias"):
+            w = w * 10.0
+        out[name] = w.to(torch.bfloat16)
+    write_safetensors(os.path.join(dst_folder, "model.safetensors"), out)
+
+
+# How much larger than N(0, 0.02) the q/k matrices of the test models are.  10 makes attention so
+# peaked that a float32 run shows any misplaced key; for bfloat16 runs 5 is used, because at 10 the
+# rounding of scores to 8 mantissa bits alone moves logits by several percent (a plain model
+# evaluated in bfloat16 is then off by 5-40 %, at 5 by 1-10 %; the engine stays below 2 %).
+QK_GAIN = {"float32": 10.0, "bfloat16": 5.0}
+
+
+class _Folders(dict):
+    """name -> folder of the float32 test model; [(name, dtype)] picks the model for that dtype."""
+    def __missing__(self, key):
+        raise KeyError(key)
+
+
+@pytest.fixture(scope="session")
+def sharp_folders(model_folders, tmp_path_factory):
+    out = _Folders()
+    for i, (name, src) in enumerate(model_folders.items()):
+        for dtype, gain in QK_GAIN.items():
+            d = str(tmp_path_factory.mktemp(f"sharp{name}{dtype}"))
+            sharpen(src, d, 200 + i, gain)
+            out[name, dtype] = d
+        out[name] = out[name, "float32"]
+    return out
+
+
+_PLAIN_CACHE = {}
+
+
+def plain_logits(folder, ids):
+    """Whole-sequence logits [S, V] of the plain implementation in float64 (cached per call)."""
+    import plain_model as pm
+    key = (folder, tuple(ids))
+    if key not in _PLAIN_CACHE:
+        if folder not in _PLAIN_CACHE:
+            _PLAIN_CACHE[folder] = pm.load_folder(folder, torch.float64)
+        cfg, W = _PLAIN_CACHE[folder]
+        _PLAIN_CACHE[key] = pm.forward(cfg, W, list(ids))
+    return _PLAIN_CACHE[key]
+
+
+def seeded_ids(seed, n, vocab):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+# Logits are compared relative to the largest logit of the row set: a float32 engine differs from
+# the float64 plain model by rounding that accumulates over a few hundred operations; a bfloat16
+# engine rounds every activation to 8 bits of mantissa.
+REL_TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+def rel_err(got, want):
+    want = want.double()
+    return float((got.double() - want).abs().max() / want.abs().max())

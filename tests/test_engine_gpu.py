@@ -1,0 +1,205 @@
+"""The engine in one process: the step function against the plain model, each part alone, long
+decoding, the first tokens, and a toy mixer with state of its own built from outside the package."""
+import math
+
+import pytest
+import torch
+
+import plain_model as pm
+from conftest import REL_TOL, TINY, plain_logits, rel_err, seeded_ids
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    from inferflux_amd.cache import OutOfPages
+    from inferflux_amd.engine.api import load_runner
+    from inferflux_amd.engine.context import StepEntry
+    from inferflux_amd.engine.runner import StepError
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def run_whole(runner, rid, ids):
+    runner.add_request(rid)
+    out = runner.step([StepEntry(rid, ids, list(range(len(ids))))]).cpu()
+    runner.free_request(rid)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_whole_prompt(name, dtype, sharp_folders):
+    folder = sharp_folders[name, dtype]
+    runner = load_runner(folder, DT[dtype], num_pages=32)
+    for n in (1, 2, 29, 200):
+        ids = seeded_ids(n, n, TINY[name]["vocab_size"])
+        got = run_whole(runner, "a", ids)
+        assert rel_err(got, plain_logits(folder, ids)) < REL_TOL[dtype], (name, n)
+    runner.manager.check()
+    assert runner.manager.free_pages() == [32] * len(runner.manager.groups)
+
+
+@pytest.mark.parametrize("name", list(TINY))
+def test_first_tokens_and_single_token_prompt(name, sharp_folders):
+    """Position 0 has one key (itself); its logits depend on the token alone."""
+    folder = sharp_folders[name]
+    runner = load_runner(folder, torch.float32, num_pages=8)
+    for tok in (0, 7, TINY[name]["vocab_size"] - 1):
+        a = run_whole(runner, "x", [tok])
+        b = run_whole(runner, "y", [tok, 3, 4])
+        assert rel_err(a, plain_logits(folder, [tok])) < REL_TOL["float32"]
+        assert torch.equal(a[0], b[0])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_stays_on_the_plain_model(dtype, sharp_folders):
+    folder, name = sharp_folders["C", dtype], "C"
+    runner = load_runner(folder, DT[dtype], num_pages=24)
+    ids = seeded_ids(11, 300, TINY[name]["vocab_size"])
+    want = plain_logits(folder, ids)
+    runner.add_request("d")
+    got = [runner.step([StepEntry("d", ids[:5], [4])]).cpu()[0]]
+    for p in range(5, 300):
+        got.append(runner.step([StepEntry("d", [ids[p]], [0])]).cpu()[0])
+        runner.manager.check()
+    assert rel_err(torch.stack(got), want[4:]) < REL_TOL[dtype]
+    # the windowed group kept only the pages a window of 24 can still see
+    held = sum(1 for p in runner.manager.block_table("d", 1) if p >= 0)
+    assert held <= 24 // 16 + 2 and sum(1 for p in runner.manager.block_table("d", 0) if p >= 0) == -(-300 // 16)
+
+
+def test_float32_results_do_not_depend_on_the_cutting_bit_for_bit(sharp_folders):
+    folder = sharp_folders["A"]
+    runner = load_runner(folder, torch.float32, num_pages=32)
+    ids = seeded_ids(12, 150, 512)
+    whole = run_whole(runner, "w", ids)
+    runner.add_request("filler")                           # other pages, another batch composition
+    runner.step([StepEntry("filler", ids[:37], [])])
+    runner.add_request("c")
+    rows, p = [], 0
+    for m in (64, 1, 2, 17, 1, 65):
+        rows.append(runner.step([StepEntry("filler", [5], [0]), StepEntry("c", ids[p:p + m], list(range(m)))]).cpu()[1:])
+        p += m
+    assert torch.equal(torch.cat(rows), whole)
+
+
+def test_step_refuses_bad_input_and_changes_nothing(sharp_folders):
+    runner = load_runner(sharp_folders["A"], torch.float32, num_pages=4)
+    runner.add_request("a")
+    with pytest.raises(StepError, match="outside"):
+        runner.step([StepEntry("a", [1, 512], [0])])
+    with pytest.raises(StepError, match="not live"):
+        runner.step([StepEntry("b", [1], [0])])
+    with pytest.raises(StepError, match="wanted places"):
+        runner.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(StepError, match="twice"):
+        runner.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(StepError, match="max_position"):
+        runner.step([StepEntry("a", [1] * 257, [])])
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("a", [1] * 65, [])])       # 5 pages wanted, 4 in the pool
+    assert runner.length("a") == 0 and runner.manager.free_pages() == [4]
+    runner.step([StepEntry("a", [1] * 64, [63])])
+    assert runner.manager.free_pages() == [0]
+    runner.manager.check()
+
+
+# ---- parts alone ----------------------------------------------------------------------------
+def test_parts_alone(sharp_folders):
+    """Each part of a layer against its plain function, on the layer's own weights."""
+    from inferflux_amd.engine.context import StepContext
+    folder = sharp_folders["B"]
+    cfg, W = pm.load_folder(folder, torch.float64)
+    runner = load_runner(folder, torch.float32, num_pages=16)
+    model = runner.model
+    ids = seeded_ids(13, 40, 1000)
+    runner.add_request("p")
+    runner.manager.reserve("p", len(ids))
+    ctx = StepContext([StepEntry("p", ids, [0, 39])], runner.manager, torch.float32, runner.device)
+    dev = runner.device
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(40, 144, generator=g)
+    blk, p = model.blocks[1], "model.layers.1"
+    # embedding
+    assert torch.equal(model.embedding.forward(ctx.token_ids).cpu().double(), W["model.embed_tokens.weight"][ids])
+    # norm (with and without a pending delta)
+    delta = torch.randn(40, 144, generator=g)
+    res = x.to(dev).clone()
+    got = blk.norm_in.forward(res, delta.to(dev), torch.float32).cpu().double()
+    assert torch.allclose(got, pm.rms_norm((x + delta).double(), W[f"{p}.input_layernorm.weight"], cfg["rms_norm_eps"]), atol=1e-5)
+    # feed-forward
+    got = blk.ffn.forward(x.to(dev), ctx).cpu().double()
+    want = pm.swiglu(x.double(), W[f"{p}.mlp.gate_proj.weight"], W[f"{p}.mlp.up_proj.weight"], W[f"{p}.mlp.down_proj.weight"])
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+    # mixer (attention with bias, rotary and cache write) on arbitrary input rows
+    got = blk.mixer.forward(x.to(dev), ctx, runner.storage.binding(1)).cpu().double()
+    want = pm.attention_block(x.double(), W, cfg, 1, list(range(40)))
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+    # head
+    h = torch.randn(3, 144, generator=g)
+    assert torch.allclose(model.head.forward(h.to(dev)).cpu().double(), h.double() @ W["lm_head.weight"].t(), rtol=1e-4, atol=1e-5)
+
+
+# ---- a toy mixer with state of its own --------------------------------------------------------
+def test_a_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A mixer defined here (a running decayed sum per request, kept in a state slot, no cache) is
+    registered, put into a plan beside an attention layer, built, loaded and stepped, without any
+    change to the package.  Its result must not depend on how the sequence is cut."""
+    from inferflux_amd.config.base import ModelConfig
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.parts import (LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec, ScheduleEntry, StateSpec,
+                                     register_part)
+
+    H, V = 32, 50
+
+    @register_part("mixer", "toy_decay_sum")
+    class DecaySum(Mixer):
+        def __init__(self, name, hidden_size, decay):
+            self.name, self.H, self.decay = name, hidden_size, decay
+        def param_specs(self):
+            return {f"{self.name}.mix.weight": ParamSpec((self.H, self.H))}
+        def load(self, tensors):
+            self.w = tensors[f"{self.name}.mix.weight"]
+        def state_spec(self):
+            return StateSpec((self.H,), "float32")
+        def forward(self, h, ctx, binding):
+            out = torch.empty_like(h)
+            for r in range(ctx.n_requests):                       # rows of a request in position order
+                s = binding.state[int(ctx.h_state_slots[r])]
+                a, n = int(ctx.h_q_start[r]), int(ctx.h_q_len[r])
+                for t in range(a, a + n):
+                    s.mul_(self.decay).add_(h[t].float())
+                    out[t] = s.to(h.dtype)
+            return out @ self.w.t()
+
+    def layer(i, mixer):
+        p = f"toy.layers.{i}"
+        return LayerSpec(p, PartSpec("prenorm"), PartSpec("rmsnorm", {"name": f"{p}.n1", "eps": 1e-5}), mixer,
+                         PartSpec("rmsnorm", {"name": f"{p}.n2", "eps": 1e-5}),
+                         PartSpec("swiglu", {"name": f"{p}.mlp", "intermediate_size": 48}))
+
+    attn = PartSpec("paged_attention", {"name": "toy.layers.0.attn", "n_heads": 2, "n_kv_heads": 1, "head_dim": 16,
+                                        "bias": False, "position": PartSpec("rotary", {"head_dim": 16, "theta": 100.0})})
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=128,
+                     embedding=PartSpec("token_embedding", {"name": "toy.embed", "vocab_size": V}),
+                     layers=(layer(0, attn), layer(1, PartSpec("toy_decay_sum", {"name": "toy.layers.1.mixer", "decay": 0.9}))),
+                     schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_from=0), ScheduleEntry(1)),
+                     final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
+    model = Model(plan=plan).init_random(3, torch.float32, "cuda")
+    runner = ModelRunner(model, num_pages=16, max_requests=3)
+    assert [g.entries for g in runner.storage.groups] == [(0,)]          # one cache owner; entry 2 reads it
+    assert runner.storage.binding(2).writes_cache is False and runner.storage.binding(2).cache is runner.storage.binding(0).cache
+    assert runner.storage.binding(1).state.shape == (3, H) and runner.storage.binding(3).state is not runner.storage.binding(1).state
+    ids = seeded_ids(15, 60, V)
+    runner.add_request("w")
+    whole = runner.step([StepEntry("w", ids, list(range(60)))]).cpu()
+    runner.free_request("w")
+    runner.add_request("other"); runner.add_request("c")                 # "c" reuses the slot "w" left: state must be zero
+    rows, p = [], 0
+    for m in (7, 1, 2, 30, 1, 19):
+        out = runner.step([StepEntry("other", ids[p:p + 1], []), StepEntry("c", ids[p:p + m], list(range(m)))])
+        rows.append(out.cpu()); p += m
+    assert torch.allclose(torch.cat(rows), whole, rtol=1e-4, atol=1e-5)
+    assert not torch.allclose(whole[1:], whole[:-1])

@@ -1,0 +1,282 @@
+"""Each HIP kernel alone against a plain float64 reference of the same operation, at sizes other
+than the tiny models' (widths that are no power of two, odd row counts, several head sizes)."""
+import math
+
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    from inferflux_amd.kernels import ops
+
+DEV = "cuda"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def tol(dtype):
+    # float32: rounding of a few dozen operations; bfloat16: one rounding of the result (2^-9 relative)
+    return dict(rtol=2e-5, atol=2e-6) if dtype == F32 else dict(rtol=8e-3, atol=1e-3)
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embedding(dtype):
+    g = gen(1)
+    table = torch.randn(77, 100, generator=g).to(dtype)
+    ids = torch.tensor([0, 76, 5, 5, 33], dtype=torch.int32)
+    out = ops.embedding(ids.to(DEV), table.to(DEV))
+    assert out.dtype == F32 and torch.equal(out.cpu(), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("H", [100, 3584])
+@pytest.mark.parametrize("wdtype", [F32, BF16])
+def test_add_rmsnorm(dtype, H, wdtype):
+    g = gen(2)
+    T, eps = 7, 1e-5
+    res = torch.randn(T, H, generator=g)
+    delta = torch.randn(T, H, generator=g).to(dtype)
+    w = (1 + 0.3 * torch.randn(H, generator=g)).to(wdtype)
+    want_res = res.double() + delta.double()
+    want = pm.rms_norm(want_res, w.double(), eps)
+    r = res.to(DEV)
+    out = ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, dtype)
+    assert torch.allclose(r.cpu().double(), want_res, rtol=1e-6, atol=1e-6)        # the stream took the delta
+    assert torch.allclose(out.cpu().double(), want, **tol(dtype))
+    out2 = ops.add_rmsnorm(res.to(DEV), None, w.to(DEV), eps, dtype)                # no delta
+    assert torch.allclose(out2.cpu().double(), pm.rms_norm(res.double(), w.double(), eps), **tol(dtype))
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    r3 = res.to(DEV)
+    out3 = ops.add_rmsnorm(r3, delta.to(DEV), w.to(DEV), eps, dtype, rows.to(DEV))  # gathered rows: stream untouched
+    assert torch.equal(r3.cpu(), res)
+    assert torch.allclose(out3.cpu().double(), want[rows.long()], **tol(dtype))
+
+
+def test_rmsnorm_eps_is_inside_the_root():
+    x = torch.full((1, 64), 1e-4)
+    w = torch.ones(64)
+    a = ops.add_rmsnorm(x.to(DEV), None, w.to(DEV), 1e-6, F32).cpu()
+    assert torch.allclose(a, x / math.sqrt(1e-8 + 1e-6), rtol=1e-5)
+
+
+def cache_rows(k_cache, v_cache, slots, page_size):
+    """Read back [T, nKV, d] keys and values from the two page layouts."""
+    pages, offs = slots // page_size, slots % page_size
+    k = k_cache[pages.long(), :, offs.long(), :]
+    v = v_cache[pages.long(), :, :, offs.long()]
+    return k, v
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("style,rot", [("split_half", None), ("consecutive", None), ("split_half", 8), ("none", None)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_rope_append(dtype, style, rot, bias):
+    g = gen(3)
+    T, nH, nKV, d, P, pages, theta = 9, 5, 1, 24, 16, 6, 1e6
+    width = (nH + 2 * nKV) * d
+    qkv = torch.randn(T, width, generator=g).to(dtype)
+    b = (0.5 * torch.randn(width, generator=g)).to(dtype) if bias else None
+    positions = torch.tensor([0, 1, 2, 40, 41, 300, 7, 8, 1000], dtype=torch.int32)
+    slots = torch.tensor([5, 17, 95, 0, 31, 32, 64, 80, 47], dtype=torch.int32)
+    kc = torch.zeros(pages, nKV, P, d, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, nKV, d, P, dtype=dtype, device=DEV)
+    rd = rot or d
+    inv_freq = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64), 2.0 * torch.arange(rd // 2, dtype=torch.float64) / rd)).float()
+    code = {"split_half": ops.ROPE_SPLIT_HALF, "consecutive": ops.ROPE_CONSECUTIVE, "none": ops.ROPE_NONE}[style]
+    q = ops.rope_append(qkv.to(DEV), b.to(DEV) if bias else None, positions.to(DEV), slots.to(DEV),
+                        inv_freq.to(DEV) if style != "none" else None, code, rd, nH, nKV, d, kc, vc, P)
+    x = qkv.double() + (b.double() if bias else 0)
+    xq, xk, xv = x[:, : nH * d].view(T, nH, d), x[:, nH * d: (nH + nKV) * d].view(T, nKV, d), x[:, (nH + nKV) * d:].view(T, nKV, d)
+
+    def rope(t):
+        if style == "none":
+            return t
+        fn = pm.rope_split_half if style == "split_half" else pm.rope_consecutive
+        return torch.cat([fn(t[..., :rd], positions.tolist(), theta), t[..., rd:]], dim=-1)
+
+    # angles are formed in float (position * rounded frequency): allow that on top of the result's rounding
+    t = dict(rtol=tol(dtype)["rtol"], atol=tol(dtype)["atol"] + 2e-4)
+    assert torch.allclose(q.cpu().double(), rope(xq), **t)
+    k_got, v_got = cache_rows(kc.cpu(), vc.cpu(), slots, P)
+    assert torch.allclose(k_got.double(), rope(xk), **t)
+    assert torch.allclose(v_got.double(), xv, **tol(dtype))
+    written = torch.zeros(pages * P, dtype=torch.bool); written[slots.long()] = True
+    assert torch.all(kc.cpu().permute(0, 2, 1, 3).reshape(pages * P, -1)[~written] == 0)   # nothing else touched
+    assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P, -1)[~written] == 0)
+
+
+def test_rope_queries_only():
+    g = gen(4)
+    T, nH, d = 4, 3, 16
+    qo = torch.randn(T, nH * d, generator=g)
+    pos = torch.tensor([3, 4, 5, 6], dtype=torch.int32)
+    inv = (1.0 / torch.pow(torch.tensor(1e4, dtype=torch.float64), 2.0 * torch.arange(d // 2, dtype=torch.float64) / d)).float()
+    q = ops.rope_append(qo.to(DEV), None, pos.to(DEV), None, inv.to(DEV), ops.ROPE_SPLIT_HALF, d, nH, 0, d, None, None, 16)
+    assert torch.allclose(q.cpu().double(), pm.rope_split_half(qo.double().view(T, nH, d), pos.tolist(), 1e4), atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_swiglu(dtype):
+    g = gen(5)
+    gu = (3 * torch.randn(5, 2 * 37, generator=g)).to(dtype)
+    out = ops.swiglu(gu.to(DEV)).cpu().double()
+    gate, up = gu.double()[:, :37], gu.double()[:, 37:]
+    assert torch.allclose(out, gate / (1 + torch.exp(-gate)) * up, **tol(dtype))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 50, 33), (7, 64, 16), (65, 130, 257), (130, 3, 1000)])
+@pytest.mark.parametrize("adtype", [F32, BF16])
+def test_gemm_f32(M, N, K, adtype):
+    g = gen(6)
+    x = torch.randn(M, K, generator=g).to(adtype)
+    w = torch.randn(N, K, generator=g)
+    b = torch.randn(N, generator=g)
+    out = ops.gemm_f32(x.to(DEV), w.to(DEV), b.to(DEV), F32).cpu().double()
+    want = x.double() @ w.double().t() + b.double()
+    assert torch.allclose(out, want, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    # a row's result does not depend on how many rows are in the product
+    one = ops.gemm_f32(x[:1].contiguous().to(DEV), w.to(DEV), b.to(DEV), F32).cpu().double()
+    assert torch.equal(one[0], out[0])
+
+
+def test_gemm_f32_is_true_32_bit():
+    """Products whose exact value needs more than 10 or 8 mantissa bits survive: no reduced-precision matrix mode."""
+    K = 64
+    x = torch.full((1, K), 1.0 + 2.0 ** -12)
+    w = torch.full((3, K), 1.0 + 2.0 ** -11)
+    out = ops.gemm_f32(x.to(DEV), w.to(DEV), None, F32).cpu().double()
+    want = (x.double() @ w.double().t())
+    assert torch.allclose(out, want, rtol=3e-7, atol=0)
+    assert not torch.allclose(out, torch.full_like(out, float(K)), rtol=1e-4, atol=0)
+
+
+# ---- attention ------------------------------------------------------------------------------
+def paged_case(seed, lens_q, lens_past, nH, nKV, d, P, dtype, window=None, n_pages=None, sharp=None):
+    """Random q/k/v for several requests, keys and values scattered into shuffled pages.
+    Returns device operands and the plain float64 result for this step's rows."""
+    g = gen(seed)
+    R = len(lens_q)
+    kv_lens = [a + b for a, b in zip(lens_q, lens_past)]
+    blocks = [-(-n // P) for n in kv_lens]
+    n_pages = n_pages or sum(blocks) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kc = torch.zeros(n_pages, nKV, P, d, dtype=dtype)
+    vc = torch.zeros(n_pages, nKV, d, P, dtype=dtype)
+    width = max(blocks)
+    table = torch.full((R, width), -1, dtype=torch.int32)
+    qs, outs, row_req, positions = [], [], [], []
+    for r in range(R):
+        n, nq = kv_lens[r], lens_q[r]
+        k = torch.randn(n, nKV, d, generator=g).to(dtype)
+        v = torch.randn(n, nKV, d, generator=g).to(dtype)
+        q = torch.randn(nq, nH, d, generator=g).to(dtype)
+        if sharp is not None:
+            # plant one far key that every query of head 0 must find: a wrong page, mask or offset changes the result
+            j = sharp if sharp >= 0 else n + sharp
+            if 0 <= j < n:
+                k[j, 0] = (4.0 * q[-1, 0] / q[-1, 0].float().norm() * math.sqrt(d)).to(dtype)
+        pages = [perm.pop() for _ in range(blocks[r])]
+        table[r, : blocks[r]] = torch.tensor(pages, dtype=torch.int32)
+        for j in range(n):
+            kc[pages[j // P], :, j % P, :] = k[j]
+            vc[pages[j // P], :, :, j % P] = v[j]
+        qpos = list(range(n - nq, n))
+        outs.append(pm.attention(q.double(), k.double(), v.double(), window=window, q_positions=qpos, k_positions=list(range(n))))
+        qs.append(q); row_req += [r] * nq; positions += qpos
+    q_all = torch.cat(qs)
+    want = torch.cat(outs).reshape(q_all.shape[0], nH * d)
+    dev = lambda t: t.to(DEV)
+    return (dev(q_all), dev(kc), dev(vc), dev(torch.tensor(row_req, dtype=torch.int32)),
+            dev(torch.tensor(positions, dtype=torch.int32)), dev(table)), want, dict(q_lens=lens_q, kv_lens=kv_lens)
+
+
+ATTN_CASES = [
+    # lens_q, lens_past, nH, nKV, d, P, window, sharp
+    ([1], [0], 4, 2, 16, 16, None, None),                       # a single key: the output is its value
+    ([5, 1, 2], [0, 63, 17], 4, 2, 16, 16, None, None),
+    ([33, 1], [40, 200], 7, 1, 40, 16, None, 3),                # MQA 7:1, head size 40, far planted key
+    ([64, 2, 1, 16], [0, 62, 129, 48], 6, 3, 32, 16, None, None),
+    ([20, 1, 3], [30, 100, 45], 6, 3, 32, 16, 24, None),        # window's edge inside and across pages
+    ([1, 1], [70, 23], 2, 2, 64, 32, 5, -5),                    # planted key at the window's last visible place
+    ([1, 1], [70, 23], 2, 2, 64, 32, 5, -6),                    # ... and just outside it
+    ([7], [250], 28, 4, 128, 16, None, 0),                      # the 7B head layout, planted key at position 0
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_attention_plain(dtype, case):
+    lens_q, lens_past, nH, nKV, d, P, window, sharp = case
+    (q, kc, vc, row_req, positions, table), want, _ = paged_case(7, lens_q, lens_past, nH, nKV, d, P, dtype, window, sharp=sharp)
+    out = ops.attention_plain(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d)).cpu().double()
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == F32 else dict(rtol=1e-2, atol=1e-2)
+    assert torch.isfinite(out).all()
+    assert torch.allclose(out, want, **t), float((out - want).abs().max())
+
+
+# ---- sampling -------------------------------------------------------------------------------
+def test_argmax_lowest_index_wins_ties():
+    l = torch.zeros(3, 1500)
+    l[0, [700, 20, 1400]] = 5.0
+    l[1, 1499] = 1.0
+    l[2] = -float("inf")
+    assert ops.argmax(l.to(DEV)).cpu().tolist() == [20, 1499, 0]
+    g = gen(8)
+    r = torch.randn(6, 152064, generator=g)
+    assert ops.argmax(r.to(DEV)).cpu().tolist() == r.argmax(-1).tolist()
+
+
+def test_penalties_and_logit_bias():
+    l = torch.tensor([[2.0, -2.0, 1.0, 0.5], [1.0, 1.0, 1.0, 1.0]])
+    d = l.to(DEV)
+    i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    f32 = lambda *v: torch.tensor(v, dtype=torch.float32, device=DEV)
+    ops.apply_penalties(d, i32(0, 0, 1), i32(0, 1, 3), i32(1, 2, 4), f32(2.0, 1.0), f32(0.25, 0.5), f32(0.5, 0.0))
+    want0 = pm.apply_penalties(l[0], [0, 1, 1], 2.0, 0.25, 0.5)
+    want1 = pm.apply_penalties(l[1], [3, 3, 3, 3], 1.0, 0.5, 0.0)
+    assert torch.allclose(d.cpu(), torch.stack([want0, want1]))
+    ops.add_logit_bias(d, i32(1), i32(2), f32(-100.0))
+    assert float(d[1, 2]) == pytest.approx(1.0 - 100.0)
+
+
+@pytest.mark.parametrize("V", [1000, 152064])
+def test_sample_matches_the_plain_rule(V):
+    g = gen(9)
+    R = 12
+    logits = 3.0 * torch.randn(R, V, generator=g)
+    temps = torch.tensor([0.0, 1.0, 0.7, 1.3, 1.0, 1.0, 0.8, 1.0, 1.0, 0.5, 1.0, 2.0])
+    top_k = torch.tensor([0, 0, 0, 40, 0, 5, 50, 0, 1, 0, 0, 0], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 0.9, 1.0, 0.3, 0.95, 0.8, 1.0, 1.0, 1.0, 0.999, 1.0])
+    min_p = torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.02, 0.1, 0.0, 0.0, 0.0, 0.0])
+    u = torch.rand(R, generator=g)
+    got = ops.sample(logits.to(DEV), temps.to(DEV), top_k.to(DEV), top_p.to(DEV), min_p.to(DEV), u.to(DEV)).cpu().tolist()
+    assert got[0] == int(logits[0].argmax())
+    assert got[8] == int(logits[8].argmax())            # top_k = 1
+    for r in range(1, R):
+        w = pm.filtered_probs(logits[r], float(temps[r]), int(top_k[r]), float(top_p[r]), float(min_p[r]))
+        assert w[got[r]] > 0, (r, "a filtered-out token was drawn")
+        cum = torch.cumsum(w, 0) / w.sum()
+        lo = float(cum[got[r] - 1]) if got[r] > 0 else 0.0
+        hi = float(cum[got[r]])
+        assert lo - 1e-4 <= float(u[r]) <= hi + 1e-4, (r, got[r], lo, float(u[r]), hi)
+
+
+def test_sample_histogram_follows_the_probabilities():
+    g = gen(10)
+    V, N = 50, 4000
+    logits = torch.randn(V, generator=g)
+    rows = logits.repeat(N, 1)
+    ones = torch.ones(N)
+    u = torch.rand(N, generator=g)
+    got = ops.sample(rows.to(DEV), ones.to(DEV), torch.zeros(N, dtype=torch.int32, device=DEV), ones.to(DEV),
+                     torch.zeros(N, device=DEV), u.to(DEV)).cpu()
+    freq = torch.bincount(got.long(), minlength=V).double() / N
+    p = torch.softmax(logits.double(), -1)
+    chi2 = float((N * (freq - p) ** 2 / p).sum())
+    assert chi2 < 100.0, chi2                            # 49 degrees of freedom: 100 is far in the tail
