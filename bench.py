@@ -1,0 +1,142 @@
+"""Decode and prefill throughput of the engine at the Qwen2.5-7B shape, random weights, one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+A step is one decode step of the whole engine (scheduler, step function, sampling).  Prints one
+JSON line: decoded tokens a second at batch 8 as ``value``, the same at batch 1 and 64 under
+``points``, a 2,048-token prefill under ``prefill`` and the decode step's share of the HBM
+roofline under ``roofline``.
+"""
+import argparse
+import json
+import sys
+import time
+
+HBM_GBS = 8000.0           # MI355X published HBM3E bandwidth, GB/s
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+SHAPE_7B = dict(model_type="qwen2", architectures=["Qwen2ForCausalLM"], vocab_size=152064, hidden_size=3584,
+                num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
+                intermediate_size=18944, max_position_embeddings=32768, rope_theta=1000000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=False, attention_bias=True, use_sliding_window=False, torch_dtype="bfloat16")
+CONTEXT = 4096
+PROMPT = 2048
+DECODE_KV_START = 3072      # mean context of a 2,048-token decode after a 2,048-token prompt
+PAGE = 16
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has (both numbers are reported)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from inferflux_amd import SamplingParams
+    from inferflux_amd.config import config_from_dict
+    from inferflux_amd.engine.context import StepEntry
+    from inferflux_amd.engine.engine import Engine
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.engine.scheduler import SchedulerConfig
+
+    shape = dict(SHAPE_7B)
+    layers_full = shape["num_hidden_layers"]
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(shape)
+    tdt = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    esz = 2 if args.dtype == "bf16" else 4
+    dev = torch.device("cuda", 0)
+    t0 = time.time()
+    model = Model(cfg).init_random(0, tdt, dev)
+    torch.cuda.synchronize()
+    print(f"[bench] {cfg.num_hidden_layers}-layer model with random weights ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    L, H, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    nH, nKV, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    layer_params = (nH + 2 * nKV) * d * H + (nH + 2 * nKV) * d + nH * d * H + 3 * I * H + 2 * H
+    weight_bytes = (L * layer_params + H + V * H) * esz          # every weight a decode step uses, once
+    kv_bytes_per_token = 2 * L * nKV * d * esz
+    gen = torch.Generator().manual_seed(1)
+
+    def make_engine(batch, kv_tokens):
+        pages = batch * (-(-kv_tokens // PAGE) + 1)
+        runner = ModelRunner(model, num_pages=pages, page_size=PAGE, max_requests=batch)
+        return Engine(runner, SchedulerConfig(max_batch_size=batch, max_batch_tokens=16384, chunked_prefill_tokens=2048))
+
+    def decode_rate(batch, steps, warmup):
+        """tokens/s and ms/step of ``steps`` decode steps at ``batch`` with contexts from DECODE_KV_START."""
+        eng = make_engine(batch, DECODE_KV_START + steps + warmup + 2)
+        sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
+        for _ in range(batch):
+            eng.add_request(torch.randint(0, V, (DECODE_KV_START,), generator=gen).tolist(), SamplingParams(**vars(sp)))
+        while any(s.is_prefilling for s in eng.scheduler.running) or eng.scheduler.waiting:
+            eng.step()                                            # prompts in; every request now decodes
+        for _ in range(warmup):
+            eng.step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            eng.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        kv_mean = DECODE_KV_START + warmup + steps / 2
+        del eng
+        torch.cuda.empty_cache()
+        return batch * steps / dt, dt / steps * 1e3, kv_mean
+
+    def prefill_rate(tokens, reps=3):
+        runner = ModelRunner(model, num_pages=-(-tokens // PAGE) + 1, page_size=PAGE, max_requests=2)
+        ids = torch.randint(0, V, (tokens,), generator=gen).tolist()
+        best = None
+        for i in range(reps + 1):
+            runner.add_request(i)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.step([StepEntry(i, ids, [tokens - 1])])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            runner.free_request(i)
+            if i > 0:
+                best = dt if best is None else min(best, dt)
+        linear = 2.0 * tokens * L * ((nH + 2 * nKV) * d * H + nH * d * H + 3 * I * H) + 2.0 * V * H
+        attn = 4.0 * L * nH * d * tokens * (tokens + 1) / 2
+        return tokens / best, best * 1e3, (linear + attn) / best / 1e12 / PEAK_TFLOPS[args.dtype]
+
+    tps, ms, kv_mean = decode_rate(args.batch, args.steps, args.warmup)
+    step_bytes = weight_bytes + args.batch * kv_mean * kv_bytes_per_token
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+    out = {
+        "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-7B shape, {args.dtype}, random weights)",
+        "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (uniform random token ids, seeded N(0,0.02) weights)",
+        "config": {"model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "1 GPU",
+                   "num_hidden_layers": layers_full, "layers_run": L, "hidden_size": H, "num_attention_heads": nH,
+                   "num_key_value_heads": nKV, "head_dim": d, "intermediate_size": I, "vocab_size": V,
+                   "prompt_len": PROMPT, "decode_kv_start": DECODE_KV_START, "kv_page_size": PAGE,
+                   "tie_word_embeddings": False, "attention_bias": True},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBS, 4)},
+    }
+    if not args.no_points:
+        ptps, pms, pfrac = prefill_rate(PROMPT)
+        out["prefill"] = {"value": round(ptps, 1), "tokens": PROMPT, "ms": round(pms, 3), "frac": round(pfrac, 4)}
+        b1 = decode_rate(1, min(args.steps, 32), min(args.warmup, 4))[0]
+        b64 = decode_rate(64, min(args.steps, 32), min(args.warmup, 4))[0]
+        out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -160,6 +160,9 @@ class CacheManager:
     def free_pages(self) -> List[int]:
         return [p.num_free for p in self.pools]
 
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
     def can_reserve(self, needs: Sequence[Tuple[Hashable, int]]) -> bool:
         """Whether all of ``needs`` [(request, n_new)] fit at once."""
         tot = [0] * len(self.groups)

@@ -31,11 +31,18 @@ def register_architecture(config_cls: Type[ModelConfig], plan_builder: Callable,
         _ARCHITECTURES[key] = (config_cls, plan_builder)
 
 
+def _ensure_builtin() -> None:
+    """The built-in architectures register themselves when their package is imported."""
+    from .. import architectures  # noqa: F401
+
+
 def registered_architectures():
+    _ensure_builtin()
     return sorted(_ARCHITECTURES)
 
 
 def resolve_architecture(d: Mapping[str, Any]) -> Tuple[Type[ModelConfig], Callable]:
+    _ensure_builtin()
     candidates = []
     mt = d.get("model_type")
     if isinstance(mt, str) and mt:
@@ -64,6 +71,7 @@ def load_config(folder: str) -> ModelConfig:
 
 def plan_for(config: ModelConfig):
     """The ModelPlan of a typed config, through the architecture's registered builder."""
+    _ensure_builtin()
     hit = _ARCHITECTURES.get(config.model_type.lower())
     if hit is None:
         raise ConfigError(f"architecture '{config.model_type}' is not registered")

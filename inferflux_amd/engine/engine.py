@@ -1,0 +1,158 @@
+"""The engine: requests in, tokens out.  Scheduler above, step function below, sampler beside.
+
+Programming interface in the shape of the reference's runtime (LoadModel / ExecuteUnifiedBatch /
+NativeFreeSequence / Generate: runtime/backends/native/native_inference_runtime.h:34-37, 91):
+``Engine.load`` (a model folder), ``add_request``, ``step`` (one scheduled step; returns what
+finished), ``abort``, ``generate`` (run a list of prompts to completion), ``stats`` (the
+reference's perf snapshot {prefill_ms, decode_ms, prompt_tokens, generated_tokens},
+native_inference_runtime.h:58-64).  Prompts are token ids; text is outside the engine.
+"""
+from __future__ import annotations
+
+import dataclasses
+import time
+from typing import Callable, Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler, SamplingState
+from .api import load_runner
+from .context import StepEntry
+from .runner import ModelRunner
+from .scheduler import RequestRefused, Scheduler, SchedulerConfig, Sequence_
+
+
+@dataclasses.dataclass
+class RequestOutput:
+    request_id: Hashable
+    prompt_token_ids: List[int]
+    token_ids: List[int]
+    finish_reason: Optional[str] = None      # "stop" (eos or a stop token), "length", "abort"; None while running
+    preemptions: int = 0
+
+    @property
+    def finished(self) -> bool:
+        return self.finish_reason is not None
+
+
+@dataclasses.dataclass
+class EngineStats:
+    prefill_ms: float = 0.0
+    decode_ms: float = 0.0
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    steps: int = 0
+    preemptions: int = 0
+
+
+class _Live:
+    def __init__(self, seq: Sequence_, params: SamplingParams, prompt: List[int]):
+        self.seq, self.params, self.prompt = seq, params, prompt
+        self.sampling = SamplingState.start(params)
+
+
+class Engine:
+    def __init__(self, runner: ModelRunner, scheduler_config: Optional[SchedulerConfig] = None):
+        self.runner = runner
+        self.config = scheduler_config or SchedulerConfig()
+        self.config.max_batch_size = min(self.config.max_batch_size, runner.manager.max_requests)
+        self.scheduler = Scheduler(runner.manager, self.config, runner.max_position)
+        self.sampler = Sampler(runner.device)
+        self.eos_token_id = runner.model.plan.eos_token_id
+        self._live: Dict[Hashable, _Live] = {}
+        self._next_id = 0
+        self.stats = EngineStats()
+
+    @classmethod
+    def load(cls, model: str, dtype: str = "bfloat16", kv_pages: int = 1024, page_size: int = 16,
+             max_batch_size: int = 32, max_batch_tokens: int = 16384, chunked_prefill_tokens: int = 512) -> "Engine":
+        dt = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}[dtype]
+        runner = load_runner(model, dt, num_pages=kv_pages, page_size=page_size, max_requests=max_batch_size)
+        return cls(runner, SchedulerConfig(max_batch_size, max_batch_tokens, chunked_prefill_tokens))
+
+    # ---- requests -----------------------------------------------------------------
+    def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                    request_id: Optional[Hashable] = None) -> Hashable:
+        params = params or SamplingParams()
+        params.validate()
+        prompt = [int(t) for t in prompt_token_ids]
+        bad = [t for t in prompt if not (0 <= t < self.runner.vocab_size)]
+        if bad:
+            raise RequestRefused(f"token ids {bad[:8]} outside [0, {self.runner.vocab_size})")
+        if request_id is None:
+            request_id = self._next_id
+            self._next_id += 1
+        seq = self.scheduler.add(request_id, prompt, params.max_tokens)
+        self._live[request_id] = _Live(seq, params, prompt)
+        self.stats.prompt_tokens += len(prompt)
+        return request_id
+
+    def abort(self, request_id: Hashable) -> Optional[RequestOutput]:
+        live = self._live.pop(request_id, None)
+        if live is None:
+            return None
+        self.scheduler.finish(live.seq)
+        return RequestOutput(request_id, live.prompt, list(live.seq.generated), "abort", live.seq.preemptions)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ---- one step -------------------------------------------------------------------
+    def _finish_reason(self, live: _Live, token: int) -> Optional[str]:
+        p = live.params
+        if not p.ignore_eos and self.eos_token_id is not None and token == self.eos_token_id:
+            return "stop"
+        if token in p.stop_token_ids:
+            return "stop"
+        if len(live.seq.generated) >= p.max_tokens:
+            return "length"
+        return None
+
+    def step(self, on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[RequestOutput]:
+        """Run one scheduled step; returns the requests that finished in it."""
+        plan = self.scheduler.schedule()
+        self.stats.preemptions += len(plan.preempted)
+        if not plan.items:
+            if self.scheduler.has_work():
+                raise RuntimeError("the scheduler has work but could plan nothing (pool too small for any request?)")
+            return []
+        t0 = time.perf_counter()
+        entries = [StepEntry(i.seq.rid, i.tokens, [len(i.tokens) - 1] if i.wants_logits else []) for i in plan.items]
+        logits = self.runner.step(entries)
+        wanting = [i for i in plan.items if i.wants_logits]
+        tokens = self.sampler.sample(logits, [self._live[i.seq.rid].sampling for i in wanting]) if wanting else []
+        dt = (time.perf_counter() - t0) * 1e3
+        if any(len(i.tokens) > 1 or i.seq.is_prefilling for i in plan.items):
+            self.stats.prefill_ms += dt
+        else:
+            self.stats.decode_ms += dt
+        self.stats.steps += 1
+        for i in plan.items:
+            self.scheduler.advance(i)
+        done: List[RequestOutput] = []
+        for i, tok in zip(wanting, tokens):
+            live = self._live[i.seq.rid]
+            i.seq.generated.append(int(tok))
+            self.stats.generated_tokens += 1
+            if on_token is not None:
+                on_token(i.seq.rid, int(tok))
+            reason = self._finish_reason(live, int(tok))
+            if reason is not None:
+                self.scheduler.finish(i.seq)
+                del self._live[i.seq.rid]
+                done.append(RequestOutput(i.seq.rid, live.prompt, list(i.seq.generated), reason, i.seq.preemptions))
+        return done
+
+    def generate(self, prompts: Sequence[Sequence[int]], params=None,
+                 on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[RequestOutput]:
+        """Run ``prompts`` (lists of token ids) to completion; results in the order of the prompts.
+        ``params`` is one SamplingParams for all or one per prompt."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [dataclasses.replace(params) if params else SamplingParams() for _ in prompts]
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        results: Dict[Hashable, RequestOutput] = {}
+        while any(i not in results for i in ids):
+            for out in self.step(on_token):
+                results[out.request_id] = out
+        return [results[i] for i in ids]

@@ -1,0 +1,1 @@
+from .params import UNSEEDED, SamplingParams, philox_uniform
