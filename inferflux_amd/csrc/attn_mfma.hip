@@ -1,0 +1,382 @@
+// Attention over the paged cache on the matrix cores (bf16 in, float accumulate), for one head
+// size fixed at compile time (-DHEAD_DIM=..., a multiple of 16 up to 256).
+//
+// Two kernels compute the same function as attn_plain.hip (causal, optionally windowed,
+// grouped-query attention; reference formula runtime/backends/cuda/kernels/flash_attention.cu:
+// 71-72, 86, 144, 152-173; split merge 944-991):
+//
+//   rows   one wave per (row, kv head, split of the key range): the query heads that share the
+//          kv head are the 16 columns of the matrix tile, so keys and values are read once for
+//          all of them (any group size; more than 16 heads take several passes).  Partial
+//          results (max, sum, unnormalised output) go to scratch and a second kernel merges
+//          the splits.  For decode tokens and short portions.
+//   tiles  one workgroup of 4 waves per (64 consecutive rows of one request, query head): key
+//          and value tiles of 64 positions are staged in LDS and shared by the 4 waves.  For
+//          long portions of prompts.
+//
+// Both work on transposed tiles so that no register shuffle is needed between the two matrix
+// products: S^T[key, q] = K Q^T leaves each lane holding four consecutive keys of one query
+// column, which is exactly the operand layout of O^T[dim, q] += V^T[dim, key] P^T[key, q].
+// The cache layouts make both A operands contiguous: K [page][kv head][offset][d] and
+// V [page][kv head][d][offset].
+//
+// Softmax runs in float on the accumulators (base-2 exponent with the scale folded in); P is
+// rounded to bf16 for the second product, the row sum is kept in float.
+#include "common.h"
+
+IFX_DEFINE_LAST_ERROR()
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<multiple of 16>"
+#endif
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "HEAD_DIM must be a multiple of 16 in 16..256");
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+constexpr int D = HEAD_DIM;
+constexpr int KS = (D + 31) / 32;  // 32-wide steps of the QK product (the last one half empty when D % 32 == 16)
+constexpr int DT = D / 16;         // 16-wide tiles of the output's head dimension
+
+extern "C" int ifx_attn_head_dim() { return D; }
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+__device__ __forceinline__ bf16x8 join4(bf16x4 a, bf16x4 b) {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { r[i] = a[i]; r[i + 4] = b[i]; }
+  return r;
+}
+
+__device__ __forceinline__ bf16x4 zero4() {
+  bf16x4 z;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// max over the four lanes that hold the same query column (lane, lane^16, lane^32, lane^48)
+__device__ __forceinline__ float col_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+  v = fmaxf(v, __shfl_xor(v, 32, WAVE));
+  return v;
+}
+__device__ __forceinline__ float col_sum(float v) {
+  v += __shfl_xor(v, 16, WAVE);
+  v += __shfl_xor(v, 32, WAVE);
+  return v;
+}
+
+// =======================================================================================
+// rows
+// =======================================================================================
+struct RowArgs {
+  const bf16_t* q;        // [T, nH, D]
+  const bf16_t* k_cache;  // [pages, nKV, P, D]
+  const bf16_t* v_cache;  // [pages, nKV, D, P]
+  const int* rows;        // [n_rows] rows of the batch this launch handles (nullptr: rows 0..n_rows-1)
+  const int* row_req;     // [T]
+  const int* positions;   // [T]
+  const int* block_table; // [R, max_blocks], -1 where no page
+  float* part_o;          // [n_rows, nH, max_splits, D]
+  float* part_ml;         // [n_rows, nH, max_splits, 2]
+  bf16_t* out;            // [T, nH * D]
+  int max_blocks, n_rows, nH, nKV, P, window, chunk, max_splits;
+  float scale_log2e;
+};
+
+__global__ __launch_bounds__(WAVE) void attn_rows_kernel(RowArgs a) {
+  const int split = blockIdx.x, kvh = blockIdx.y, ri = blockIdx.z;
+  const int lane = threadIdx.x, col = lane & 15, g4 = lane >> 4;
+  const int row = a.rows ? a.rows[ri] : ri;
+  const int pos = a.positions[row];
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int ka = max(lo, split * a.chunk), kb = min(pos + 1, (split + 1) * a.chunk);  // keys [ka, kb)
+  const int ratio = a.nH / a.nKV;
+  const int P = a.P;
+  const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
+
+  for (int qt = 0; qt < ratio; qt += 16) {
+    const int head = kvh * ratio + qt + col;
+    const bool head_ok = qt + col < ratio;
+    float* po = a.part_o + (((size_t)ri * a.nH + head) * a.max_splits + split) * D;
+    float* pml = a.part_ml + (((size_t)ri * a.nH + head) * a.max_splits + split) * 2;
+    if (ka >= kb) {  // nothing of this split is visible: the merge skips it
+      if (head_ok && g4 == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
+      continue;
+    }
+    bf16x8 qop[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = 32 * ks + 8 * g4;
+      qop[ks] = (head_ok && c < D) ? *(const bf16x8*)(a.q + ((size_t)row * a.nH + head) * D + c) : zero8();
+    }
+    floatx4 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int j0 = (ka / 32) * 32; j0 < kb; j0 += 32) {
+      floatx4 s[2];
+      int page[2], off[2];
+      bool live[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int k0 = j0 + 16 * t;  // 16 keys k0..k0+15, all in one page
+        live[t] = k0 < kb && k0 + 16 > ka;
+        page[t] = live[t] ? table[k0 / P] : -1;
+        off[t] = k0 % P;
+        live[t] = live[t] && page[t] >= 0;
+        s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (live[t]) {
+          const bf16_t* kp = a.k_cache + (((size_t)page[t] * a.nKV + kvh) * P + off[t] + col) * D + 8 * g4;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 kop = (32 * ks + 8 * g4 < D) ? *(const bf16x8*)(kp + 32 * ks) : zero8();
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[ks], s[t], 0, 0, 0);
+          }
+        }
+      }
+      float mb = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = j0 + 16 * t + 4 * g4 + r;
+          const bool vis = live[t] && key >= ka && key < kb;
+          s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
+          mb = fmaxf(mb, s[t][r]);
+        }
+      const float m_new = fmaxf(m, col_max(mb));
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = exp2f(m - m_safe);
+      float psum = 0.f;
+      bf16x4 pb[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = exp2f(s[t][r] - m_safe);
+          psum += p;
+          pb[t][r] = (__bf16)p;
+        }
+      l = l * alpha + psum;
+      m = m_new;
+      const bf16x8 pop = join4(pb[0], pb[1]);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        bf16x4 v0 = zero4(), v1 = zero4();
+        if (live[0]) v0 = *(const bf16x4*)(a.v_cache + (((size_t)page[0] * a.nKV + kvh) * D + 16 * dt + col) * P + off[0] + 4 * g4);
+        if (live[1]) v1 = *(const bf16x4*)(a.v_cache + (((size_t)page[1] * a.nKV + kvh) * D + 16 * dt + col) * P + off[1] + 4 * g4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join4(v0, v1), pop, o[dt], 0, 0, 0);
+      }
+    }
+    l = col_sum(l);
+    if (head_ok) {
+      if (g4 == 0) { pml[0] = m; pml[1] = l; }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = o[dt];
+    }
+  }
+}
+
+// out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s
+__global__ void attn_rows_merge_kernel(RowArgs a) {
+  const int ri = blockIdx.x, head = blockIdx.y;
+  const int row = a.rows ? a.rows[ri] : ri;
+  const int pos = a.positions[row];
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int s0 = lo / a.chunk, s1 = pos / a.chunk;  // first and last split that hold a visible key
+  const float* po = a.part_o + ((size_t)ri * a.nH + head) * a.max_splits * D;
+  const float* pml = a.part_ml + ((size_t)ri * a.nH + head) * a.max_splits * 2;
+  float M = -INFINITY;
+  for (int s = s0; s <= s1; ++s) M = fmaxf(M, pml[2 * s]);
+  for (int e = threadIdx.x; e < D; e += blockDim.x) {
+    float L = 0.f, acc = 0.f;
+    for (int s = s0; s <= s1; ++s) {
+      const float ms = pml[2 * s];
+      if (ms == -INFINITY) continue;
+      const float w = exp2f(ms - M);
+      L += w * pml[2 * s + 1];
+      acc += w * po[(size_t)s * D + e];
+    }
+    a.out[((size_t)row * a.nH + head) * D + e] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+  }
+}
+
+extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_cache, void* out, const int* rows,
+                             const int* row_req, const int* positions, const int* block_table, int max_blocks,
+                             int n_rows, int nH, int nKV, int d, int page_size, int window, int chunk,
+                             int max_splits, float scale, float* part_o, float* part_ml, void* stream) {
+  IFX_REQUIRE(d == D, "attn_rows: built for head_dim %d, called with %d", D, d);
+  IFX_REQUIRE(n_rows >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_rows: bad head counts nH=%d nKV=%d", nH, nKV);
+  IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_rows: page_size %d must be a multiple of 16", page_size);
+  IFX_REQUIRE(chunk > 0 && chunk % 32 == 0 && max_splits > 0 && max_splits <= 65535, "attn_rows: bad chunk %d / splits %d", chunk, max_splits);
+  IFX_REQUIRE(nKV <= 65535 && n_rows <= 65535, "attn_rows: too many kv heads or rows for one launch");
+  if (n_rows == 0) return 0;
+  RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
+            part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
+            scale * 1.4426950408889634f};
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(attn_rows_kernel, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+  hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(D >= 128 ? 128 : 64), 0, s, a);
+  IFX_LAUNCH_CHECK();
+}
+
+// =======================================================================================
+// tiles
+// =======================================================================================
+constexpr int TQ = 64;            // query rows per workgroup (16 per wave)
+constexpr int TK = 64;            // keys per staged tile
+constexpr int KPAD = D + 8;       // bf16 elements per K row in LDS
+constexpr int VPAD = TK + 8;      // bf16 elements per V^T row in LDS
+
+struct TileArgs {
+  const bf16_t* q;
+  const bf16_t* k_cache;
+  const bf16_t* v_cache;
+  bf16_t* out;
+  const int* tile_req;    // [n_tiles] request of each tile
+  const int* tile_q0;     // [n_tiles] first row of the tile within its request's rows
+  const int* q_start;     // [R] first batch row of each request
+  const int* q_len;       // [R]
+  const int* kv_len;      // [R] length after this step
+  const int* block_table;
+  int max_blocks, nH, nKV, P, window;
+  float scale_log2e;
+};
+
+__global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t k_s[TK * KPAD];
+  __shared__ __attribute__((aligned(16))) bf16_t v_s[D * VPAD];
+  const int tid = threadIdx.x, wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g4 = lane >> 4;
+  const int req = a.tile_req[blockIdx.x], q0 = a.tile_q0[blockIdx.x], head = blockIdx.y;
+  const int kvh = head / (a.nH / a.nKV);
+  const int qlen = a.q_len[req], kvlen = a.kv_len[req], P = a.P;
+  const int start = kvlen - qlen;                       // position of the request's first row in this step
+  const int* table = a.block_table + (size_t)req * a.max_blocks;
+  const int rows_here = min(TQ, qlen - q0);
+  const int pos_first = start + q0, pos_last = pos_first + rows_here - 1;
+  const int lo_wg = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+
+  const int my_q = q0 + 16 * wid + col;                 // this lane's query column, as a row of the request
+  const bool q_ok = my_q < qlen;
+  const int my_pos = start + my_q;
+  const int my_lo = a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
+  const size_t my_row = (size_t)a.q_start[req] + my_q;
+  bf16x8 qop[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int c = 32 * ks + 8 * g4;
+    qop[ks] = (q_ok && c < D) ? *(const bf16x8*)(a.q + (my_row * a.nH + head) * D + c) : zero8();
+  }
+  floatx4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int j0 = (lo_wg / TK) * TK; j0 <= pos_last; j0 += TK) {
+    __syncthreads();  // everyone is done with the previous tile
+    // K tile: TK rows of D elements, in 16-byte pieces
+    for (int c = tid; c < TK * (D / 8); c += 256) {
+      const int key = c / (D / 8), c8 = c % (D / 8);
+      const int j = j0 + key, blk = j / P;
+      const int page = (j <= pos_last && blk < a.max_blocks) ? table[blk] : -1;
+      bf16x8 v = zero8();
+      if (page >= 0) v = *(const bf16x8*)(a.k_cache + (((size_t)page * a.nKV + kvh) * P + j % P) * D + 8 * c8);
+      *(bf16x8*)(k_s + key * KPAD + 8 * c8) = v;
+    }
+    // V^T tile: D rows of TK keys, in 16-byte pieces of 8 keys (8 keys never straddle a page)
+    for (int c = tid; c < D * (TK / 8); c += 256) {
+      const int dim = c / (TK / 8), k8 = c % (TK / 8);
+      const int j = j0 + 8 * k8, blk = j / P;
+      const int page = (j <= pos_last && blk < a.max_blocks) ? table[blk] : -1;
+      bf16x8 v = zero8();
+      if (page >= 0) v = *(const bf16x8*)(a.v_cache + (((size_t)page * a.nKV + kvh) * D + dim) * P + j % P);
+      *(bf16x8*)(v_s + dim * VPAD + 8 * k8) = v;
+    }
+    __syncthreads();
+
+    floatx4 s[4];
+    float mb = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int c = 32 * ks + 8 * g4;
+        const bf16x8 kop = c < D ? *(const bf16x8*)(k_s + (16 * t + col) * KPAD + c) : zero8();
+        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[ks], s[t], 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = j0 + 16 * t + 4 * g4 + r;
+        const bool vis = q_ok && key <= my_pos && key >= my_lo;
+        s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
+        mb = fmaxf(mb, s[t][r]);
+      }
+    }
+    const float m_new = fmaxf(m, col_max(mb));
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(m - m_safe);
+    float psum = 0.f;
+    bf16x4 pb[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = exp2f(s[t][r] - m_safe);
+        psum += p;
+        pb[t][r] = (__bf16)p;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    const bf16x8 pop0 = join4(pb[0], pb[1]), pop1 = join4(pb[2], pb[3]);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 4 * g4;
+      const bf16x8 vop0 = join4(*(const bf16x4*)(vr), *(const bf16x4*)(vr + 16));
+      const bf16x8 vop1 = join4(*(const bf16x4*)(vr + 32), *(const bf16x4*)(vr + 48));
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop0, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop1, o[dt], 0, 0, 0);
+    }
+  }
+  l = col_sum(l);
+  if (q_ok) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* orow = a.out + (my_row * a.nH + head) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x4 w;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) w[r] = (__bf16)(o[dt][r] * inv);
+      *(bf16x4*)(orow + 16 * dt + 4 * g4) = w;
+    }
+  }
+}
+
+extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_cache, void* out,
+                              const int* tile_req, const int* tile_q0, int n_tiles, const int* q_start,
+                              const int* q_len, const int* kv_len, const int* block_table, int max_blocks,
+                              int nH, int nKV, int d, int page_size, int window, float scale, void* stream) {
+  IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
+  IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
+  IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_tiles: page_size %d must be a multiple of 16", page_size);
+  IFX_REQUIRE(nH <= 65535, "attn_tiles: too many heads for one launch");
+  if (n_tiles == 0) return 0;
+  TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
+             q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f};
+  hipLaunchKernelGGL(attn_tiles_kernel, dim3(n_tiles, nH), dim3(256), 0, (hipStream_t)stream, a);
+  IFX_LAUNCH_CHECK();
+}

@@ -1,18 +1,63 @@
-"""Chooses the attention kernel for a step.
+"""Chooses the attention kernels for a step.
 
 Every choice computes the same function (causal, optionally windowed, grouped-query attention
-over the paged cache); they differ in speed and in which sizes they accept.
+over the paged cache); they differ in speed and in which sizes they accept.  In bfloat16 with a
+head size the matrix-core module takes, requests that bring at least TILE_MIN rows go to the
+tile kernel and all other rows (decode tokens, short portions) to the row kernel; everything
+else (float32, other head sizes) goes to the plain kernel.
 """
 from __future__ import annotations
 
 from typing import Optional
 
+import numpy as np
 import torch
 
 from . import ops
 
+TILE_MIN = 16       # fewer rows than this are cheaper one by one
+TILE_ROWS = 64      # rows per tile of the tile kernel
+ROW_CHUNK = 128     # keys per split of the row kernel ...
+ROW_MAX_SPLITS = 64  # ... doubled until a row has at most this many splits
+
+
+def _work_lists(ctx):
+    """What the kernels need beyond the step's own arrays, computed once per step."""
+    q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
+    tiled = q_len >= TILE_MIN
+    tile_req, tile_q0 = [], []
+    for r in np.nonzero(tiled)[0]:
+        for q0 in range(0, int(q_len[r]), TILE_ROWS):
+            tile_req.append(r); tile_q0.append(q0)
+    row_mask = ~tiled[ctx.h_row_req] if ctx.n_tokens else np.zeros(0, bool)
+    rows = np.nonzero(row_mask)[0].astype(np.int32)
+    out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1}
+    if tile_req:
+        out["tile_req"] = ctx.upload(np.asarray(tile_req, np.int32))
+        out["tile_q0"] = ctx.upload(np.asarray(tile_q0, np.int32))
+    if rows.size:
+        if rows.size != ctx.n_tokens:
+            out["rows"] = ctx.upload(rows)
+        max_kv = int(kv_len[~tiled].max())
+        chunk = ROW_CHUNK
+        while -(-max_kv // chunk) > ROW_MAX_SPLITS:
+            chunk *= 2
+        out["chunk"], out["max_splits"] = chunk, -(-max_kv // chunk)
+    return out
+
 
 def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: float) -> torch.Tensor:
     """q [T, nH, d] of this step's rows against ``cache`` (a LayerCache); returns [T, nH*d]."""
-    return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, ctx.block_table(cache.group),
-                               window, scale)
+    T, nH, d = q.shape
+    table = ctx.block_table(cache.group)
+    if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
+        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
+    w = ctx.derived("attention_work_lists", lambda: _work_lists(ctx))
+    out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
+    if w["n_tiles"]:
+        ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
+                            table, window, scale)
+    if w["n_rows"]:
+        ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
+                           window, scale, w["chunk"], w["max_splits"])
+    return out

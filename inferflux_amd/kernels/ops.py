@@ -24,6 +24,11 @@ _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
 
 ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
 
+# The matrix-core attention module is compiled per head size, when a model with that head size
+# first runs; these sizes are compiled ahead by build_all().
+MFMA_HEAD_DIMS_PREBUILT = (16, 32, 64, 128)
+MFMA_MAX_HEAD_DIM = 128
+
 
 class KernelError(RuntimeError):
     pass
@@ -34,6 +39,8 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("gemm_f32", ())
     yield ("attn_plain", ())
     yield ("sampling", ())
+    for d in MFMA_HEAD_DIMS_PREBUILT:
+        yield ("attn_mfma", (("HEAD_DIM", d),))
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -219,6 +226,65 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, page_size,
           int(window or 0), float(scale), _stream())
     return out
+
+
+def mfma_attention_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= MFMA_MAX_HEAD_DIM and page_size % 16 == 0
+
+
+def _attn_common(q, k_cache, v_cache):
+    _check(q, "q", (None, None, None), torch.bfloat16)
+    T, nH, d = q.shape
+    _check(k_cache, "k_cache", (None, None, None, d), torch.bfloat16)
+    n_pages, nKV, page_size, _ = k_cache.shape
+    _check(v_cache, "v_cache", (n_pages, nKV, d, page_size), torch.bfloat16)
+    if not mfma_attention_supported(q.dtype, d, page_size):
+        raise KernelError(f"matrix-core attention needs bfloat16, head_dim a multiple of 16 up to {MFMA_MAX_HEAD_DIM} and "
+                          f"page_size a multiple of 16; got head_dim {d}, page_size {page_size}")
+    return T, nH, d, nKV, page_size, load_module("attn_mfma", (("HEAD_DIM", d),))
+
+
+def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                   rows: Optional[torch.Tensor], n_rows: int, row_req: torch.Tensor, positions: torch.Tensor,
+                   block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int) -> None:
+    """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].
+    Split s of a row covers key positions [s*chunk, (s+1)*chunk); ``max_splits`` * chunk must reach
+    past the largest position among the rows."""
+    T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache)
+    _check(out, "out", (T, nH * d), torch.bfloat16)
+    _check(row_req, "row_req", (T,), torch.int32)
+    _check(positions, "positions", (T,), torch.int32)
+    _check(block_table, "block_table", (None, None), torch.int32)
+    if rows is not None:
+        _check(rows, "rows", (n_rows,), torch.int32)
+    elif n_rows != T:
+        raise KernelError("attention_rows: without a row list every row of the batch is handled")
+    part_o = torch.empty((n_rows, nH, max_splits, d), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
+    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, P),
+          q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(rows), row_req.data_ptr(),
+          positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_rows, nH, nKV, d, page_size,
+          int(window or 0), chunk, max_splits, float(scale), part_o.data_ptr(), part_ml.data_ptr(), _stream())
+
+
+def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                    tile_req: torch.Tensor, tile_q0: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                    kv_len: torch.Tensor, block_table: torch.Tensor, window: Optional[int], scale: float) -> None:
+    """Attention of tiles of 64 consecutive rows of one request each (tile t: request tile_req[t], rows
+    from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d]."""
+    T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache)
+    _check(out, "out", (T, nH * d), torch.bfloat16)
+    n_tiles = tile_req.shape[0]
+    _check(tile_req, "tile_req", (n_tiles,), torch.int32)
+    _check(tile_q0, "tile_q0", (n_tiles,), torch.int32)
+    R = q_start.shape[0]
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (kv_len, "kv_len")):
+        _check(t, nm, (R,), torch.int32)
+    _check(block_table, "block_table", (R, None), torch.int32)
+    _call(mod, "ifx_attn_tiles", (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, P),
+          q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
+          n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
+          block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), _stream())
 
 
 # ----------------------------------------------------------------------------------------

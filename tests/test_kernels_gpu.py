@@ -280,3 +280,67 @@ def test_sample_histogram_follows_the_probabilities():
     p = torch.softmax(logits.double(), -1)
     chi2 = float((N * (freq - p) ** 2 / p).sum())
     assert chi2 < 100.0, chi2                            # 49 degrees of freedom: 100 is far in the tail
+
+
+# ---- matrix-core attention --------------------------------------------------------------------
+MFMA_CASES = [c for c in ATTN_CASES if c[4] % 16 == 0 and c[4] <= 128] + [
+    ([100, 64, 17], [0, 100, 300], 4, 2, 16, 16, None, None),      # tiles that end inside a page, head size 16
+    ([130], [61], 8, 2, 48, 16, None, 5),                          # head size 48 (half-empty last step), planted key
+    ([70, 1], [200, 1000], 28, 4, 128, 16, None, None),            # 7B head layout
+    ([64, 64], [0, 192], 3, 3, 64, 32, 40, None),                  # window across tiles, pages of 32
+    ([33], [90], 40, 2, 32, 16, None, 64),                         # 20 query heads per kv head: two passes of 16
+]
+
+
+def run_rows(q, kc, vc, row_req, positions, table, window, scale, rows=None, chunk=128):
+    T, nH, d = q.shape
+    out = torch.zeros(T, nH * d, dtype=q.dtype, device=DEV)
+    n = T if rows is None else rows.shape[0]
+    max_kv = int(positions.max()) + 1
+    ops.attention_rows(q, kc, vc, out, rows, n, row_req, positions, table, window, scale, chunk, -(-max_kv // chunk))
+    return out
+
+
+@pytest.mark.parametrize("chunk", [32, 128])
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_attention_rows(case, chunk):
+    lens_q, lens_past, nH, nKV, d, P, window, sharp = case
+    (q, kc, vc, row_req, positions, table), want, _ = paged_case(7, lens_q, lens_past, nH, nKV, d, P, BF16, window, sharp=sharp)
+    out = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), chunk=chunk).cpu().double()
+    assert torch.isfinite(out).all()
+    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
+
+
+def test_attention_rows_subset_leaves_other_rows_alone():
+    (q, kc, vc, row_req, positions, table), want, _ = paged_case(8, [5, 1, 3], [10, 99, 40], 6, 2, 32, 16, BF16)
+    rows = torch.tensor([5, 0, 8], dtype=torch.int32, device=DEV)
+    out = run_rows(q, kc, vc, row_req, positions, table, None, 1.0 / math.sqrt(32), rows=rows).cpu().double()
+    assert torch.allclose(out[[5, 0, 8]], want[[5, 0, 8]], rtol=1e-2, atol=1e-2)
+    rest = [i for i in range(9) if i not in (5, 0, 8)]
+    assert torch.all(out[rest] == 0)
+
+
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_attention_tiles(case):
+    lens_q, lens_past, nH, nKV, d, P, window, sharp = case
+    (q, kc, vc, row_req, positions, table), want, info = paged_case(7, lens_q, lens_past, nH, nKV, d, P, BF16, window, sharp=sharp)
+    T = q.shape[0]
+    out = torch.zeros(T, nH * d, dtype=BF16, device=DEV)
+    q_len = torch.tensor(info["q_lens"], dtype=torch.int32)
+    q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
+    tiles = [(r, q0) for r, n in enumerate(info["q_lens"]) for q0 in range(0, n, 64)]
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ops.attention_tiles(q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV),
+                        q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d))
+    out = out.cpu().double()
+    assert torch.isfinite(out).all()
+    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
+
+
+def test_mfma_attention_refuses_what_it_cannot_do():
+    q = torch.zeros(1, 2, 24, dtype=BF16, device=DEV)
+    kc = torch.zeros(2, 1, 16, 24, dtype=BF16, device=DEV)
+    vc = torch.zeros(2, 1, 24, 16, dtype=BF16, device=DEV)
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(ops.KernelError, match="head_dim"):
+        ops.attention_rows(q, kc, vc, torch.zeros(1, 48, dtype=BF16, device=DEV), None, 1, z, z, z.view(1, 1), None, 1.0, 128, 1)
