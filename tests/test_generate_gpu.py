@@ -1,0 +1,119 @@
+"""Generation through the entry points: greedy tokens against the plain implementation, sampling
+with a seed against the plain rule, preemption by recomputation, and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+from conftest import ROOT, TINY, seeded_ids
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    from inferflux_amd import Engine, SamplingParams
+    from inferflux_amd.sampling.params import philox_uniform
+
+# BASELINE workloads of the tiny configurations: prompts of 7/13/29 tokens with 16 greedy tokens
+# each (A); prompts of 1/17/64/100/250 with 24 tokens, prefill portions of 32, pages of 16 (B).
+WORKLOADS = {"A": ([7, 13, 29], 16, 512), "B": ([1, 17, 64, 100, 250], 24, 32), "C": ([40, 3, 90], 20, 16)}
+
+
+def plain_greedy(folder, prompt, n):
+    cfg, W = pm.load_folder(folder, torch.float64)
+    return pm.greedy_generate(cfg, W, prompt, n)
+
+
+@pytest.mark.parametrize("name", list(TINY))
+def test_greedy_generation_equals_the_plain_model(name, model_folders):
+    folder = model_folders[name]
+    lens, n_new, chunk = WORKLOADS[name]
+    prompts = [seeded_ids(50 + i, n, TINY[name]["vocab_size"]) for i, n in enumerate(lens)]
+    engine = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=8, chunked_prefill_tokens=chunk)
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o.finish_reason == "length" and o.token_ids == plain_greedy(folder, p, n_new)
+    assert engine.runner.manager.free_pages() == [64] * len(engine.runner.manager.groups)
+    st = engine.stats
+    assert st.generated_tokens == n_new * len(prompts) and st.prompt_tokens == sum(lens)
+
+
+def test_preemption_by_recomputation_changes_no_token(model_folders):
+    folder = model_folders["A"]
+    prompts = [seeded_ids(70 + i, 40, 512) for i in range(3)]
+    sp = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    roomy = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=4)
+    want = [o.token_ids for o in roomy.generate(prompts, sp)]
+    tight = Engine.load(folder, dtype="float32", kv_pages=8, max_batch_size=4)     # 15 pages would be needed
+    outs = tight.generate(prompts, sp)
+    assert [o.token_ids for o in outs] == want
+    assert tight.stats.preemptions >= 1 and outs[0].preemptions == 0
+    tight.runner.manager.check()
+    assert tight.runner.manager.free_pages() == [8]
+
+
+def test_seeded_sampling_follows_the_plain_rule_and_ignores_batch_composition(model_folders):
+    folder = model_folders["B"]
+    cfg, W = pm.load_folder(folder, torch.float64)
+    prompts = [seeded_ids(80 + i, n, 1000) for i, n in enumerate((5, 33, 12))]
+    params = [SamplingParams(temperature=0.8, seed=11, max_tokens=24, ignore_eos=True),
+              SamplingParams(temperature=1.0, top_p=0.9, top_k=50, seed=12, max_tokens=24, ignore_eos=True),
+              SamplingParams(temperature=1.2, min_p=0.001, repetition_penalty=1.3, frequency_penalty=0.1,
+                             presence_penalty=0.2, seed=13, max_tokens=24, ignore_eos=True)]
+    engine = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=4, chunked_prefill_tokens=32)
+    together = [o.token_ids for o in engine.generate(prompts, params)]
+    alone = [engine.generate([p], [sp])[0].token_ids for p, sp in zip(prompts, params)]
+    assert together == alone                                  # (seed, step) alone decides the draw
+    assert len({tuple(t) for t in together}) == 3
+    for prompt, sp, toks in zip(prompts, params, together):
+        hist = []
+        for step, tok in enumerate(toks):
+            logits = pm.forward(cfg, W, prompt + toks[:step])[-1]
+            logits = pm.apply_penalties(logits, hist[-sp.penalty_last_n:], sp.repetition_penalty, sp.frequency_penalty, sp.presence_penalty)
+            w = pm.filtered_probs(logits, sp.temperature, sp.top_k, sp.top_p, sp.min_p)
+            u = float(philox_uniform(np.array([sp.seed]), np.array([step]))[0])
+            want = pm.cdf_walk(w, u)
+            if tok != want:                                   # only a draw on the edge between two tokens may differ
+                cum = torch.cumsum(w, 0) / w.sum()
+                assert abs(tok - want) >= 1 and min(abs(float(cum[min(tok, want)]) - u), abs(float(cum[max(tok, want) - 1]) - u)) < 1e-4
+                break
+            hist.append(tok)
+
+
+def test_stop_tokens_and_eos(model_folders, tmp_path):
+    import shutil
+    folder = str(tmp_path / "eos")
+    shutil.copytree(model_folders["A"], folder)
+    prompt = seeded_ids(90, 9, 512)
+    free_run = plain_greedy(folder, prompt, 12)
+    cfg = json.load(open(os.path.join(folder, "config.json")))
+    cfg["eos_token_id"] = free_run[5]
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    engine = Engine.load(folder, dtype="float32", kv_pages=16)
+    first = free_run.index(free_run[5])
+    out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12))[0]
+    assert out.finish_reason == "stop" and out.token_ids == free_run[: first + 1]
+    out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))[0]
+    assert out.finish_reason == "length" and out.token_ids == free_run
+    stop = free_run[2]
+    out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True, stop_token_ids=(stop,)))[0]
+    assert out.finish_reason == "stop" and out.token_ids == free_run[: free_run.index(stop) + 1]
+
+
+def test_command_line(model_folders):
+    folder = model_folders["A"]
+    prompt = seeded_ids(95, 11, 512)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "inferctl"), "completion", "--model", folder,
+                           "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "8", "--temperature", "0",
+                           "--dtype", "float32", "--ignore-eos", "--stream", "--ctx-size", "256", "--max-parallel-sequences", "2"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    want = plain_greedy(folder, prompt, 8)
+    assert [l["token"] for l in lines if "token" in l] == want           # streamed one by one
+    final = [l for l in lines if "token_ids" in l][0]
+    assert final["token_ids"] == want and final["finish_reason"] == "length" and final["prompt_tokens"] == 11
