@@ -92,6 +92,77 @@ struct RowArgs {
   float scale_log2e;
 };
 
+// The operands of one block of 32 keys (two pages' worth of 16): loaded together, K and V at once,
+// so that a block costs one trip to memory, and one block ahead of the arithmetic.
+struct RowBlock {
+  bf16x8 k[2][KS];
+  bf16x4 v[DT][2];
+  bool live[2];
+};
+
+__device__ __forceinline__ void load_row_block(RowBlock& b, const RowArgs& a, const int* table, int kvh, int j0,
+                                               int ka, int kb, int col, int g4) {
+  const int P = a.P;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int k0 = j0 + 16 * t;  // 16 keys k0..k0+15, all in one page
+    bool live = k0 < kb && k0 + 16 > ka;
+    const int page = live ? table[k0 / P] : -1;
+    live = live && page >= 0;
+    b.live[t] = live;
+    const int off = k0 % P;
+    const bf16_t* kp = a.k_cache + (((size_t)(live ? page : 0) * a.nKV + kvh) * P + off + col) * D + 8 * g4;
+    const bf16_t* vp = a.v_cache + (((size_t)(live ? page : 0) * a.nKV + kvh) * D + col) * P + off + 4 * g4;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      b.k[t][ks] = (live && 32 * ks + 8 * g4 < D) ? *(const bf16x8*)(kp + 32 * ks) : zero8();
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      b.v[dt][t] = live ? *(const bf16x4*)(vp + (size_t)16 * dt * P) : zero4();
+  }
+}
+
+__device__ __forceinline__ void use_row_block(const RowBlock& b, const RowArgs& a, const bf16x8* qop, floatx4* o, float& m,
+                                              float& l, int j0, int ka, int kb, int g4) {
+  floatx4 s[2];
+  float mb = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[t][ks], qop[ks], s[t], 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = j0 + 16 * t + 4 * g4 + r;
+      const bool vis = b.live[t] && key >= ka && key < kb;
+      s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
+      mb = fmaxf(mb, s[t][r]);
+    }
+  }
+  const float m_new = fmaxf(m, col_max(mb));
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = exp2f(m - m_safe);
+  float psum = 0.f;
+  bf16x4 pb[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float p = exp2f(s[t][r] - m_safe);
+      psum += p;
+      pb[t][r] = (__bf16)p;
+    }
+  l = l * alpha + psum;
+  m = m_new;
+  const bf16x8 pop = join4(pb[0], pb[1]);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join4(b.v[dt][0], b.v[dt][1]), pop, o[dt], 0, 0, 0);
+  }
+}
+
 __global__ __launch_bounds__(WAVE) void attn_rows_kernel(RowArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, ri = blockIdx.z;
   const int lane = threadIdx.x, col = lane & 15, g4 = lane >> 4;
@@ -100,7 +171,6 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(RowArgs a) {
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int ka = max(lo, split * a.chunk), kb = min(pos + 1, (split + 1) * a.chunk);  // keys [ka, kb)
   const int ratio = a.nH / a.nKV;
-  const int P = a.P;
   const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
 
   for (int qt = 0; qt < ratio; qt += 16) {
@@ -123,61 +193,16 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(RowArgs a) {
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int j0 = (ka / 32) * 32; j0 < kb; j0 += 32) {
-      floatx4 s[2];
-      int page[2], off[2];
-      bool live[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int k0 = j0 + 16 * t;  // 16 keys k0..k0+15, all in one page
-        live[t] = k0 < kb && k0 + 16 > ka;
-        page[t] = live[t] ? table[k0 / P] : -1;
-        off[t] = k0 % P;
-        live[t] = live[t] && page[t] >= 0;
-        s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-        if (live[t]) {
-          const bf16_t* kp = a.k_cache + (((size_t)page[t] * a.nKV + kvh) * P + off[t] + col) * D + 8 * g4;
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) {
-            const bf16x8 kop = (32 * ks + 8 * g4 < D) ? *(const bf16x8*)(kp + 32 * ks) : zero8();
-            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[ks], s[t], 0, 0, 0);
-          }
-        }
-      }
-      float mb = -INFINITY;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int key = j0 + 16 * t + 4 * g4 + r;
-          const bool vis = live[t] && key >= ka && key < kb;
-          s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
-          mb = fmaxf(mb, s[t][r]);
-        }
-      const float m_new = fmaxf(m, col_max(mb));
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = exp2f(m - m_safe);
-      float psum = 0.f;
-      bf16x4 pb[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float p = exp2f(s[t][r] - m_safe);
-          psum += p;
-          pb[t][r] = (__bf16)p;
-        }
-      l = l * alpha + psum;
-      m = m_new;
-      const bf16x8 pop = join4(pb[0], pb[1]);
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        bf16x4 v0 = zero4(), v1 = zero4();
-        if (live[0]) v0 = *(const bf16x4*)(a.v_cache + (((size_t)page[0] * a.nKV + kvh) * D + 16 * dt + col) * P + off[0] + 4 * g4);
-        if (live[1]) v1 = *(const bf16x4*)(a.v_cache + (((size_t)page[1] * a.nKV + kvh) * D + 16 * dt + col) * P + off[1] + 4 * g4);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join4(v0, v1), pop, o[dt], 0, 0, 0);
+    RowBlock b0, b1;
+    int j0 = (ka / 32) * 32;
+    load_row_block(b0, a, table, kvh, j0, ka, kb, col, g4);
+    for (; j0 < kb; j0 += 64) {
+      const bool more1 = j0 + 32 < kb, more2 = j0 + 64 < kb;
+      if (more1) load_row_block(b1, a, table, kvh, j0 + 32, ka, kb, col, g4);
+      use_row_block(b0, a, qop, o, m, l, j0, ka, kb, g4);
+      if (more1) {
+        if (more2) load_row_block(b0, a, table, kvh, j0 + 64, ka, kb, col, g4);
+        use_row_block(b1, a, qop, o, m, l, j0 + 32, ka, kb, g4);
       }
     }
     l = col_sum(l);
@@ -189,27 +214,54 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(RowArgs a) {
   }
 }
 
-// out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s
-__global__ void attn_rows_merge_kernel(RowArgs a) {
-  const int ri = blockIdx.x, head = blockIdx.y;
+// out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s.
+// One wave per (row, head): lane s first weighs split s, then every lane sums its elements over
+// the splits in ascending order.
+__global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
+  __shared__ float w_s[WAVE];
+  const int ri = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int row = a.rows ? a.rows[ri] : ri;
   const int pos = a.positions[row];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int s0 = lo / a.chunk, s1 = pos / a.chunk;  // first and last split that hold a visible key
   const float* po = a.part_o + ((size_t)ri * a.nH + head) * a.max_splits * D;
   const float* pml = a.part_ml + ((size_t)ri * a.nH + head) * a.max_splits * 2;
+  float acc[(D + WAVE - 1) / WAVE];
+#pragma unroll
+  for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = 0.f;
+  float L = 0.f;
+  // The launcher bounds the splits of a row by 64 per round; rounds handle longer rows.
   float M = -INFINITY;
-  for (int s = s0; s <= s1; ++s) M = fmaxf(M, pml[2 * s]);
-  for (int e = threadIdx.x; e < D; e += blockDim.x) {
-    float L = 0.f, acc = 0.f;
-    for (int s = s0; s <= s1; ++s) {
-      const float ms = pml[2 * s];
-      if (ms == -INFINITY) continue;
-      const float w = exp2f(ms - M);
-      L += w * pml[2 * s + 1];
-      acc += w * po[(size_t)s * D + e];
+  for (int sb = s0; sb <= s1; sb += WAVE) {
+    const int s = sb + lane;
+    M = fmaxf(M, s <= s1 ? pml[2 * s] : -INFINITY);
+  }
+  M = wave_max(M);
+  for (int sb = s0; sb <= s1; sb += WAVE) {
+    const int s = sb + lane;
+    const float ms = s <= s1 ? pml[2 * s] : -INFINITY;
+    const float w = ms == -INFINITY ? 0.f : exp2f(ms - M);
+    L += s <= s1 ? w * pml[2 * s + 1] : 0.f;
+    __syncthreads();
+    w_s[lane] = w;
+    __syncthreads();
+    const int n = min(WAVE, s1 - sb + 1);
+    for (int i = 0; i < n; ++i) {
+      const float wi = w_s[i];
+      if (wi == 0.f) continue;
+#pragma unroll
+      for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
+        const int e = lane + c * WAVE;
+        if (e < D) acc[c] = fmaf(wi, po[(size_t)(sb + i) * D + e], acc[c]);
+      }
     }
-    a.out[((size_t)row * a.nH + head) * D + e] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+  }
+  L = wave_sum(L);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+#pragma unroll
+  for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
+    const int e = lane + c * WAVE;
+    if (e < D) a.out[((size_t)row * a.nH + head) * D + e] = (bf16_t)(acc[c] * inv);
   }
 }
 
@@ -228,7 +280,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
             scale * 1.4426950408889634f};
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(attn_rows_kernel, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
-  hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(D >= 128 ? 128 : 64), 0, s, a);
+  hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, a);
   IFX_LAUNCH_CHECK();
 }
 

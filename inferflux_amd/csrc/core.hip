@@ -71,6 +71,89 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   }
 }
 
+// The same, for H a multiple of 4 up to 4 * 256 * NV: each thread keeps its elements in registers,
+// so the row is read once, in 16-byte pieces.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float4 type; };
+template <> struct Vec4<bf16_t> { typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 type; };
+
+template <typename T> __device__ __forceinline__ void load4(const T* p, float* v);
+template <> __device__ __forceinline__ void load4<float>(const float* p, float* v) {
+  const float4 t = *(const float4*)p; v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <> __device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float* v) {
+  const typename Vec4<bf16_t>::type t = *(const typename Vec4<bf16_t>::type*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = (float)t[i];
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, const float* v);
+template <> __device__ __forceinline__ void store4<float>(float* p, const float* v) {
+  *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float* v) {
+  typename Vec4<bf16_t>::type t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) t[i] = (__bf16)v[i];
+  *(typename Vec4<bf16_t>::type*)p = t;
+}
+
+template <typename TD, typename TO, typename TW, int NV>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                                              const TW* __restrict__ weight, TO* __restrict__ out,
+                                                              const int* __restrict__ rows, int H, float eps, int write_back) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* res = residual + src * H;
+  const TD* dl = delta ? delta + src * H : nullptr;
+  float x[NV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int i = 4 * (threadIdx.x + 256 * v);
+    if (i < H) {
+      load4<float>(res + i, x[v]);
+      if (dl) {
+        float d4[4];
+        load4<TD>(dl + i, d4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[v][e] += d4[e];
+        if (write_back) store4<float>(res + i, x[v]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += x[v][e] * x[v][e];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rms = rsqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)r * H;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int i = 4 * (threadIdx.x + 256 * v);
+    if (i < H) {
+      float w4[4], y[4];
+      load4<TW>(weight + i, w4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = x[v][e] * rms * w4[e];
+      store4<TO>(o + i, y);
+    }
+  }
+}
+
+template <typename TD, typename TO, typename TW>
+static void launch_rmsnorm_vec(float* residual, const void* delta, const void* weight, void* out, const int* rows,
+                               int n_rows, int H, float eps, int write_back, hipStream_t s) {
+  if (H <= 4 * 256 * 2)
+    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 2>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
+                       (const TW*)weight, (TO*)out, rows, H, eps, write_back);
+  else if (H <= 4 * 256 * 4)
+    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 4>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
+                       (const TW*)weight, (TO*)out, rows, H, eps, write_back);
+  else
+    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 8>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
+                       (const TW*)weight, (TO*)out, rows, H, eps, write_back);
+}
+
 extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* weight,
                                int weight_dtype, void* out, int out_dtype, const int* rows, int n_rows,
                                int H, float eps, int write_back, void* stream) {
@@ -78,16 +161,31 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
   IFX_REQUIRE(!(rows && write_back), "add_rmsnorm: a row gather cannot write the residual back");
   if (n_rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const int dd = delta ? delta_dtype : out_dtype;
+  IFX_REQUIRE((dd == DT_F32 || dd == DT_BF16) && (out_dtype == DT_F32 || out_dtype == DT_BF16) &&
+              (weight_dtype == DT_F32 || weight_dtype == DT_BF16),
+              "add_rmsnorm: unknown dtypes delta=%d out=%d weight=%d", delta_dtype, out_dtype, weight_dtype);
+  if (H % 4 == 0 && H <= 4 * 256 * 8) {
+#define VEC(TD, TO)                                                                                                  \
+  do {                                                                                                               \
+    if (weight_dtype == DT_F32) launch_rmsnorm_vec<TD, TO, float>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, s); \
+    else launch_rmsnorm_vec<TD, TO, bf16_t>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, s);      \
+  } while (0)
+    if (dd == DT_F32 && out_dtype == DT_F32) VEC(float, float);
+    else if (dd == DT_BF16 && out_dtype == DT_BF16) VEC(bf16_t, bf16_t);
+    else if (dd == DT_F32 && out_dtype == DT_BF16) VEC(float, bf16_t);
+    else VEC(bf16_t, float);
+#undef VEC
+    IFX_LAUNCH_CHECK();
+  }
   const int threads = H >= 2048 ? 512 : 256;
 #define LAUNCH(TD, TO)                                                                              \
   hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(threads), 0, s, residual,     \
                      (const TD*)delta, weight, weight_dtype, (TO*)out, rows, H, eps, write_back)
-  const int dd = delta ? delta_dtype : out_dtype;
   if (dd == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
   else if (dd == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
   else if (dd == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
-  else if (dd == DT_BF16 && out_dtype == DT_F32) LAUNCH(bf16_t, float);
-  else IFX_FAIL("add_rmsnorm: unknown dtypes delta=%d out=%d", delta_dtype, out_dtype);
+  else LAUNCH(bf16_t, float);
 #undef LAUNCH
   IFX_LAUNCH_CHECK();
 }
@@ -114,10 +212,13 @@ struct RopeArgs {
   void* v_cache;
 };
 
+#define ROPE_MAX_PAIRS 128  // rotary_dim / 2 up to this is tabulated per token in LDS
+
 template <typename T>
-__global__ void rope_append_kernel(RopeArgs a) {
+__global__ __launch_bounds__(256) void rope_append_kernel(RopeArgs a) {
+  __shared__ float cs_s[ROPE_MAX_PAIRS], sn_s[ROPE_MAX_PAIRS];
   const int t = blockIdx.x;
-  const int d = a.d, half = d / 2, rot_half = a.rotary_dim / 2;
+  const int d = a.d, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
   const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
   const float pos = (float)a.positions[t];
@@ -125,18 +226,22 @@ __global__ void rope_append_kernel(RopeArgs a) {
   const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
   T* qo = (T*)a.q_out + (size_t)t * q_width;
 
+  // the token's angles, once for all heads
+  for (int p = threadIdx.x; p < rot_half; p += blockDim.x) sincosf(pos * a.inv_freq[p], &sn_s[p], &cs_s[p]);
+  __syncthreads();
+
   const int n_rot_items = (a.nH + a.nKV) * half;
   for (int it = threadIdx.x; it < n_rot_items; it += blockDim.x) {
     const int head = it / half, p = it % half;
     const bool is_q = head < a.nH;
     if (!is_q && slot < 0) continue;
     int i0, i1;
-    bool rotate = a.rope_style != 0 && p < rot_half;
+    const bool rotate = p < rot_half;
     if (rotate) {
       if (a.rope_style == 1) { i0 = p; i1 = p + rot_half; }
       else { i0 = 2 * p; i1 = 2 * p + 1; }
     } else {
-      const int base = a.rope_style != 0 ? a.rotary_dim + 2 * (p - rot_half) : 2 * p;
+      const int base = 2 * rot_half + 2 * (p - rot_half);
       i0 = base; i1 = base + 1;
     }
     const int col = head * d;  // q heads first, then k heads: the same offset rule
@@ -147,8 +252,7 @@ __global__ void rope_append_kernel(RopeArgs a) {
     }
     float y0 = x0, y1 = x1;
     if (rotate) {
-      float sn, cs;
-      sincosf(pos * a.inv_freq[p], &sn, &cs);
+      const float cs = cs_s[p], sn = sn_s[p];
       y0 = x0 * cs - x1 * sn;
       y1 = x0 * sn + x1 * cs;
     }
@@ -183,6 +287,7 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   IFX_REQUIRE(rope_style == 0 || (rotary_dim > 0 && rotary_dim <= d && rotary_dim % 2 == 0 && inv_freq),
               "rope_append: rotary_dim %d must be even, within head_dim %d, with a frequency table", rotary_dim, d);
   IFX_REQUIRE(!slots || (page_size > 0 && k_cache && v_cache), "rope_append: cache write without cache");
+  IFX_REQUIRE(rope_style == 0 || rotary_dim / 2 <= ROPE_MAX_PAIRS, "rope_append: rotary_dim %d above %d", rotary_dim, 2 * ROPE_MAX_PAIRS);
   if (T == 0) return 0;
   RopeArgs a{qkv, bias, bias_dtype, positions, slots, inv_freq, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
   hipStream_t s = (hipStream_t)stream;

@@ -39,6 +39,7 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("gemm_f32", ())
     yield ("attn_plain", ())
     yield ("sampling", ())
+    yield ("gemm_bf16", ())
     for d in MFMA_HEAD_DIMS_PREBUILT:
         yield ("attn_mfma", (("HEAD_DIM", d),))
 
@@ -187,13 +188,33 @@ def gemm_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
     return out
 
 
+SKINNY_MAX_M = 64
+
+
+def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                nt: int = 0, waves: int = 0, unroll: int = 0) -> torch.Tensor:
+    """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
+    accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose."""
+    _check(x, "x", (None, None), torch.bfloat16)
+    M, K = x.shape
+    _check(weight, "weight", (None, K), torch.bfloat16)
+    N = weight.shape[0]
+    if M > SKINNY_MAX_M or K % 8:
+        raise KernelError(f"skinny_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, P),
+          x.data_ptr(), weight.data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves, unroll, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """x [M, K] times ``weight`` [N, K] transposed, chosen by the weight's type.
+    """x [M, K] times ``weight`` [N, K] transposed, chosen by the weight's type and by M.
 
     A float32 weight takes the true 32-bit kernel whatever the activation's type.  A bfloat16
-    weight with bfloat16 activations takes the library product with float accumulation, as
-    the reference does for every dense projection
-    (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).
+    weight with bfloat16 activations takes the weight-streaming kernel for up to 64 rows and the
+    library product with float accumulation beyond, as the reference does for every dense
+    projection (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).  float32 output (logits)
+    always comes from float accumulators, never through a bfloat16 rounding.
     """
     if weight.dtype == torch.float32:
         return gemm_f32(x, weight, None, out_dtype or x.dtype)
@@ -201,10 +222,16 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
         raise KernelError(f"linear: weight {weight.dtype} with activation {x.dtype} is not supported")
     _check(x, "x", (None, weight.shape[1]))
     _check(weight, "weight", (None, None))
-    out = torch.matmul(x, weight.t())
-    if out_dtype is not None and out_dtype != out.dtype:
-        out = cast(out, out_dtype)
-    return out
+    out_dtype = out_dtype or torch.bfloat16
+    M, K = x.shape
+    N = weight.shape[0]
+    # Measured on the 7B shapes: the streaming kernel wins up to 16 rows everywhere and up to 32 rows
+    # on the narrow products; beyond that the library's tiles reuse the rows better.
+    if K % 8 == 0 and (M <= 16 or (M <= 32 and N <= 4096)):
+        return skinny_gemm(x, weight, out_dtype)
+    if out_dtype == torch.float32:
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+    return torch.matmul(x, weight.t())
 
 
 # ----------------------------------------------------------------------------------------

@@ -344,3 +344,41 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     z = torch.zeros(1, dtype=torch.int32, device=DEV)
     with pytest.raises(ops.KernelError, match="head_dim"):
         ops.attention_rows(q, kc, vc, torch.zeros(1, 48, dtype=BF16, device=DEV), None, 1, z, z, z.view(1, 1), None, 1.0, 128, 1)
+
+
+# ---- weight-streaming matrix product ---------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(50, 64), (3, 8), (130, 200), (577, 1000), (4608, 3584)])
+@pytest.mark.parametrize("out_dtype", [BF16, F32])
+def test_skinny_gemm(M, N, K, out_dtype):
+    g = gen(11)
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = torch.randn(N, K, generator=g).to(BF16)
+    want = x.double() @ w.double().t()
+    out = ops.skinny_gemm(x.to(DEV), w.to(DEV), out_dtype).cpu().double()
+    t = dict(rtol=1e-2, atol=1e-2 * math.sqrt(K)) if out_dtype == BF16 else dict(rtol=1e-4, atol=1e-4 * math.sqrt(K))
+    assert torch.allclose(out, want, **t), float((out - want).abs().max())
+
+
+@pytest.mark.parametrize("nt,waves,unroll", [(1, 1, 4), (2, 4, 2), (1, 16, 2), (2, 8, 4), (1, 3, 8)])
+def test_skinny_gemm_every_launch_shape_gives_the_same_product(nt, waves, unroll):
+    g = gen(12)
+    x = torch.randn(9, 1096, generator=g).to(BF16)
+    w = torch.randn(333, 1096, generator=g).to(BF16)
+    want = x.double() @ w.double().t()
+    out = ops.skinny_gemm(x.to(DEV), w.to(DEV), F32, nt=nt, waves=waves, unroll=unroll).cpu().double()
+    assert torch.allclose(out, want, rtol=1e-4, atol=3e-3)
+
+
+def test_linear_picks_by_weight_type_and_rows():
+    g = gen(13)
+    w = torch.randn(96, 72, generator=g)
+    for M in (3, 64, 65, 200):
+        x = torch.randn(M, 72, generator=g)
+        want = x.bfloat16().double() @ w.bfloat16().double().t()
+        got = ops.linear(x.bfloat16().to(DEV), w.bfloat16().to(DEV))
+        assert got.dtype == BF16 and torch.allclose(got.cpu().double(), want, rtol=1e-2, atol=0.1)
+        logits = ops.linear(x.bfloat16().to(DEV), w.bfloat16().to(DEV), out_dtype=F32)
+        assert logits.dtype == F32 and torch.allclose(logits.cpu().double(), want, rtol=1e-4, atol=1e-3)   # no bf16 rounding
+        mixed = ops.linear(x.bfloat16().to(DEV), w.to(DEV))                  # a float32 weight in bf16 mode
+        assert mixed.dtype == BF16 and torch.allclose(mixed.cpu().double(), x.bfloat16().double() @ w.double().t(), rtol=1e-2, atol=0.1)
