@@ -246,14 +246,23 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
     w_s[lane] = w;
     __syncthreads();
     const int n = min(WAVE, s1 - sb + 1);
-    for (int i = 0; i < n; ++i) {
-      const float wi = w_s[i];
-      if (wi == 0.f) continue;
+    // four splits at a time, so that their loads are in flight together; an empty split (weight 0) is
+    // never read, its scratch may hold anything
+    for (int i = 0; i < n; i += 4) {
+      float wi[4], val[4][(D + WAVE - 1) / WAVE];
 #pragma unroll
-      for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
-        const int e = lane + c * WAVE;
-        if (e < D) acc[c] = fmaf(wi, po[(size_t)(sb + i) * D + e], acc[c]);
+      for (int u = 0; u < 4; ++u) {
+        wi[u] = i + u < n ? w_s[i + u] : 0.f;
+#pragma unroll
+        for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
+          const int e = lane + c * WAVE;
+          val[u][c] = (wi[u] != 0.f && e < D) ? po[(size_t)(sb + i + u) * D + e] : 0.f;
+        }
       }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = fmaf(wi[u], val[u][c], acc[c]);
     }
   }
   L = wave_sum(L);

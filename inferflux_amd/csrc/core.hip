@@ -191,19 +191,41 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
 }
 
 // ---------------------------------------------------------------------------------------
+// cos[t, p], sin[t, p] of angle = float(positions[t]) * inv_freq[p]: the step's rotation table, made
+// once per step and read by every layer.
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float* __restrict__ cs, float* __restrict__ sn, int n_pairs, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int t = i / n_pairs, p = i % n_pairs;
+  sincosf((float)positions[t] * inv_freq[p], &sn[i], &cs[i]);
+}
+
+extern "C" int ifx_rope_table(const int* positions, const float* inv_freq, float* cs, float* sn, int T, int n_pairs,
+                              void* stream) {
+  IFX_REQUIRE(T >= 0 && n_pairs > 0, "rope_table: bad sizes T=%d pairs=%d", T, n_pairs);
+  if (T == 0) return 0;
+  const int n = T * n_pairs;
+  hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, positions, inv_freq, cs, sn,
+                     n_pairs, n);
+  IFX_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
 // Per token t: qkv[t] = [q (nH*d) | k (nKV*d) | v (nKV*d)].  Adds the bias, rotates q and k by
 // the token's position, writes q to q_out[t] and k, v into the paged cache at slot[t]
 // (slot = page * page_size + offset; slot < 0: nothing is written to the cache).
 // Cache layouts: K [page][kv head][offset][d], V [page][kv head][d][offset].
 // rope_style: 0 none, 1 split-half pairs (p, p + rot/2), 2 consecutive pairs (2p, 2p+1);
-// angle = float(position) * inv_freq[p]; elements at or beyond rotary_dim are copied.
+// cos/sin come from the step's table [T, rotary_dim / 2]; elements at or beyond rotary_dim are
+// copied.  One block per (token, head): q heads, then k heads, then v heads.
 struct RopeArgs {
   const void* qkv;
   const void* bias;
   int bias_dtype;
-  const int* positions;
   const int* slots;
-  const float* inv_freq;
+  const float* cs;
+  const float* sn;
   int rope_style;
   int rotary_dim;
   int nH, nKV, d, page_size;
@@ -212,112 +234,96 @@ struct RopeArgs {
   void* v_cache;
 };
 
-#define ROPE_MAX_PAIRS 128  // rotary_dim / 2 up to this is tabulated per token in LDS
-
 template <typename T>
-__global__ __launch_bounds__(256) void rope_append_kernel(RopeArgs a) {
-  __shared__ float cs_s[ROPE_MAX_PAIRS], sn_s[ROPE_MAX_PAIRS];
-  const int t = blockIdx.x;
+__global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
+  const int t = blockIdx.x, head = blockIdx.y;
   const int d = a.d, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
   const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
-  const float pos = (float)a.positions[t];
   const int slot = a.slots ? a.slots[t] : -1;
   const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
-  T* qo = (T*)a.q_out + (size_t)t * q_width;
-
-  // the token's angles, once for all heads
-  for (int p = threadIdx.x; p < rot_half; p += blockDim.x) sincosf(pos * a.inv_freq[p], &sn_s[p], &cs_s[p]);
-  __syncthreads();
-
-  const int n_rot_items = (a.nH + a.nKV) * half;
-  for (int it = threadIdx.x; it < n_rot_items; it += blockDim.x) {
-    const int head = it / half, p = it % half;
+  const int col = head * d;  // q heads, k heads and v heads follow each other in the row
+  if (head < a.nH + a.nKV) {
     const bool is_q = head < a.nH;
-    if (!is_q && slot < 0) continue;
-    int i0, i1;
-    const bool rotate = p < rot_half;
-    if (rotate) {
-      if (a.rope_style == 1) { i0 = p; i1 = p + rot_half; }
-      else { i0 = 2 * p; i1 = 2 * p + 1; }
-    } else {
-      const int base = 2 * rot_half + 2 * (p - rot_half);
-      i0 = base; i1 = base + 1;
+    if (!is_q && slot < 0) return;
+    T* dst = is_q ? (T*)a.q_out + (size_t)t * q_width + col
+                  : (T*)a.k_cache + (((size_t)page * a.nKV + (head - a.nH)) * a.page_size + off) * d;
+    for (int p = threadIdx.x; p < half; p += blockDim.x) {
+      int i0, i1;
+      const bool rotate = p < rot_half;
+      if (rotate) {
+        if (a.rope_style == 1) { i0 = p; i1 = p + rot_half; }
+        else { i0 = 2 * p; i1 = 2 * p + 1; }
+      } else {
+        i0 = 2 * p; i1 = 2 * p + 1;  // beyond the rotated part pairs are consecutive in both styles
+      }
+      float x0 = to_f(row[col + i0]), x1 = to_f(row[col + i1]);
+      if (a.bias) {
+        x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
+        x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
+      }
+      float y0 = x0, y1 = x1;
+      if (rotate) {
+        const float cs = a.cs[(size_t)t * rot_half + p], sn = a.sn[(size_t)t * rot_half + p];
+        y0 = x0 * cs - x1 * sn;
+        y1 = x0 * sn + x1 * cs;
+      }
+      dst[i0] = from_f<T>(y0);
+      dst[i1] = from_f<T>(y1);
     }
-    const int col = head * d;  // q heads first, then k heads: the same offset rule
-    float x0 = to_f(row[col + i0]), x1 = to_f(row[col + i1]);
-    if (a.bias) {
-      x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
-      x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
-    }
-    float y0 = x0, y1 = x1;
-    if (rotate) {
-      const float cs = cs_s[p], sn = sn_s[p];
-      y0 = x0 * cs - x1 * sn;
-      y1 = x0 * sn + x1 * cs;
-    }
-    if (is_q) {
-      qo[col + i0] = from_f<T>(y0);
-      qo[col + i1] = from_f<T>(y1);
-    } else {
-      const int kh = head - a.nH;
-      T* kc = (T*)a.k_cache + (((size_t)page * a.nKV + kh) * a.page_size + off) * d;
-      kc[i0] = from_f<T>(y0);
-      kc[i1] = from_f<T>(y1);
-    }
-  }
-  if (slot >= 0) {
-    for (int it = threadIdx.x; it < kv_width; it += blockDim.x) {
-      const int kh = it / d, e = it % d;
-      const int col = q_width + kv_width + it;
-      float x = to_f(row[col]);
-      if (a.bias) x += load_dyn(a.bias, a.bias_dtype, col);
-      T* vc = (T*)a.v_cache + (((size_t)page * a.nKV + kh) * d + e) * a.page_size + off;
-      *vc = from_f<T>(x);
+  } else {
+    if (slot < 0) return;
+    const int kh = head - a.nH - a.nKV;
+    T* vc = (T*)a.v_cache + ((size_t)page * a.nKV + kh) * d * a.page_size + off;
+    for (int e = threadIdx.x; e < d; e += blockDim.x) {
+      float x = to_f(row[col + e]);
+      if (a.bias) x += load_dyn(a.bias, a.bias_dtype, col + e);
+      vc[(size_t)e * a.page_size] = from_f<T>(x);
     }
   }
 }
 
-extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype,
-                               const int* positions, const int* slots, const float* inv_freq,
-                               int rope_style, int rotary_dim, int T, int nH, int nKV, int d,
-                               int page_size, void* q_out, void* k_cache, void* v_cache, void* stream) {
+extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const int* slots,
+                               const float* cs, const float* sn, int rope_style, int rotary_dim, int T, int nH,
+                               int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, void* stream) {
   IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
   IFX_REQUIRE(rope_style >= 0 && rope_style <= 2, "rope_append: unknown rope style %d", rope_style);
-  IFX_REQUIRE(rope_style == 0 || (rotary_dim > 0 && rotary_dim <= d && rotary_dim % 2 == 0 && inv_freq),
-              "rope_append: rotary_dim %d must be even, within head_dim %d, with a frequency table", rotary_dim, d);
+  IFX_REQUIRE(rope_style == 0 || (rotary_dim > 0 && rotary_dim <= d && rotary_dim % 2 == 0 && cs && sn),
+              "rope_append: rotary_dim %d must be even, within head_dim %d, with a rotation table", rotary_dim, d);
   IFX_REQUIRE(!slots || (page_size > 0 && k_cache && v_cache), "rope_append: cache write without cache");
-  IFX_REQUIRE(rope_style == 0 || rotary_dim / 2 <= ROPE_MAX_PAIRS, "rope_append: rotary_dim %d above %d", rotary_dim, 2 * ROPE_MAX_PAIRS);
+  IFX_REQUIRE(nH + 2 * nKV <= 65535, "rope_append: too many heads for one launch");
   if (T == 0) return 0;
-  RopeArgs a{qkv, bias, bias_dtype, positions, slots, inv_freq, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
+  RopeArgs a{qkv, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DT_F32) hipLaunchKernelGGL(rope_append_kernel<float>, dim3(T), dim3(256), 0, s, a);
-  else if (dtype == DT_BF16) hipLaunchKernelGGL(rope_append_kernel<bf16_t>, dim3(T), dim3(256), 0, s, a);
+  const dim3 grid(T, nH + 2 * nKV);
+  if (dtype == DT_F32) hipLaunchKernelGGL(rope_append_kernel<float>, grid, dim3(64), 0, s, a);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(rope_append_kernel<bf16_t>, grid, dim3(64), 0, s, a);
   else IFX_FAIL("rope_append: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }
 
 // ---------------------------------------------------------------------------------------
-// gu[t] = [gate (I) | up (I)];  out[t, i] = gate / (1 + exp(-gate)) * up
+// out[t, i] = gate / (1 + exp(-gate)) * up, with gu[t] = [gate (I) | up (I)] or, interleaved,
+// gu[t] = [gate_0, up_0, gate_1, up_1, ...].
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n, int interleaved) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const size_t t = idx / I;
   const int i = (int)(idx % I);
-  const float g = to_f(gu[t * 2 * I + i]);
-  const float u = to_f(gu[t * 2 * I + I + i]);
+  const float g = to_f(gu[t * 2 * I + (interleaved ? 2 * i : i)]);
+  const float u = to_f(gu[t * 2 * I + (interleaved ? 2 * i + 1 : I + i)]);
   out[idx] = from_f<T>(g / (1.0f + expf(-g)) * u);
 }
 
-extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, void* stream) {
+extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, int interleaved, void* stream) {
   IFX_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   const size_t n = (size_t)T * I;
   const unsigned blocks = (unsigned)((n + 255) / 256);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n);
-  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n);
+  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n, interleaved);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n, interleaved);
   else IFX_FAIL("swiglu: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

@@ -26,7 +26,9 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-template <int MT, int NT, int U, typename TO>
+// EPI 0: out[m, n] = acc.  EPI 1: the rows of W alternate gate, up, gate, up ...; a lane holds two
+// such pairs of one output row and writes silu(gate) * up to out[m, n / 2] (out is [M, N / 2]).
+template <int MT, int NT, int U, typename TO, int EPI>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out,
                                    int M, int N, int K) {
   extern __shared__ float red[];  // [(waves - 1)][NT * MT][64 lanes][4]
@@ -103,31 +105,44 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
     for (int mt = 0; mt < MT; ++mt) {
       const int m = 16 * mt + col;
       if (m >= M) continue;
+      if (EPI == 0) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n_base + 16 * nt + 4 * g + r;
-        if (n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r]);
+        for (int r = 0; r < 4; ++r) {
+          const int n = n_base + 16 * nt + 4 * g + r;
+          if (n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; r += 2) {
+          const int n = n_base + 16 * nt + 4 * g + r;  // even: gate at n, up at n + 1
+          const float gt = acc[nt][mt][r], up = acc[nt][mt][r + 1];
+          if (n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+        }
       }
     }
 }
 
 template <int MT, int NT, int U>
-static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int waves, hipStream_t s) {
+static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int waves, int epi, hipStream_t s) {
   const int groups = (N + 16 * NT - 1) / (16 * NT);
   const size_t lds = (size_t)(waves - 1) * NT * MT * WAVE * 4 * sizeof(float);
   IFX_REQUIRE(lds <= 64 * 1024, "skinny_gemm: %d waves of %dx%d tiles need %zu bytes of LDS", waves, NT, MT, lds);
-  if (out_dtype == DT_BF16)
-    hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, bf16_t>), dim3(groups), dim3(waves * WAVE), lds, s,
-                       (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K);
-  else
-    hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, float>), dim3(groups), dim3(waves * WAVE), lds, s,
-                       (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K);
+#define GO(TO_, EPI_)                                                                                              \
+  hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, TO_, EPI_>), dim3(groups), dim3(waves * WAVE), lds, s,         \
+                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K)
+  if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
+  else if (out_dtype == DT_BF16) GO(bf16_t, 1);
+  else if (epi == 0) GO(float, 0);
+  else GO(float, 1);
+#undef GO
   IFX_LAUNCH_CHECK();
 }
 
 // nt, waves, unroll = 0: chosen here from the shape.
+// epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2].
 extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int nt,
-                               int waves, int unroll, void* stream) {
+                               int waves, int unroll, int epi, void* stream) {
+  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "skinny_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "skinny_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "skinny_gemm: unknown out dtype %d", out_dtype);
@@ -147,7 +162,7 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   }
   IFX_REQUIRE(waves >= 1 && waves <= 16, "skinny_gemm: waves=%d outside 1..16", waves);
   hipStream_t s = (hipStream_t)stream;
-#define CASE(MT_, NT_, U_) if (mt == MT_ && nt == NT_ && unroll == U_) return launch<MT_, NT_, U_>(x, W, out, out_dtype, M, N, K, waves, s)
+#define CASE(MT_, NT_, U_) if (mt == MT_ && nt == NT_ && unroll == U_) return launch<MT_, NT_, U_>(x, W, out, out_dtype, M, N, K, waves, epi, s)
   CASE(1, 1, 4); CASE(1, 2, 4); CASE(1, 1, 2); CASE(1, 2, 2); CASE(1, 1, 8); CASE(1, 2, 8);
   CASE(2, 1, 4); CASE(2, 2, 2); CASE(2, 1, 2); CASE(2, 2, 4);
   CASE(3, 1, 2); CASE(3, 2, 2); CASE(3, 1, 4);

@@ -115,26 +115,37 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     return out
 
 
-def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
-                slots: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], rope_style: int,
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
+    """cos and sin [T, pairs] of float(position) * inv_freq, computed in float."""
+    _check(positions, "positions", (None,), torch.int32)
+    _check(inv_freq, "inv_freq", (None,), torch.float32)
+    T, n = positions.shape[0], inv_freq.shape[0]
+    cs = torch.empty((T, n), dtype=torch.float32, device=positions.device)
+    sn = torch.empty((T, n), dtype=torch.float32, device=positions.device)
+    _call(load_module("core"), "ifx_rope_table", (P, P, P, P, I, I, P),
+          positions.data_ptr(), inv_freq.data_ptr(), cs.data_ptr(), sn.data_ptr(), T, n, _stream())
+    return cs, sn
+
+
+def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rope_style: int,
                 rotary_dim: int, n_heads: int, n_kv_heads: int, head_dim: int,
                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
     """Bias, rotation and cache write of one step's projections; returns q [T, n_heads, head_dim].
 
     ``qkv`` is [T, (n_heads + 2 n_kv_heads) head_dim] when the keys and values are written
     (``slots`` int32 [T] = page * page_size + offset), or [T, n_heads head_dim] with
-    ``n_kv_heads`` = 0 for a mixer that only reads another's cache.
+    ``n_kv_heads`` = 0 for a mixer that only reads another's cache.  ``cos`` / ``sin`` are the
+    step's rotation table [T, rotary_dim / 2] (from rope_table).
     """
     T = qkv.shape[0]
     width = (n_heads + 2 * n_kv_heads) * head_dim
     _check(qkv, "qkv", (T, width))
-    _check(positions, "positions", (T,), torch.int32)
     if bias is not None:
         _check(bias, "bias", (width,))
-    if inv_freq is not None:
-        _check(inv_freq, "inv_freq", (None,), torch.float32)
-        if rope_style != ROPE_NONE and inv_freq.shape[0] < rotary_dim // 2:
-            raise KernelError("inv_freq shorter than rotary_dim / 2")
+    if rope_style != ROPE_NONE:
+        _check(cos, "cos", (T, rotary_dim // 2), torch.float32)
+        _check(sin, "sin", (T, rotary_dim // 2), torch.float32)
     if slots is not None:
         _check(slots, "slots", (T,), torch.int32)
         _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), qkv.dtype)
@@ -143,21 +154,21 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
         raise KernelError("rope_append: keys and values given but no slots to write them to")
     q = torch.empty((T, n_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, P),
-          qkv.data_ptr(), _dt(qkv), _ptr(bias), _dt(bias) if bias is not None else 0, positions.data_ptr(),
-          _ptr(slots), _ptr(inv_freq), rope_style, rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size,
-          q.data_ptr(), _ptr(k_cache), _ptr(v_cache), _stream())
+          qkv.data_ptr(), _dt(qkv), _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
+          _ptr(cos) if rope_style != ROPE_NONE else 0, _ptr(sin) if rope_style != ROPE_NONE else 0, rope_style,
+          rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache), _ptr(v_cache), _stream())
     return q
 
 
-def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
-    """[T, 2I] = [gate | up]  ->  silu(gate) * up  [T, I]."""
+def swiglu(gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """silu(gate) * up [T, I] from [T, 2I] laid out [gate | up] or, interleaved, gate_0, up_0, gate_1, ..."""
     _check(gate_up, "gate_up", (None, None))
     T, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError("swiglu: odd width")
     out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
-    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, P),
-          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, _stream())
+    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, I, P),
+          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, 1 if interleaved else 0, _stream())
     return out
 
 
@@ -192,18 +203,22 @@ SKINNY_MAX_M = 64
 
 
 def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                nt: int = 0, waves: int = 0, unroll: int = 0) -> torch.Tensor:
+                nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
-    accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose."""
+    accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose.
+    With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2]."""
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     _check(weight, "weight", (None, K), torch.bfloat16)
     N = weight.shape[0]
     if M > SKINNY_MAX_M or K % 8:
         raise KernelError(f"skinny_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
-    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, P),
-          x.data_ptr(), weight.data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves, unroll, _stream())
+    if swiglu_pairs and N % 2:
+        raise KernelError("skinny_gemm: gate/up pairs need an even number of weight rows")
+    out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
+    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, I, P),
+          x.data_ptr(), weight.data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves, unroll,
+          1 if swiglu_pairs else 0, _stream())
     return out
 
 
@@ -224,14 +239,26 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     _check(weight, "weight", (None, None))
     out_dtype = out_dtype or torch.bfloat16
     M, K = x.shape
-    N = weight.shape[0]
-    # Measured on the 7B shapes: the streaming kernel wins up to 16 rows everywhere and up to 32 rows
-    # on the narrow products; beyond that the library's tiles reuse the rows better.
-    if K % 8 == 0 and (M <= 16 or (M <= 32 and N <= 4096)):
+    if _use_skinny(M, weight.shape[0], K):
         return skinny_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
     return torch.matmul(x, weight.t())
+
+
+def _use_skinny(M: int, N: int, K: int) -> bool:
+    # Measured on the 7B shapes: the streaming kernel wins up to 16 rows everywhere and up to 32 rows
+    # on the narrow products; beyond that the library's tiles reuse the rows better.
+    return K % 8 == 0 and (M <= 16 or (M <= 32 and N <= 4096))
+
+
+def linear_swiglu(x: torch.Tensor, weight_pairs: torch.Tensor) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) where ``weight_pairs`` [2I, K] alternates the rows of Wg and Wu.
+    For few rows the activation is the product's epilogue; otherwise a second kernel applies it."""
+    M, K = x.shape
+    if weight_pairs.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and _use_skinny(M, weight_pairs.shape[0], K):
+        return skinny_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
+    return swiglu(linear(x, weight_pairs), interleaved=True)
 
 
 # ----------------------------------------------------------------------------------------

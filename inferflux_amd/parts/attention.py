@@ -68,7 +68,7 @@ class PagedAttention(Mixer):
         nH, d = self.n_heads, self.head_dim
         nKV = self.n_kv_heads if binding.writes_cache else 0
         width = (nH + 2 * nKV) * d
-        style, rotary_dim, inv_freq = self.position.kernel_args(h.device)
+        style, rotary_dim, cos, sin = self.position.kernel_args(ctx)
         w, b = self.w_qkv, self.b_qkv
         if not binding.writes_cache:  # only the queries: the first nH*d rows of the fused matrix
             w, b = w[:width], (b[:width] if b is not None else None)
@@ -76,7 +76,7 @@ class PagedAttention(Mixer):
         if self.position.needs_apply:
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
         slots = ctx.write_slots(cache.group) if binding.writes_cache else None
-        q = ops.rope_append(qkv, b, ctx.positions, slots, inv_freq, style, rotary_dim, nH, nKV, d,
+        q = ops.rope_append(qkv, b, slots, cos, sin, style, rotary_dim, nH, nKV, d,
                             cache.k if slots is not None else None, cache.v if slots is not None else None,
                             cache.page_size)
         out = paged_attention(q, cache, ctx, self.window, self.scale)

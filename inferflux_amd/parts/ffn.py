@@ -3,8 +3,10 @@
 g = h Wg^T, u = h Wu^T, a = g / (1 + exp(-g)) * u in float, delta = a Wd^T
 (runtime/backends/cuda/native/transformer_forward.cu:2383-2419, 2487-2494, 2528-2547;
 cuda_kernels.cu:139-151).  The reference runs gate and up as two products; here the two
-matrices are concatenated at load time into one [2I, H] product, which changes nothing in
-the arithmetic of any output element.
+matrices are merged at load time into one [2I, H] matrix whose rows alternate gate_i, up_i, so
+that one product yields both and the kernel that holds a gate value also holds its up value
+(the activation is then the product's epilogue).  This changes nothing in the arithmetic of
+any output element.
 """
 from __future__ import annotations
 
@@ -41,9 +43,11 @@ class SwiGLU(FeedForward):
         }
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.w_gate_up = concat_weights([tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]])
+        g, u = tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
         self.w_down = tensors[f"{self.name}.down_proj.weight"]
 
     def forward(self, h, ctx):
-        gu = ops.linear(h, self.w_gate_up)
-        return ops.linear(ops.swiglu(gu), self.w_down)
+        return ops.linear(ops.linear_swiglu(h, self.w_gate_up), self.w_down)

@@ -1,9 +1,10 @@
 """Position encodings applied to queries and keys before the cache write.
 
-A position part hands the mixer what its fused kernel needs: ``kernel_args(device)`` returns
-(style, rotary_dim, inv_freq).  The kernel computes angle = float(position) * inv_freq[p] in
-float and rotates pair p of every head.  A position part that cannot be expressed this way
-implements ``apply(q, k, positions)`` instead and returns style ROPE_NONE from kernel_args.
+A position part hands the mixer what its fused kernel needs: ``kernel_args(ctx)`` returns
+(style, rotary_dim, cos, sin), the last two being the step's table [T, rotary_dim / 2] of
+angle = float(position) * inv_freq[p], computed in float once per step and shared by every
+layer with the same constants.  The kernel rotates pair p of every head by it.  A position part
+that cannot be expressed this way sets ``needs_apply`` and implements ``apply(q, k, positions)``.
 
 Rotary, split-half ("NeoX") pairing as the reference applies it to qwen2
 (runtime/backends/cuda/native/model_loader.h:39-61 chooses the pairing;
@@ -23,8 +24,8 @@ from .base import Part, register_part
 
 
 class PositionEncoding(Part):
-    def kernel_args(self, device) -> Tuple[int, int, Optional[torch.Tensor]]:
-        return ops.ROPE_NONE, 0, None
+    def kernel_args(self, ctx) -> Tuple[int, int, Optional[torch.Tensor], Optional[torch.Tensor]]:
+        return ops.ROPE_NONE, 0, None, None
 
     def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], positions: torch.Tensor):
         """Transform q [T, nH, d] and k [T, nKV, d] (or None) outside the fused kernel."""
@@ -66,5 +67,7 @@ class RotaryPosition(PositionEncoding):
             self._inv_freq[key] = t
         return t
 
-    def kernel_args(self, device):
-        return self.STYLES[self.style], self.rotary_dim, self.inv_freq(device)
+    def kernel_args(self, ctx):
+        cos, sin = ctx.derived(("rotary_table", self.theta, self.rotary_dim),
+                               lambda: ops.rope_table(ctx.positions, self.inv_freq(ctx.device)))
+        return self.STYLES[self.style], self.rotary_dim, cos, sin

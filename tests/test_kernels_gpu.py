@@ -89,8 +89,8 @@ def test_rope_append(dtype, style, rot, bias):
     rd = rot or d
     inv_freq = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64), 2.0 * torch.arange(rd // 2, dtype=torch.float64) / rd)).float()
     code = {"split_half": ops.ROPE_SPLIT_HALF, "consecutive": ops.ROPE_CONSECUTIVE, "none": ops.ROPE_NONE}[style]
-    q = ops.rope_append(qkv.to(DEV), b.to(DEV) if bias else None, positions.to(DEV), slots.to(DEV),
-                        inv_freq.to(DEV) if style != "none" else None, code, rd, nH, nKV, d, kc, vc, P)
+    cs, sn = ops.rope_table(positions.to(DEV), inv_freq.to(DEV)) if style != "none" else (None, None)
+    q = ops.rope_append(qkv.to(DEV), b.to(DEV) if bias else None, slots.to(DEV), cs, sn, code, rd, nH, nKV, d, kc, vc, P)
     x = qkv.double() + (b.double() if bias else 0)
     xq, xk, xv = x[:, : nH * d].view(T, nH, d), x[:, nH * d: (nH + nKV) * d].view(T, nKV, d), x[:, (nH + nKV) * d:].view(T, nKV, d)
 
@@ -117,7 +117,8 @@ def test_rope_queries_only():
     qo = torch.randn(T, nH * d, generator=g)
     pos = torch.tensor([3, 4, 5, 6], dtype=torch.int32)
     inv = (1.0 / torch.pow(torch.tensor(1e4, dtype=torch.float64), 2.0 * torch.arange(d // 2, dtype=torch.float64) / d)).float()
-    q = ops.rope_append(qo.to(DEV), None, pos.to(DEV), None, inv.to(DEV), ops.ROPE_SPLIT_HALF, d, nH, 0, d, None, None, 16)
+    cs, sn = ops.rope_table(pos.to(DEV), inv.to(DEV))
+    q = ops.rope_append(qo.to(DEV), None, None, cs, sn, ops.ROPE_SPLIT_HALF, d, nH, 0, d, None, None, 16)
     assert torch.allclose(q.cpu().double(), pm.rope_split_half(qo.double().view(T, nH, d), pos.tolist(), 1e4), atol=1e-5)
 
 
@@ -127,6 +128,9 @@ def test_swiglu(dtype):
     gu = (3 * torch.randn(5, 2 * 37, generator=g)).to(dtype)
     out = ops.swiglu(gu.to(DEV)).cpu().double()
     gate, up = gu.double()[:, :37], gu.double()[:, 37:]
+    assert torch.allclose(out, gate / (1 + torch.exp(-gate)) * up, **tol(dtype))
+    out = ops.swiglu(gu.to(DEV), interleaved=True).cpu().double()
+    gate, up = gu.double()[:, 0::2], gu.double()[:, 1::2]
     assert torch.allclose(out, gate / (1 + torch.exp(-gate)) * up, **tol(dtype))
 
 
@@ -382,3 +386,17 @@ def test_linear_picks_by_weight_type_and_rows():
         assert logits.dtype == F32 and torch.allclose(logits.cpu().double(), want, rtol=1e-4, atol=1e-3)   # no bf16 rounding
         mixed = ops.linear(x.bfloat16().to(DEV), w.to(DEV))                  # a float32 weight in bf16 mode
         assert mixed.dtype == BF16 and torch.allclose(mixed.cpu().double(), x.bfloat16().double() @ w.double().t(), rtol=1e-2, atol=0.1)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 40, 100])
+def test_linear_swiglu_pairs(M):
+    g = gen(14)
+    I, K = 1000 if M != 8 else 37, 144
+    x = torch.randn(M, K, generator=g).to(BF16)
+    wg, wu = torch.randn(I, K, generator=g).to(BF16) * 0.2, torch.randn(I, K, generator=g).to(BF16) * 0.2
+    pairs = torch.stack([wg, wu], dim=1).reshape(2 * I, K).contiguous()
+    got = ops.linear_swiglu(x.to(DEV), pairs.to(DEV)).cpu().double()
+    gt, up = x.double() @ wg.double().t(), x.double() @ wu.double().t()
+    assert got.shape == (M, I) and torch.allclose(got, gt / (1 + torch.exp(-gt)) * up, rtol=2e-2, atol=2e-2)
+    got32 = ops.linear_swiglu(x.float().to(DEV), pairs.float().to(DEV)).cpu().double()     # the 32-bit path
+    assert torch.allclose(got32, gt / (1 + torch.exp(-gt)) * up, rtol=1e-4, atol=1e-4)
