@@ -62,6 +62,10 @@ __device__ __forceinline__ bf16x4 zero4() {
   return z;
 }
 
+// 2^x on the hardware's exponent unit.  Arguments are <= 0 here and results below the smallest
+// normal float may flush to zero, which a softmax weight of that size may.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // max over the four lanes that hold the same query column (lane, lane^16, lane^32, lane^48)
 __device__ __forceinline__ float col_max(float v) {
   v = fmaxf(v, __shfl_xor(v, 16, WAVE));
@@ -141,14 +145,14 @@ __device__ __forceinline__ void use_row_block(const RowBlock& b, const RowArgs& 
   }
   const float m_new = fmaxf(m, col_max(mb));
   const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = exp2f(m - m_safe);
+  const float alpha = fast_exp2(m - m_safe);
   float psum = 0.f;
   bf16x4 pb[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float p = exp2f(s[t][r] - m_safe);
+      const float p = fast_exp2(s[t][r] - m_safe);
       psum += p;
       pb[t][r] = (__bf16)p;
     }
@@ -314,15 +318,96 @@ struct TileArgs {
   const int* block_table;
   int max_blocks, nH, nKV, P, window;
   float scale_log2e;
+  int page_shift;         // log2(P): the tile kernel takes power-of-two pages and splits positions by shift and mask
+  int n_tiles, per_xcd;   // work items are (tile, head); per_xcd = ceil(n_tiles * nH / 8)
 };
+
+constexpr int N_PIECES = TK * (D / 8);                // 16-byte pieces of a K tile, and as many of a V^T tile
+constexpr int K_PIECES = (N_PIECES + 255) / 256;      // ... per thread (256 threads)
+constexpr int V_PIECES = K_PIECES;
+
+// A thread's share of one K tile and one V^T tile, fetched into registers one tile ahead of the
+// arithmetic and stored to LDS when the previous tile has been consumed.
+struct TileRegs {
+  bf16x8 k[K_PIECES];
+  bf16x8 v[V_PIECES];
+};
+
+// The pages of a tile's four runs of 16 keys (-1: none), the same for every thread.  They are looked
+// up one tile before the data is fetched, so that fetching costs one trip to memory, not two.
+__device__ __forceinline__ void tile_pages(int* pg, const TileArgs& a, const int* table, int j0, int pos_last) {
+#pragma unroll
+  for (int i = 0; i < TK / 16; ++i) {
+    const int j = j0 + 16 * i, blk = j >> a.page_shift;
+    pg[i] = (j <= pos_last && blk < a.max_blocks) ? table[blk] : -1;
+  }
+}
+
+__device__ __forceinline__ int pick_page(const int* pg, int sub) {
+  int p = pg[0];
+#pragma unroll
+  for (int i = 1; i < TK / 16; ++i) p = sub == i ? pg[i] : p;
+  return p;
+}
+
+__device__ __forceinline__ void fetch_tile(TileRegs& r, const TileArgs& a, const int* pg, int kvh, int j0, int tid) {
+  const int P = a.P;
+#pragma unroll
+  for (int i = 0; i < K_PIECES; ++i) {
+    const int c = tid + 256 * i;
+    const int key = c / (D / 8), c8 = c % (D / 8);
+    const int page = c < N_PIECES ? pick_page(pg, key >> 4) : -1;
+    r.k[i] = page >= 0 ? *(const bf16x8*)(a.k_cache + (((size_t)page * a.nKV + kvh) * P + ((j0 + key) & (P - 1))) * D + 8 * c8) : zero8();
+  }
+#pragma unroll
+  for (int i = 0; i < V_PIECES; ++i) {
+    const int c = tid + 256 * i;
+    const int dim = c / (TK / 8), k8 = c % (TK / 8);  // 8 keys never straddle a page
+    const int page = c < N_PIECES ? pick_page(pg, k8 >> 1) : -1;
+    r.v[i] = page >= 0 ? *(const bf16x8*)(a.v_cache + (((size_t)page * a.nKV + kvh) * D + dim) * P + ((j0 + 8 * k8) & (P - 1))) : zero8();
+  }
+}
+
+__device__ __forceinline__ void stage_tile(const TileRegs& r, bf16_t* k_s, bf16_t* v_s, int tid) {
+#pragma unroll
+  for (int i = 0; i < K_PIECES; ++i) {
+    const int c = tid + 256 * i;
+    if (c < N_PIECES) *(bf16x8*)(k_s + (c / (D / 8)) * KPAD + 8 * (c % (D / 8))) = r.k[i];
+  }
+#pragma unroll
+  for (int i = 0; i < V_PIECES; ++i) {
+    const int c = tid + 256 * i;
+    if (c < N_PIECES) {
+      // Keys are stored in the order the second product consumes them: within each run of 32 keys,
+      // position 8 g + 4 h + r holds key 16 h + 4 g + r, so that one 16-byte read gives a lane its
+      // four keys of both 16-key score tiles.  A piece of 8 consecutive keys lands as two halves.
+      const int dim = c / (TK / 8), k8 = c % (TK / 8);
+      bf16_t* dst = v_s + dim * VPAD + 32 * (k8 / 4) + 16 * (k8 % 2) + 4 * ((k8 % 4) / 2);
+      bf16x4 lo, hi;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { lo[e] = r.v[i][e]; hi[e] = r.v[i][e + 4]; }
+      *(bf16x4*)dst = lo;
+      *(bf16x4*)(dst + 8) = hi;
+    }
+  }
+}
 
 __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t k_s[TK * KPAD];
   __shared__ __attribute__((aligned(16))) bf16_t v_s[D * VPAD];
   const int tid = threadIdx.x, wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g4 = lane >> 4;
-  const int req = a.tile_req[blockIdx.x], q0 = a.tile_q0[blockIdx.x], head = blockIdx.y;
-  const int kvh = head / (a.nH / a.nKV);
-  const int qlen = a.q_len[req], kvlen = a.kv_len[req], P = a.P;
+  // Workgroups go to the 8 XCDs round-robin by their number, and every XCD has an L2 of its own.
+  // Work items are ordered kv head first and dealt to the XCDs in contiguous runs, so that the
+  // workgroups that read one kv head's keys and values share an L2 instead of filling all eight with
+  // everything; within a run the tiles with the most keys (the latest rows) come first.
+  const int ratio = a.nH / a.nKV;
+  const int item = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
+  if (blockIdx.x / 8 >= a.per_xcd || item >= a.n_tiles * a.nH) return;   // the whole workgroup leaves together
+  const int per_kv = ratio * a.n_tiles;
+  const int kvh = item / per_kv, rem = item % per_kv;
+  const int head = kvh * ratio + rem / a.n_tiles, ti = a.n_tiles - 1 - rem % a.n_tiles;
+  const int req = a.tile_req[ti], q0 = a.tile_q0[ti];
+  const int qlen = a.q_len[req], kvlen = a.kv_len[req];
   const int start = kvlen - qlen;                       // position of the request's first row in this step
   const int* table = a.block_table + (size_t)req * a.max_blocks;
   const int rows_here = min(TQ, qlen - q0);
@@ -334,6 +419,9 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
   const int my_pos = start + my_q;
   const int my_lo = a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
   const size_t my_row = (size_t)a.q_start[req] + my_q;
+  // the keys this wave's 16 rows can see at all: tiles outside are skipped by the whole wave
+  const int wave_hi = min(pos_last, pos_first + 16 * wid + 15);
+  const int wave_lo = a.window > 0 ? max(0, pos_first + 16 * wid - a.window + 1) : 0;
   bf16x8 qop[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -345,27 +433,21 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
   for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  for (int j0 = (lo_wg / TK) * TK; j0 <= pos_last; j0 += TK) {
+  TileRegs regs;
+  int pg[TK / 16];
+  int j0 = (lo_wg / TK) * TK;
+  tile_pages(pg, a, table, j0, pos_last);
+  fetch_tile(regs, a, pg, kvh, j0, tid);
+  tile_pages(pg, a, table, j0 + TK, pos_last);
+  for (; j0 <= pos_last; j0 += TK) {
     __syncthreads();  // everyone is done with the previous tile
-    // K tile: TK rows of D elements, in 16-byte pieces
-    for (int c = tid; c < TK * (D / 8); c += 256) {
-      const int key = c / (D / 8), c8 = c % (D / 8);
-      const int j = j0 + key, blk = j / P;
-      const int page = (j <= pos_last && blk < a.max_blocks) ? table[blk] : -1;
-      bf16x8 v = zero8();
-      if (page >= 0) v = *(const bf16x8*)(a.k_cache + (((size_t)page * a.nKV + kvh) * P + j % P) * D + 8 * c8);
-      *(bf16x8*)(k_s + key * KPAD + 8 * c8) = v;
-    }
-    // V^T tile: D rows of TK keys, in 16-byte pieces of 8 keys (8 keys never straddle a page)
-    for (int c = tid; c < D * (TK / 8); c += 256) {
-      const int dim = c / (TK / 8), k8 = c % (TK / 8);
-      const int j = j0 + 8 * k8, blk = j / P;
-      const int page = (j <= pos_last && blk < a.max_blocks) ? table[blk] : -1;
-      bf16x8 v = zero8();
-      if (page >= 0) v = *(const bf16x8*)(a.v_cache + (((size_t)page * a.nKV + kvh) * D + dim) * P + j % P);
-      *(bf16x8*)(v_s + dim * VPAD + 8 * k8) = v;
-    }
+    stage_tile(regs, k_s, v_s, tid);
     __syncthreads();
+    if (j0 + TK <= pos_last) {  // the next tile's data and the one after's pages: in flight during the arithmetic
+      fetch_tile(regs, a, pg, kvh, j0 + TK, tid);
+      tile_pages(pg, a, table, j0 + 2 * TK, pos_last);
+    }
+    if (j0 > wave_hi || j0 + TK <= wave_lo) continue;   // uniform over the wave; barriers are at the loop's top
 
     floatx4 s[4];
     float mb = -INFINITY;
@@ -388,27 +470,29 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
     }
     const float m_new = fmaxf(m, col_max(mb));
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f(m - m_safe);
+    const float alpha = fast_exp2(m - m_safe);
     float psum = 0.f;
     bf16x4 pb[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = exp2f(s[t][r] - m_safe);
+        const float p = fast_exp2(s[t][r] - m_safe);
         psum += p;
         pb[t][r] = (__bf16)p;
       }
     l = l * alpha + psum;
     m = m_new;
     const bf16x8 pop0 = join4(pb[0], pb[1]), pop1 = join4(pb[2], pb[3]);
+    const bool rescale = __any(alpha != 1.0f);   // once the running maxima have settled nothing is rescaled
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 4 * g4;
-      const bf16x8 vop0 = join4(*(const bf16x4*)(vr), *(const bf16x4*)(vr + 16));
-      const bf16x8 vop1 = join4(*(const bf16x4*)(vr + 32), *(const bf16x4*)(vr + 48));
+      const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 8 * g4;
+      const bf16x8 vop0 = *(const bf16x8*)(vr), vop1 = *(const bf16x8*)(vr + 32);
+      if (rescale) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+      }
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop0, o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop1, o[dt], 0, 0, 0);
     }
@@ -435,9 +519,16 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_tiles: page_size %d must be a multiple of 16", page_size);
   IFX_REQUIRE(nH <= 65535, "attn_tiles: too many heads for one launch");
+  IFX_REQUIRE((page_size & (page_size - 1)) == 0, "attn_tiles: page_size %d must be a power of two", page_size);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
   if (n_tiles == 0) return 0;
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
-             q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f};
-  hipLaunchKernelGGL(attn_tiles_kernel, dim3(n_tiles, nH), dim3(256), 0, (hipStream_t)stream, a);
+             q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
+             n_tiles, 0};
+  const long long items = (long long)n_tiles * nH;
+  IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
+  a.per_xcd = (int)((items + 7) / 8);
+  hipLaunchKernelGGL(attn_tiles_kernel, dim3(8 * a.per_xcd), dim3(256), 0, (hipStream_t)stream, a);
   IFX_LAUNCH_CHECK();
 }

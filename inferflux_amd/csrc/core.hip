@@ -316,10 +316,32 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   out[idx] = from_f<T>(g / (1.0f + expf(-g)) * u);
 }
 
+// The interleaved bf16 case in 32-byte pieces: 8 gate/up pairs in, 8 results out (I a multiple of 8).
+__global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, size_t n8) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n8) return;
+  const bf16x8 a = *(const bf16x8*)(gu + 16 * i), b = *(const bf16x8*)(gu + 16 * i + 8);
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float g0 = (float)a[2 * e], u0 = (float)a[2 * e + 1], g1 = (float)b[2 * e], u1 = (float)b[2 * e + 1];
+    o[e] = (__bf16)(g0 / (1.0f + expf(-g0)) * u0);
+    o[e + 4] = (__bf16)(g1 / (1.0f + expf(-g1)) * u1);
+  }
+  *(bf16x8*)(out + 8 * i) = o;
+}
+
 extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, int interleaved, void* stream) {
   IFX_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   const size_t n = (size_t)T * I;
+  if (interleaved && dtype == DT_BF16 && I % 8 == 0) {
+    const size_t n8 = n / 8;
+    hipLaunchKernelGGL(swiglu_pairs_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t*)gu, (bf16_t*)out, n8);
+    IFX_LAUNCH_CHECK();
+  }
   const unsigned blocks = (unsigned)((n + 255) / 256);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n, interleaved);

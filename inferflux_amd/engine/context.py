@@ -31,7 +31,12 @@ class StepEntry:
 
 
 class StepContext:
-    def __init__(self, entries: Sequence[StepEntry], manager, act_dtype: torch.dtype, device):
+    """``width_multiple`` rounds the block tables' width up (a replayed graph needs the same layout
+    for many steps).  ``slab`` is a device buffer to fill instead of a new one, ``pinned`` the host
+    buffer the copy goes through; ``layout_key`` tells whether two steps have the same layout."""
+
+    def __init__(self, entries: Sequence[StepEntry], manager, act_dtype: torch.dtype, device,
+                 width_multiple: int = 8, slab: torch.Tensor = None, pinned: torch.Tensor = None, upload: bool = True):
         self.act_dtype, self.device = act_dtype, device
         self.entries = list(entries)
         R = self.n_requests = len(self.entries)
@@ -59,7 +64,7 @@ class StepContext:
         self.h_write_slots: List[np.ndarray] = []
         for g in range(n_groups):
             tables = [manager.block_table(e.rid, g) for e in self.entries]
-            width = max(8, -(-max((len(t) for t in tables), default=1) // 8) * 8)
+            width = max(width_multiple, -(-max((len(t) for t in tables), default=1) // width_multiple) * width_multiple)
             bt = np.full((R, width), -1, dtype=np.int32)
             for i, t in enumerate(tables):
                 bt[i, :len(t)] = t
@@ -81,16 +86,45 @@ class StepContext:
         for name, a in named:
             offs[name] = (total, a.size, a.shape)
             total += (a.size + 3) // 4 * 4
-        slab = np.zeros(max(total, 4), dtype=np.int32)
-        for name, a in named:
-            o, n, _ = offs[name]
-            slab[o:o + n] = a.reshape(-1)
-        self._slab = torch.from_numpy(slab).to(device)
+        self.layout_key = (R, T, self.n_logit_rows, tuple(bt.shape[1] for bt in self.h_block_tables))
+        # No request of this step holds more positions than its block table has room for.  Kernels size
+        # their grids by this bound, not by the lengths themselves, so that a captured step stays valid
+        # while lengths grow within the same table width.
+        self.kv_bound = max((bt.shape[1] for bt in self.h_block_tables), default=0) * P
+        self.slab_size = max(total, 4)
+        self._named, self._offs = named, offs
         self._views: Dict[str, torch.Tensor] = {}
-        for name, _ in named:
-            o, n, shape = offs[name]
-            self._views[name] = self._slab[o:o + n].view(shape)
         self._derived: Dict[object, object] = {}
+        self._slab = None
+        if upload:
+            self.bind(slab, pinned)
+
+    def bind(self, slab: torch.Tensor = None, pinned: torch.Tensor = None) -> None:
+        """Put the step's arrays on the device: into ``slab`` through ``pinned`` when given (an
+        asynchronous copy on the current stream), else into a new tensor."""
+        if pinned is not None:
+            host = pinned.numpy()
+        else:
+            host = np.zeros(self.slab_size, dtype=np.int32)
+        for name, a in self._named:
+            o, n, _ = self._offs[name]
+            host[o:o + n] = a.reshape(-1)
+        if slab is None:
+            slab = torch.from_numpy(host).to(self.device)
+        elif pinned is not None:
+            slab.copy_(pinned, non_blocking=True)
+        else:
+            slab.copy_(torch.from_numpy(host))
+        self.use_slab(slab)
+
+    def use_slab(self, slab: torch.Tensor) -> None:
+        """Take ``slab`` (which already holds a step of this layout) as the device arrays."""
+        self._slab = slab
+        self._views = {}
+        for name, _ in self._named:
+            o, n, shape = self._offs[name]
+            self._views[name] = slab[o:o + n].view(shape)
+        self._derived = {}
 
     # ---- device views -------------------------------------------------------------
     @property

@@ -47,6 +47,10 @@ class Model:
         yield from _walk(self.final_norm)
         yield from _walk(self.head)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts())
+
     def schedule_mixers(self) -> List:
         return [self.blocks[e.layer].mixer for e in self.plan.schedule]
 

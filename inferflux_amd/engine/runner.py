@@ -27,8 +27,21 @@ class StepError(ValueError):
     """A step that cannot run; the cache is unchanged."""
 
 
+class _DecodeGraph:
+    """A captured decode step: the device arrays it reads, the host buffer they are filled through,
+    the graph and the logits it writes."""
+
+    def __init__(self, slab, pinned, graph, ctx, logits):
+        self.slab, self.pinned, self.graph, self.ctx, self.logits = slab, pinned, graph, ctx, logits
+        self.copied = torch.cuda.Event()
+
+
 class ModelRunner:
-    def __init__(self, model: Model, num_pages: int, page_size: int = 16, max_requests: int = 64):
+    GRAPH_WIDTH_MULTIPLE = 64     # block-table width (pages) a captured step is valid for, in steps of this
+    MAX_GRAPHS = 12
+
+    def __init__(self, model: Model, num_pages: int, page_size: int = 16, max_requests: int = 64,
+                 decode_graphs: bool = True):
         if model.device is None:
             raise ValueError("the model has no weights yet (load_folder / init_random first)")
         if model.device.type != "cuda":
@@ -41,6 +54,12 @@ class ModelRunner:
         self.page_size = page_size
         self.vocab_size = model.plan.vocab_size
         self.max_position = model.plan.max_position
+        # Steps in which every request brings one token are captured as HIP graphs, one per layout
+        # (batch size, wanted rows, block-table width), and replayed: a decode step is some 250
+        # launches, which the host cannot issue as fast as the GPU runs them.  The reference does the
+        # same per batch size (runtime/backends/cuda/native/transformer_forward.cu:3068-3117).
+        self.decode_graphs = decode_graphs and model.graph_safe
+        self._graphs = {}
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, rid: Hashable) -> None:
@@ -92,8 +111,40 @@ class ModelRunner:
             raise OutOfPages(g, tot[g], self.manager.pools[g].num_free)
         for rid, n in needs:
             self.manager.reserve(rid, n)
-        ctx = StepContext(entries, self.manager, self.dtype, self.device)
-        logits = self.model.forward(ctx, self.storage)
+        if self.decode_graphs and all(n == 1 for _, n in needs):
+            logits = self._decode_step(entries)
+        else:
+            ctx = StepContext(entries, self.manager, self.dtype, self.device)
+            logits = self.model.forward(ctx, self.storage)
         for rid, n in needs:
             self.manager.commit(rid, n)
+        return logits
+
+    def _decode_step(self, entries) -> torch.Tensor:
+        """A step of single tokens through a captured graph.  The first step of a layout runs as usual
+        and is then captured; later steps copy their arrays into the graph's buffer and replay it.
+        The logits returned by a replay live in the graph's memory: they are valid until the next step."""
+        ctx = StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
+                          upload=False)
+        g = self._graphs.get(ctx.layout_key)
+        if g is not None:
+            g.copied.synchronize()          # the host buffer is free again once the last copy out of it is done
+            ctx.bind(g.slab, g.pinned)
+            g.copied.record()
+            g.graph.replay()
+            return g.logits
+        slab = torch.empty(ctx.slab_size, dtype=torch.int32, device=self.device)
+        pinned = torch.empty(ctx.slab_size, dtype=torch.int32, pin_memory=True)
+        ctx.bind(slab, pinned)
+        logits = self.model.forward(ctx, self.storage)            # this step, eagerly (also loads every kernel)
+        if len(self._graphs) >= self.MAX_GRAPHS:
+            self._graphs.pop(next(iter(self._graphs)))
+        torch.cuda.synchronize()
+        cap_ctx = StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
+                              upload=False)
+        cap_ctx.use_slab(slab)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cap_logits = self.model.forward(cap_ctx, self.storage)
+        self._graphs[ctx.layout_key] = _DecodeGraph(slab, pinned, graph, cap_ctx, cap_logits)
         return logits

@@ -38,7 +38,7 @@ def _work_lists(ctx):
     if rows.size:
         if rows.size != ctx.n_tokens:
             out["rows"] = ctx.upload(rows)
-        max_kv = int(kv_len[~tiled].max())
+        max_kv = ctx.kv_bound     # not the lengths themselves: see StepContext.kv_bound
         chunk = ROW_CHUNK
         while -(-max_kv // chunk) > ROW_MAX_SPLITS:
             chunk *= 2

@@ -283,7 +283,8 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 
 def mfma_attention_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
-    return dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= MFMA_MAX_HEAD_DIM and page_size % 16 == 0
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= MFMA_MAX_HEAD_DIM
+            and page_size >= 16 and page_size & (page_size - 1) == 0)
 
 
 def _attn_common(q, k_cache, v_cache):
@@ -294,7 +295,7 @@ def _attn_common(q, k_cache, v_cache):
     _check(v_cache, "v_cache", (n_pages, nKV, d, page_size), torch.bfloat16)
     if not mfma_attention_supported(q.dtype, d, page_size):
         raise KernelError(f"matrix-core attention needs bfloat16, head_dim a multiple of 16 up to {MFMA_MAX_HEAD_DIM} and "
-                          f"page_size a multiple of 16; got head_dim {d}, page_size {page_size}")
+                          f"page_size a power of two from 16; got head_dim {d}, page_size {page_size}")
     return T, nH, d, nKV, page_size, load_module("attn_mfma", (("HEAD_DIM", d),))
 
 

@@ -28,6 +28,8 @@ from .plan import CacheSpec, ParamSpec, PartSpec
 
 @register_part("mixer", "paged_attention")
 class PagedAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, name: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, bias: bool = True, window: Optional[int] = None,
                  scale: Optional[float] = None, init_std: float = 0.02):

@@ -63,7 +63,16 @@ def registered_parts(category: str):
 
 
 class Part:
-    """Base of all parts."""
+    """Base of all parts.
+
+    ``graph_safe`` says that ``forward`` reads a step's metadata only from the context's device
+    tensors and launches the same kernels with the same grid for every step of one layout
+    (``StepContext.layout_key``), so that a decode step may be captured once and replayed.  A part
+    that loops on the host over ``ctx.h_*`` arrays must leave it False; a model with such a part
+    runs every step eagerly.
+    """
+
+    graph_safe = False
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         """Full tensor names this part reads from the model file."""

@@ -14,6 +14,8 @@ from .plan import LayerSpec
 
 @register_part("block", "prenorm")
 class PreNormBlock(Block):
+    graph_safe = True
+
     def __init__(self, layer: LayerSpec, hidden_size: int):
         self.prefix = layer.prefix
         self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)

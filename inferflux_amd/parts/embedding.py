@@ -20,6 +20,8 @@ from .plan import ParamSpec
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02):
         self.name, self.vocab_size, self.hidden_size, self.init_std = name, int(vocab_size), int(hidden_size), init_std
         self.table: Optional[torch.Tensor] = None
@@ -36,6 +38,8 @@ class TokenEmbedding(Part):
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
+    graph_safe = True
+
     """``tied_to`` names the tensor (the embedding table) a tied head shares; None for its own."""
 
     def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, init_std: float = 0.02):

@@ -28,6 +28,8 @@ def concat_weights(parts):
 
 @register_part("ffn", "swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, name: str, hidden_size: int, intermediate_size: int, init_std: float = 0.02):
         self.name, self.hidden_size, self.intermediate_size = name, int(hidden_size), int(intermediate_size)
         self.init_std = init_std

@@ -16,6 +16,8 @@ from .plan import ParamSpec
 
 @register_part("norm", "rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, name: str, hidden_size: int, eps: float):
         self.name, self.hidden_size, self.eps = name, int(hidden_size), float(eps)
         self.weight: Optional[torch.Tensor] = None

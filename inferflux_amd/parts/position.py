@@ -36,12 +36,16 @@ class PositionEncoding(Part):
 
 @register_part("position", "none")
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, head_dim: int = 0):
         self.head_dim = head_dim
 
 
 @register_part("position", "rotary")
 class RotaryPosition(PositionEncoding):
+    graph_safe = True
+
     """``style``: "split_half" pairs (p, p + rot/2); "consecutive" pairs (2p, 2p+1)."""
 
     STYLES = {"split_half": ops.ROPE_SPLIT_HALF, "consecutive": ops.ROPE_CONSECUTIVE}

@@ -203,3 +203,45 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         rows.append(out.cpu()); p += m
     assert torch.allclose(torch.cat(rows), whole, rtol=1e-4, atol=1e-5)
     assert not torch.allclose(whole[1:], whole[:-1])
+
+
+# ---- captured decode steps ----------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_replayed_decode_graphs_equal_eager_steps(name, dtype, sharp_folders):
+    """The same trace with captured decode steps and without: every replay (many per graph, with eager
+    prefill steps and synchronisations between them, across block-table widths and changing batches)
+    must give the eager logits."""
+    folder = sharp_folders[name, dtype]
+    V = TINY[name]["vocab_size"]
+    eager = load_runner(folder, DT[dtype], num_pages=64)
+    eager.decode_graphs = False
+    graphed = load_runner(folder, DT[dtype], num_pages=64)
+    graphed.GRAPH_WIDTH_MULTIPLE = 2                     # a new layout every 32 positions
+    assert graphed.decode_graphs
+    seqs = {r: seeded_ids(400 + i, n, V) for i, (r, n) in enumerate({"a": 150, "b": 90, "c": 120}.items())}
+    pos = {r: 0 for r in seqs}
+    plan = [("a", 20), ("b", 5)] + [("ab", 1)] * 30 + [("c", 33)] + [("abc", 1)] * 25 + [("free b", 0)] + [("ac", 1)] * 27
+    replays = 0
+    for who, n in plan:
+        if who.startswith("free"):
+            for r in (eager, graphed):
+                r.free_request(who.split()[1])
+            continue
+        entries = []
+        for rid in who:
+            for r in (eager, graphed):
+                if not r.has_request(rid):
+                    r.add_request(rid)
+            entries.append(StepEntry(rid, seqs[rid][pos[rid]: pos[rid] + n], [n - 1]))
+            pos[rid] += n
+        before = len(graphed._graphs)
+        want, got = eager.step(entries).cpu(), graphed.step(entries).cpu()
+        replays += n == 1 and len(graphed._graphs) == before
+        if dtype == "float32":
+            assert torch.equal(got, want), (who, pos)
+        else:
+            assert torch.allclose(got, want, rtol=0, atol=0), (who, pos)   # same kernels, same order: equal bits
+    assert replays > 60 and len(graphed._graphs) >= 4
+    want = plain_logits(folder, seqs["a"][: pos["a"]])[-1]
+    assert rel_err(got[0], want) < REL_TOL[dtype]
