@@ -34,6 +34,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -48,6 +49,15 @@ def main() -> int:
     from inferflux_amd.engine.runner import ModelRunner
     from inferflux_amd.engine.scheduler import SchedulerConfig
 
+    from inferflux_amd.kernels import ops
+    if not args.no_gemm_tuning:
+        # Prefill and batch-64 products go to the library: let it time its kernels for the shapes that
+        # are measured (not for the one-off shapes of the set-up).
+        ops.enable_library_gemm_tuning(300)
+        ops.pause_library_gemm_tuning(True)
+
+    def note(msg):
+        print(f"[bench] {msg}", file=sys.stderr, flush=True)
     shape = dict(SHAPE_7B)
     layers_full = shape["num_hidden_layers"]
     if args.layers:
@@ -81,8 +91,11 @@ def main() -> int:
             eng.add_request(torch.randint(0, V, (DECODE_KV_START,), generator=gen).tolist(), SamplingParams(**vars(sp)))
         while any(s.is_prefilling for s in eng.scheduler.running) or eng.scheduler.waiting:
             eng.step()                                            # prompts in; every request now decodes
+        note(f"batch {batch}: prompts are in, decoding")
+        ops.pause_library_gemm_tuning(False)
         for _ in range(warmup):
             eng.step()
+        ops.pause_library_gemm_tuning(True)
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
@@ -98,6 +111,7 @@ def main() -> int:
         runner = ModelRunner(model, num_pages=-(-tokens // PAGE) + 1, page_size=PAGE, max_requests=2)
         ids = torch.randint(0, V, (tokens,), generator=gen).tolist()
         best = None
+        ops.pause_library_gemm_tuning(False)
         for i in range(reps + 1):
             runner.add_request(i)
             torch.cuda.synchronize()
@@ -106,13 +120,16 @@ def main() -> int:
             torch.cuda.synchronize()
             dt = time.perf_counter() - t
             runner.free_request(i)
+            ops.pause_library_gemm_tuning(True)
+            note(f"prefill of {tokens} tokens: {dt * 1e3:.1f} ms")
             if i > 0:
                 best = dt if best is None else min(best, dt)
         linear = 2.0 * tokens * L * ((nH + 2 * nKV) * d * H + nH * d * H + 3 * I * H) + 2.0 * V * H
         attn = 4.0 * L * nH * d * tokens * (tokens + 1) / 2
         return tokens / best, best * 1e3, (linear + attn) / best / 1e12 / PEAK_TFLOPS[args.dtype]
 
-    tps, ms, kv_mean = decode_rate(args.batch, args.steps, args.warmup)
+    tps, ms, kv_mean = decode_rate(args.batch, args.steps, max(args.warmup, 1))
+    note(f"batch {args.batch}: {tps:.0f} tokens/s")
     step_bytes = weight_bytes + args.batch * kv_mean * kv_bytes_per_token
     achieved = step_bytes / (ms * 1e-3) / 1e9
     out = {
@@ -124,7 +141,7 @@ def main() -> int:
                    "num_hidden_layers": layers_full, "layers_run": L, "hidden_size": H, "num_attention_heads": nH,
                    "num_key_value_heads": nKV, "head_dim": d, "intermediate_size": I, "vocab_size": V,
                    "prompt_len": PROMPT, "decode_kv_start": DECODE_KV_START, "kv_page_size": PAGE,
-                   "tie_word_embeddings": False, "attention_bias": True},
+                   "tie_word_embeddings": False, "library_gemm_tuning": not args.no_gemm_tuning},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
     }

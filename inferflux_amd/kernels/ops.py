@@ -202,6 +202,29 @@ def gemm_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
 SKINNY_MAX_M = 64
 
 
+def enable_library_gemm_tuning(max_ms_per_shape: int = 300, filename: Optional[str] = None) -> None:
+    """Let the library pick, by timing, the fastest of its kernels for every matrix-product shape it
+    meets (torch's TunableOp over hipBLASLt and rocBLAS).  The first product of a shape then takes
+    up to ``max_ms_per_shape`` longer; worth it when shapes repeat (a fixed prefill portion, a steady
+    decode batch), not for one-off shapes, so it is off unless asked for."""
+    import torch.cuda.tunable as tunable
+    tunable.enable(True)
+    tunable.tuning_enable(True)
+    tunable.set_max_tuning_duration(int(max_ms_per_shape))
+    if not filename:
+        import os
+        import tempfile
+        filename = os.path.join(tempfile.gettempdir(), f"inferflux_amd-{os.getuid()}-tunableop.csv")
+    tunable.set_filename(filename)     # choices are kept there and reused by later runs
+
+
+def pause_library_gemm_tuning(paused: bool) -> None:
+    """While paused, shapes already timed keep their chosen kernel and new shapes take the default."""
+    import torch.cuda.tunable as tunable
+    if tunable.is_enabled():
+        tunable.tuning_enable(not paused)
+
+
 def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                 nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
