@@ -85,8 +85,11 @@ def main() -> int:
 
     def decode_rate(batch, steps, warmup):
         """tokens/s and ms/step of ``steps`` decode steps at ``batch`` with contexts from DECODE_KV_START."""
-        eng = make_engine(batch, DECODE_KV_START + steps + warmup + 2)
-        sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
+        # While the last prompts are still coming in, the first requests already decode: give every
+        # request enough tokens (and pages) that none finishes before the timed steps are over.
+        slack = -(-batch * DECODE_KV_START // 16384) + 2
+        eng = make_engine(batch, DECODE_KV_START + steps + warmup + slack + 2)
+        sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + slack + 1, ignore_eos=True)
         for _ in range(batch):
             eng.add_request(torch.randint(0, V, (DECODE_KV_START,), generator=gen).tolist(), SamplingParams(**vars(sp)))
         while any(s.is_prefilling for s in eng.scheduler.running) or eng.scheduler.waiting:
@@ -102,6 +105,7 @@ def main() -> int:
             eng.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
+        assert len(eng.scheduler.running) == batch and eng.stats.preemptions == 0, "a request finished or was preempted while timing"
         kv_mean = DECODE_KV_START + warmup + steps / 2
         del eng
         torch.cuda.empty_cache()

@@ -55,10 +55,50 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __r
   if (threadIdx.x == 0) out[r] = best;
 }
 
-extern "C" int ifx_argmax(const float* logits, int R, int V, int* out, void* stream) {
+// Two stages for wide rows, so that a handful of rows still fills the chip: stage 1 finds the best
+// of each of ARGMAX_SLICES slices of a row, stage 2 the best of those (lowest index on ties in both).
+#define ARGMAX_SLICES 32
+
+__global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits, int V, float* __restrict__ pv,
+                                                            int* __restrict__ pi) {
+  __shared__ float red_v[16];
+  __shared__ int red_i[16];
+  const int r = blockIdx.y, sl = blockIdx.x;
+  const int per = (V + ARGMAX_SLICES - 1) / ARGMAX_SLICES;
+  const int lo = min(V, sl * per), hi = min(V, lo + per);
+  const float* row = logits + (size_t)r * V;
+  int best = hi > lo ? lo + block_argmax(row + lo, hi - lo, red_v, red_i) : V;
+  if (threadIdx.x == 0) {
+    pv[r * ARGMAX_SLICES + sl] = best < V ? row[best] : -INFINITY;
+    pi[r * ARGMAX_SLICES + sl] = best;
+  }
+}
+
+__global__ __launch_bounds__(WAVE) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi, int V,
+                                                           int* __restrict__ out) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  float bv = lane < ARGMAX_SLICES ? pv[r * ARGMAX_SLICES + lane] : -INFINITY;
+  int bi = lane < ARGMAX_SLICES ? pi[r * ARGMAX_SLICES + lane] : V;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, WAVE);
+    const int oi = __shfl_xor(bi, o, WAVE);
+    argmax_merge(bv, bi, ov, oi);
+  }
+  if (lane == 0) out[r] = bi < V ? bi : 0;
+}
+
+// scratch: ARGMAX_SLICES floats and ints per row (used when V is large), or null.
+extern "C" int ifx_argmax(const float* logits, int R, int V, int* out, float* scratch_v, int* scratch_i, void* stream) {
   IFX_REQUIRE(R >= 0 && V > 0, "argmax: bad sizes R=%d V=%d", R, V);
   if (R == 0) return 0;
-  hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, logits, V, out);
+  hipStream_t s = (hipStream_t)stream;
+  if (V >= 16384 && scratch_v && scratch_i && R <= 65535) {
+    hipLaunchKernelGGL(argmax_slices_kernel, dim3(ARGMAX_SLICES, R), dim3(256), 0, s, logits, V, scratch_v, scratch_i);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(WAVE), 0, s, scratch_v, scratch_i, V, out);
+  } else {
+    hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, s, logits, V, out);
+  }
   IFX_LAUNCH_CHECK();
 }
 

@@ -17,12 +17,14 @@ from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
 TILE_ROWS = 64      # rows per tile of the tile kernel
-ROW_CHUNK = 128     # keys per split of the row kernel ...
-ROW_MAX_SPLITS = 64  # ... doubled until a row has at most this many splits
+ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
+ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
+ROW_MAX_SPLITS = 64  # and until a row has at most this many splits
 
 
-def _work_lists(ctx):
-    """What the kernels need beyond the step's own arrays, computed once per step."""
+def _work_lists(ctx, ctx_kv_heads):
+    """What the kernels need beyond the step's own arrays, computed once per step (and per number of
+    kv heads, which decides how many waves a launch has)."""
     q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
     tiled = q_len >= TILE_MIN
     tile_req, tile_q0 = [], []
@@ -40,7 +42,9 @@ def _work_lists(ctx):
             out["rows"] = ctx.upload(rows)
         max_kv = ctx.kv_bound     # not the lengths themselves: see StepContext.kv_bound
         chunk = ROW_CHUNK
-        while -(-max_kv // chunk) > ROW_MAX_SPLITS:
+        n_kv_heads = ctx_kv_heads
+        while (-(-max_kv // chunk) > ROW_MAX_SPLITS
+               or int(rows.size) * n_kv_heads * -(-max_kv // (2 * chunk)) >= ROW_MIN_WAVES):
             chunk *= 2
         out["chunk"], out["max_splits"] = chunk, -(-max_kv // chunk)
     return out
@@ -52,7 +56,8 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     table = ctx.block_table(cache.group)
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
-    w = ctx.derived("attention_work_lists", lambda: _work_lists(ctx))
+    n_kv = cache.k.shape[1]
+    w = ctx.derived(("attention_work_lists", n_kv), lambda: _work_lists(ctx, n_kv))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,

@@ -371,7 +371,10 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _check(logits, "logits", (None, None), torch.float32)
     R, V = logits.shape
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    _call(load_module("sampling"), "ifx_argmax", (P, I, I, P, P), logits.data_ptr(), R, V, out.data_ptr(), _stream())
+    pv = torch.empty((R, 32), dtype=torch.float32, device=logits.device)
+    pi = torch.empty((R, 32), dtype=torch.int32, device=logits.device)
+    _call(load_module("sampling"), "ifx_argmax", (P, I, I, P, P, P, P), logits.data_ptr(), R, V, out.data_ptr(),
+          pv.data_ptr(), pi.data_ptr(), _stream())
     return out
 
 
