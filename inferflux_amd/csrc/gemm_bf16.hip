@@ -170,3 +170,178 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
 #undef CASE
   IFX_FAIL("skinny_gemm: no kernel for m-tiles=%d n-tiles=%d unroll=%d", mt, nt, unroll);
 }
+
+
+// =======================================================================================
+// The same product for up to 64 rows with x staged in LDS.
+//
+// A workgroup of 4 waves owns 64 weight rows (one 16-row tile per wave) and one slice of K.  The
+// rows of x that belong to the current 128-wide piece of K are copied to LDS once and read from
+// there by all four waves, so x crosses the L2 once per 64 weight rows instead of once per 16;
+// at 64 rows of x that is the difference between x traffic of four times the weights and x
+// traffic equal to the weights.  The weight stream is as above: 32 contiguous bytes per lane per
+// 64 k-values, U pieces in flight.  With more than one slice of K, slices write float partial
+// sums that a second kernel adds in slice order (a fixed order: the result does not depend on
+// timing).
+// =======================================================================================
+#define KC 128
+#define XPAD 8
+
+template <int MT, int U, typename TO, int EPI>
+__global__ __launch_bounds__(256) void staged_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                                                          TO* __restrict__ out, float* __restrict__ part, int M, int N,
+                                                          int K, int chunks_per_slice) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][KC + XPAD];
+  const int tid = threadIdx.x, wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g = lane >> 4;
+  const int n_base = blockIdx.x * 64 + 16 * wid;
+  const int n_chunks = (K + KC - 1) / KC;
+  const int c_begin = blockIdx.y * chunks_per_slice, n = min(n_chunks, c_begin + chunks_per_slice) - c_begin;
+  const bf16_t* wrow = W + (size_t)min(n_base + col, N - 1) * K;  // rows past N are read again, never stored
+  floatx4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 wreg[U][4], xr[MT];
+
+  auto load_w = [&](int c, bf16x8* w) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {  // q = 2 * (64-block of the piece) + (half of the lane's 16 values)
+      const int k = c * KC + (q >> 1) * 64 + 16 * g + 8 * (q & 1);
+      w[q] = k < K ? *(const bf16x8*)(wrow + k) : zero8();
+    }
+  };
+  auto load_x = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int p = tid + 256 * i, row = p >> 4, k = c * KC + 8 * (p & 15);
+      xr[i] = (row < M && k < K) ? *(const bf16x8*)(x + (size_t)row * K + k) : zero8();
+    }
+  };
+  auto store_x = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int p = tid + 256 * i;
+      *(bf16x8*)&xs[buf][p >> 4][8 * (p & 15)] = xr[i];
+    }
+  };
+
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (u < n) load_w(c_begin + u, wreg[u]);
+  if (n > 0) {
+    load_x(c_begin);
+    store_x(0);
+  }
+  __syncthreads();
+  for (int i0 = 0; i0 < n; i0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u;
+      if (i >= n) break;  // the same for every thread
+      if (i + 1 < n) load_x(c_begin + i + 1);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const bf16x8 xb = *(const bf16x8*)&xs[u & 1][16 * mt + col][(q >> 1) * 64 + 16 * g + 8 * (q & 1)];
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wreg[u][q], xb, acc[mt], 0, 0, 0);
+        }
+      if (i + U < n) load_w(c_begin + i + U, wreg[u]);
+      if (i + 1 < n) store_x((u + 1) & 1);
+      __syncthreads();
+    }
+  }
+  // acc[mt][r] = out[m = 16 mt + col][n = n_base + 4 g + r]
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + col;
+    if (m >= M) continue;
+    if (gridDim.y > 1) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int nn = n_base + 4 * g + r;
+        if (nn < N) part[((size_t)blockIdx.y * M + m) * N + nn] = acc[mt][r];
+      }
+    } else if (EPI == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int nn = n_base + 4 * g + r;
+        if (nn < N) out[(size_t)m * N + nn] = from_f<TO>(acc[mt][r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; r += 2) {
+        const int nn = n_base + 4 * g + r;  // even: gate at nn, up at nn + 1
+        const float gt = acc[mt][r], up = acc[mt][r + 1];
+        if (nn + 1 < N) out[(size_t)m * (N / 2) + nn / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+      }
+    }
+  }
+}
+
+template <typename TO>
+__global__ void sum_slices_kernel(const float* __restrict__ part, TO* __restrict__ out, int S, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float a = 0.f;
+  for (int s = 0; s < S; ++s) a += part[(size_t)s * n + i];
+  out[i] = from_f<TO>(a);
+}
+
+template <int MT, int U>
+static int launch_staged(const void* x, const void* W, void* out, int out_dtype, float* part, int M, int N, int K,
+                         int slices, int cps, int epi, hipStream_t s) {
+  const dim3 grid((N + 63) / 64, slices);
+#define GO(TO_, EPI_)                                                                                         \
+  hipLaunchKernelGGL((staged_gemm_kernel<MT, U, TO_, EPI_>), grid, dim3(256), 0, s, (const bf16_t*)x,         \
+                     (const bf16_t*)W, (TO_*)out, part, M, N, K, cps)
+  if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
+  else if (out_dtype == DT_BF16) GO(bf16_t, 1);
+  else if (epi == 0) GO(float, 0);
+  else GO(float, 1);
+#undef GO
+  if (slices > 1) {
+    const size_t n = (size_t)M * N;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out_dtype == DT_BF16) hipLaunchKernelGGL(sum_slices_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, part, (bf16_t*)out, slices, n);
+    else hipLaunchKernelGGL(sum_slices_kernel<float>, dim3(blocks), dim3(256), 0, s, part, (float*)out, slices, n);
+  }
+  IFX_LAUNCH_CHECK();
+}
+
+// Largest number of K slices ifx_staged_gemm will use for a shape: the caller sizes ``part``
+// (slices * M * N floats) by it.
+extern "C" int ifx_staged_gemm_slices(int M, int N, int K, int slices) {
+  const int n_chunks = (K + KC - 1) / KC;
+  if (slices <= 0) {
+    const int groups = (N + 63) / 64;
+    slices = groups >= 512 ? 1 : (1024 + groups - 1) / groups;
+    if (slices > n_chunks / 4) slices = n_chunks / 4;
+  }
+  if (slices < 1) slices = 1;
+  if (slices > n_chunks) slices = n_chunks;
+  const int cps = (n_chunks + slices - 1) / slices;
+  return (n_chunks + cps - 1) / cps;
+}
+
+extern "C" int ifx_staged_gemm(const void* x, const void* W, void* out, int out_dtype, float* part, int M, int N, int K,
+                               int slices, int unroll, int epi, void* stream) {
+  IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "staged_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
+  IFX_REQUIRE(K % 8 == 0, "staged_gemm: K=%d must be a multiple of 8", K);
+  IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "staged_gemm: unknown out dtype %d", out_dtype);
+  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0), "staged_gemm: epilogue %d with N=%d", epi, N);
+  if (M == 0) return 0;
+  const int mt = (M + 15) / 16;
+  const int n_chunks = (K + KC - 1) / KC;
+  if (epi != 0) slices = 1;
+  slices = ifx_staged_gemm_slices(M, N, K, slices);
+  IFX_REQUIRE(slices == 1 || part, "staged_gemm: %d slices of K need a scratch buffer", slices);
+  const int cps = (n_chunks + slices - 1) / slices;
+  if (unroll == 0) unroll = 4;
+  hipStream_t s = (hipStream_t)stream;
+#define CASE(MT_, U_) if (mt == MT_ && unroll == U_) return launch_staged<MT_, U_>(x, W, out, out_dtype, part, M, N, K, slices, cps, epi, s)
+  CASE(1, 4); CASE(2, 4); CASE(3, 4); CASE(4, 4);
+  CASE(1, 2); CASE(2, 2); CASE(3, 2); CASE(4, 2);
+  CASE(1, 6); CASE(2, 6); CASE(3, 6); CASE(4, 6);
+#undef CASE
+  IFX_FAIL("staged_gemm: no kernel for m-tiles=%d unroll=%d", mt, unroll);
+}

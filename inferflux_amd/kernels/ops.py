@@ -245,6 +245,28 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
+def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                slices: int = 0, unroll: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
+    """The same product as skinny_gemm with x staged in LDS and shared by the waves of a workgroup
+    (64 weight rows per workgroup, K cut into ``slices``; 0 lets the kernel choose)."""
+    _check(x, "x", (None, None), torch.bfloat16)
+    M, K = x.shape
+    _check(weight, "weight", (None, K), torch.bfloat16)
+    N = weight.shape[0]
+    if M > SKINNY_MAX_M or K % 8:
+        raise KernelError(f"staged_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
+    if swiglu_pairs and N % 2:
+        raise KernelError("staged_gemm: gate/up pairs need an even number of weight rows")
+    mod = load_module("gemm_bf16")
+    n_slices = 1 if swiglu_pairs else mod.fn("ifx_staged_gemm_slices", (I, I, I, I))(M, N, K, slices)
+    part = torch.empty((n_slices, M, N), dtype=torch.float32, device=x.device) if n_slices > 1 else None
+    out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
+    _call(mod, "ifx_staged_gemm", (P, P, P, I, P, I, I, I, I, I, I, P),
+          x.data_ptr(), weight.data_ptr(), out.data_ptr(), _DT[out_dtype], _ptr(part), M, N, K, slices, unroll,
+          1 if swiglu_pairs else 0, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [M, K] times ``weight`` [N, K] transposed, chosen by the weight's type and by M.
 
@@ -262,25 +284,40 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     _check(weight, "weight", (None, None))
     out_dtype = out_dtype or torch.bfloat16
     M, K = x.shape
-    if _use_skinny(M, weight.shape[0], K):
+    kind = _small_m_kernel(M, weight.shape[0], K)
+    if kind == "skinny":
         return skinny_gemm(x, weight, out_dtype)
+    if kind == "staged":
+        return staged_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
     return torch.matmul(x, weight.t())
 
 
-def _use_skinny(M: int, N: int, K: int) -> bool:
-    # Measured on the 7B shapes: the streaming kernel wins up to 16 rows everywhere and up to 32 rows
-    # on the narrow products; beyond that the library's tiles reuse the rows better.
-    return K % 8 == 0 and (M <= 16 or (M <= 32 and N <= 4096))
+def _small_m_kernel(M: int, N: int, K: int) -> Optional[str]:
+    """Which of the two streaming kernels takes a bfloat16 product of this shape, or None for the
+    library.  Measured on the 7B shapes: streaming wins up to 16 rows everywhere (with x staged in LDS
+    for very tall weights such as the head's) and up to 32 rows on the narrow products; beyond that
+    the library's tiles reuse the rows better."""
+    if K % 8:
+        return None
+    if M <= 16:
+        return "staged" if N >= 65536 else "skinny"
+    if M <= 32 and N <= 4096:
+        return "skinny"
+    return None
 
 
 def linear_swiglu(x: torch.Tensor, weight_pairs: torch.Tensor) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) where ``weight_pairs`` [2I, K] alternates the rows of Wg and Wu.
     For few rows the activation is the product's epilogue; otherwise a second kernel applies it."""
     M, K = x.shape
-    if weight_pairs.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and _use_skinny(M, weight_pairs.shape[0], K):
-        return skinny_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
+    if weight_pairs.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
+        kind = _small_m_kernel(M, weight_pairs.shape[0], K)
+        if kind == "skinny":
+            return skinny_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
+        if kind == "staged":
+            return staged_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
     return swiglu(linear(x, weight_pairs), interleaved=True)
 
 

@@ -400,3 +400,29 @@ def test_linear_swiglu_pairs(M):
     assert got.shape == (M, I) and torch.allclose(got, gt / (1 + torch.exp(-gt)) * up, rtol=2e-2, atol=2e-2)
     got32 = ops.linear_swiglu(x.float().to(DEV), pairs.float().to(DEV)).cpu().double()     # the 32-bit path
     assert torch.allclose(got32, gt / (1 + torch.exp(-gt)) * up, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 33, 64])
+@pytest.mark.parametrize("N,K,slices", [(50, 64, 0), (3, 8, 0), (130, 200, 2), (577, 1000, 0), (4608, 3584, 0), (200, 2104, 5)])
+@pytest.mark.parametrize("out_dtype", [BF16, F32])
+def test_staged_gemm(M, N, K, slices, out_dtype):
+    g = gen(15)
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = torch.randn(N, K, generator=g).to(BF16)
+    want = x.double() @ w.double().t()
+    out = ops.staged_gemm(x.to(DEV), w.to(DEV), out_dtype, slices=slices).cpu().double()
+    t = dict(rtol=1e-2, atol=1e-2 * math.sqrt(K)) if out_dtype == BF16 else dict(rtol=1e-4, atol=1e-4 * math.sqrt(K))
+    assert torch.allclose(out, want, **t), float((out - want).abs().max())
+
+
+def test_staged_gemm_swiglu_pairs_and_unrolls():
+    g = gen(16)
+    I, K = 300, 520
+    x = torch.randn(40, K, generator=g).to(BF16)
+    wg, wu = torch.randn(I, K, generator=g).to(BF16) * 0.1, torch.randn(I, K, generator=g).to(BF16) * 0.1
+    pairs = torch.stack([wg, wu], dim=1).reshape(2 * I, K).contiguous()
+    gt, up = x.double() @ wg.double().t(), x.double() @ wu.double().t()
+    want = gt / (1 + torch.exp(-gt)) * up
+    for unroll in (2, 4, 6):
+        got = ops.staged_gemm(x.to(DEV), pairs.to(DEV), BF16, unroll=unroll, swiglu_pairs=True).cpu().double()
+        assert got.shape == (40, I) and torch.allclose(got, want, rtol=2e-2, atol=2e-2)

@@ -107,7 +107,6 @@ def test_pages_run_out_the_youngest_is_preempted_and_results_do_not_change():
     out = drive(m, s, log=log)
     for i, p in prompts.items():
         assert out[i] == expected(p, 40), i                   # recomputation changes nothing
-    pre = {q.rid: q.preemptions for q in []}
     assert m.free_pages() == [8] and not m.live()
     # the oldest request is never the victim
     m2, s2 = make(pages=8)
