@@ -19,6 +19,17 @@ SHAPE_7B = dict(model_type="qwen2", architectures=["Qwen2ForCausalLM"], vocab_si
                 num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
                 intermediate_size=18944, max_position_embeddings=32768, rope_theta=1000000.0, rms_norm_eps=1e-6,
                 tie_word_embeddings=False, attention_bias=True, use_sliding_window=False, torch_dtype="bfloat16")
+# The two other workloads the family is sized for: many requests of mixed length with chunked
+# prefill beside decoding (3B shape), and long prompts that stress cache capacity and long-context
+# decode attention (14B shape).
+SHAPE_3B = dict(SHAPE_7B, vocab_size=151936, hidden_size=2048, num_hidden_layers=36, num_attention_heads=16,
+                num_key_value_heads=2, intermediate_size=11008, tie_word_embeddings=True)
+SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
+                 intermediate_size=13824, rms_norm_eps=1e-5)
+WORKLOADS = {
+    "mixed3b": dict(shape=SHAPE_3B, name="Qwen2.5-3B shape", requests=64, prompt=(128, 2048), new=256, chunk=512),
+    "long14b": dict(shape=SHAPE_14B, name="Qwen2.5-14B shape", requests=32, prompt=(8192, 8192), new=512, chunk=2048),
+}
 CONTEXT = 4096
 PROMPT = 2048
 DECODE_KV_START = 3072      # mean context of a 2,048-token decode after a 2,048-token prompt
@@ -35,6 +46,8 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
+    ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
+                    help="decode: the headline measurement; mixed3b / long14b: whole workloads through the scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -58,6 +71,8 @@ def main() -> int:
 
     def note(msg):
         print(f"[bench] {msg}", file=sys.stderr, flush=True)
+    if args.workload != "decode":
+        return run_workload(args, WORKLOADS[args.workload])
     shape = dict(SHAPE_7B)
     layers_full = shape["num_hidden_layers"]
     if args.layers:
@@ -155,6 +170,62 @@ def main() -> int:
         b1 = decode_rate(1, min(args.steps, 32), min(args.warmup, 4))[0]
         b64 = decode_rate(64, min(args.steps, 32), min(args.warmup, 4))[0]
         out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def run_workload(args, w) -> int:
+    """A whole workload through the engine: every request added at once, chunked prefill mixed with
+    decoding, greedy sampling.  A step here is one engine step; the value is generated tokens a second."""
+    import torch
+    from inferflux_amd import SamplingParams
+    from inferflux_amd.config import config_from_dict
+    from inferflux_amd.engine.engine import Engine
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.engine.scheduler import SchedulerConfig
+
+    shape = dict(w["shape"])
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(shape)
+    tdt = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    model = Model(cfg).init_random(0, tdt, torch.device("cuda", 0))
+    gen = torch.Generator().manual_seed(2)
+    lo, hi = w["prompt"]
+    lens = torch.randint(lo, hi + 1, (w["requests"],), generator=gen).tolist()
+    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lens]
+    pages = sum(-(-(n + w["new"]) // PAGE) + 1 for n in lens)
+    runner = ModelRunner(model, num_pages=pages, page_size=PAGE, max_requests=w["requests"])
+    eng = Engine(runner, SchedulerConfig(max_batch_size=w["requests"], max_batch_tokens=16384, chunked_prefill_tokens=w["chunk"]))
+    first, t0 = {}, time.perf_counter()
+
+    def on_token(rid, tok):
+        if rid not in first:
+            first[rid] = time.perf_counter() - t0
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=w["new"], ignore_eos=True), on_token)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    n_gen = sum(len(o.token_ids) for o in outs)
+    ttft = sorted(first.values())
+    out = {
+        "metric": f"generated tok/s, {w['requests']} requests, prompts {lo}-{hi}, {w['new']} new tokens each ({w['name']}, {args.dtype}, random weights)",
+        "value": round(n_gen / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": eng.stats.steps, "warmup": 0,
+        "ms_per_step": round(dt / eng.stats.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (uniform random token ids, seeded N(0,0.02) weights)",
+        "config": {"model": w["name"], "global_batch": w["requests"], "seq_len": hi + w["new"], "parallelism": "1 GPU",
+                   "num_hidden_layers": w["shape"]["num_hidden_layers"], "layers_run": cfg.num_hidden_layers,
+                   "hidden_size": cfg.hidden_size, "num_attention_heads": cfg.num_attention_heads,
+                   "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+                   "prompt_tokens": sum(lens), "chunked_prefill_tokens": w["chunk"], "kv_page_size": PAGE, "kv_pages": pages},
+        "total_s": round(dt, 2), "prompt_tok_per_s_overall": round(sum(lens) / dt, 1),
+        "ttft_s": {"min": round(ttft[0], 3), "median": round(ttft[len(ttft) // 2], 3), "max": round(ttft[-1], 3)},
+        "preemptions": eng.stats.preemptions,
+    }
     print(json.dumps(out), flush=True)
     return 0
 
