@@ -392,6 +392,64 @@ __device__ __forceinline__ void stage_tile(const TileRegs& r, bf16_t* k_s, bf16_
   }
 }
 
+// One staged tile of 64 keys against a wave's 16 query rows: scores, running softmax, output.
+// Scores stay unscaled; the scale (with log2 e) enters the exponent through one fused multiply-add.
+// MASKED adds the causal / window / row-validity test per score.
+template <bool MASKED>
+__device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, const bf16x8* qop, floatx4* o, float& m,
+                                          float& l, float c_log2e, int j0, int my_pos, int my_lo, bool q_ok, int col, int g4) {
+  floatx4 s[4];
+  float mb = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = 32 * ks + 8 * g4;
+      const bf16x8 kop = c < D ? *(const bf16x8*)(k_s + (16 * t + col) * KPAD + c) : zero8();
+      s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[ks], s[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (MASKED) {
+        const int key = j0 + 16 * t + 4 * g4 + r;
+        const bool vis = q_ok && key <= my_pos && key >= my_lo;
+        s[t][r] = vis ? s[t][r] : -INFINITY;
+      }
+      mb = fmaxf(mb, s[t][r]);
+    }
+  }
+  const float m_new = fmaxf(m, col_max(mb));
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = fast_exp2((m - m_safe) * c_log2e);
+  const float ms = m_safe * c_log2e;
+  float psum = 0.f;
+  bf16x4 pb[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float p = fast_exp2(fmaf(s[t][r], c_log2e, -ms));
+      psum += p;
+      pb[t][r] = (__bf16)p;
+    }
+  l = l * alpha + psum;
+  m = m_new;
+  const bf16x8 pop0 = join4(pb[0], pb[1]), pop1 = join4(pb[2], pb[3]);
+  const bool rescale = __any(alpha != 1.0f);   // once the running maxima have settled nothing is rescaled
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 8 * g4;
+    const bf16x8 vop0 = *(const bf16x8*)(vr), vop1 = *(const bf16x8*)(vr + 32);
+    if (rescale) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+    }
+    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop0, o[dt], 0, 0, 0);
+    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop1, o[dt], 0, 0, 0);
+  }
+}
+
 __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t k_s[TK * KPAD];
   __shared__ __attribute__((aligned(16))) bf16_t v_s[D * VPAD];
@@ -420,6 +478,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
   const int my_lo = a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
   const size_t my_row = (size_t)a.q_start[req] + my_q;
   // the keys this wave's 16 rows can see at all: tiles outside are skipped by the whole wave
+  const int wave_first = pos_first + 16 * wid;
   const int wave_hi = min(pos_last, pos_first + 16 * wid + 15);
   const int wave_lo = a.window > 0 ? max(0, pos_first + 16 * wid - a.window + 1) : 0;
   bf16x8 qop[KS];
@@ -449,53 +508,10 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
     }
     if (j0 > wave_hi || j0 + TK <= wave_lo) continue;   // uniform over the wave; barriers are at the loop's top
 
-    floatx4 s[4];
-    float mb = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int c = 32 * ks + 8 * g4;
-        const bf16x8 kop = c < D ? *(const bf16x8*)(k_s + (16 * t + col) * KPAD + c) : zero8();
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[ks], s[t], 0, 0, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = j0 + 16 * t + 4 * g4 + r;
-        const bool vis = q_ok && key <= my_pos && key >= my_lo;
-        s[t][r] = vis ? s[t][r] * a.scale_log2e : -INFINITY;
-        mb = fmaxf(mb, s[t][r]);
-      }
-    }
-    const float m_new = fmaxf(m, col_max(mb));
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m - m_safe);
-    float psum = 0.f;
-    bf16x4 pb[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = fast_exp2(s[t][r] - m_safe);
-        psum += p;
-        pb[t][r] = (__bf16)p;
-      }
-    l = l * alpha + psum;
-    m = m_new;
-    const bf16x8 pop0 = join4(pb[0], pb[1]), pop1 = join4(pb[2], pb[3]);
-    const bool rescale = __any(alpha != 1.0f);   // once the running maxima have settled nothing is rescaled
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 8 * g4;
-      const bf16x8 vop0 = *(const bf16x8*)(vr), vop1 = *(const bf16x8*)(vr + 32);
-      if (rescale) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
-      }
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop0, o[dt], 0, 0, 0);
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop1, o[dt], 0, 0, 0);
-    }
+    // A tile every key of which every row of this wave sees needs no mask: the common case.
+    const bool full = j0 + TK - 1 <= wave_first && (a.window <= 0 || j0 >= wave_hi - a.window + 1);
+    if (full) tile_math<false>(k_s, v_s, qop, o, m, l, a.scale_log2e, j0, my_pos, my_lo, q_ok, col, g4);
+    else tile_math<true>(k_s, v_s, qop, o, m, l, a.scale_log2e, j0, my_pos, my_lo, q_ok, col, g4);
   }
   l = col_sum(l);
   if (q_ok) {

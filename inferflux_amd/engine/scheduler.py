@@ -43,7 +43,7 @@ class RequestRefused(ValueError):
     pass
 
 
-@dataclasses.dataclass
+@dataclasses.dataclass(eq=False)     # requests are compared by identity (they sit in lists and deques)
 class Sequence_:
     """A request as the scheduler sees it.
 
