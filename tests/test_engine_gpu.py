@@ -245,3 +245,92 @@ def test_replayed_decode_graphs_equal_eager_steps(name, dtype, sharp_folders):
     assert replays > 60 and len(graphed._graphs) >= 4
     want = plain_logits(folder, seqs["a"][: pos["a"]])[-1]
     assert rel_err(got[0], want) < REL_TOL[dtype]
+
+
+# ---- other toy parts: a position encoding of its own, a feed-forward with routing --------------------
+def test_toy_position_encoding_and_routed_feed_forward(tmp_path):
+    """Two more parts defined here and registered from outside the package: a position encoding that
+    transforms q and k itself (through ``apply``, not the fused rotary kernel) and a feed-forward that
+    routes each row to one of two experts.  A model built from them must agree with a plain
+    computation of the same formulas and must not depend on the cutting."""
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.parts import (FeedForward, LayerSpec, ModelPlan, ParamSpec, PartSpec, PositionEncoding,
+                                     ScheduleEntry, register_part)
+
+    H, V, nH, d = 32, 40, 2, 16
+
+    @register_part("position", "toy_decay_scale")
+    class DecayScale(PositionEncoding):
+        """q is scaled by 1 + pos/100 and k by 1/(1 + pos/50): scores then depend on both positions."""
+        needs_apply = True
+        def __init__(self, head_dim):
+            self.head_dim = head_dim
+        def apply(self, q, k, positions):
+            p = positions.to(torch.float32)[:, None, None]
+            q = (q.float() * (1 + p / 100)).to(q.dtype)
+            if k is not None:
+                k = (k.float() / (1 + p / 50)).to(k.dtype)
+            return q, k
+
+    @register_part("ffn", "toy_two_experts")
+    class TwoExperts(FeedForward):
+        def __init__(self, name, hidden_size):
+            self.name, self.H = name, hidden_size
+        def param_specs(self):
+            return {f"{self.name}.router.weight": ParamSpec((2, self.H), ("normal", 1.0)),
+                    f"{self.name}.experts.0.weight": ParamSpec((self.H, self.H), ("normal", 0.2)),
+                    f"{self.name}.experts.1.weight": ParamSpec((self.H, self.H), ("normal", 0.2))}
+        def load(self, tensors):
+            self.router = tensors[f"{self.name}.router.weight"]
+            self.experts = [tensors[f"{self.name}.experts.{e}.weight"] for e in (0, 1)]
+        def forward(self, h, ctx):
+            choice = (h.float() @ self.router.float().t()).argmax(-1)          # router logits in 32-bit
+            out = torch.zeros_like(h)
+            for e in (0, 1):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    out[rows] = torch.tanh(h[rows] @ self.experts[e].t())
+            return out
+
+    p = "toy.layers.0"
+    layer = LayerSpec(p, PartSpec("prenorm"), PartSpec("rmsnorm", {"name": f"{p}.n1", "eps": 1e-5}),
+                      PartSpec("paged_attention", {"name": f"{p}.attn", "n_heads": nH, "n_kv_heads": 1, "head_dim": d,
+                                                   "bias": True, "position": PartSpec("toy_decay_scale", {"head_dim": d})}),
+                      PartSpec("rmsnorm", {"name": f"{p}.n2", "eps": 1e-5}),
+                      PartSpec("toy_two_experts", {"name": f"{p}.moe"}))
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=128,
+                     embedding=PartSpec("token_embedding", {"name": "toy.embed", "vocab_size": V}),
+                     layers=(layer,), schedule=(ScheduleEntry(0),),
+                     final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
+    model = Model(plan=plan).init_random(5, torch.float32, "cuda")
+    assert not model.graph_safe                                         # parts from outside are not replayed as graphs
+    runner = ModelRunner(model, num_pages=16, max_requests=2)
+    assert not runner.decode_graphs
+    ids = seeded_ids(16, 50, V)
+    runner.add_request("w")
+    whole = runner.step([StepEntry("w", ids, list(range(50)))]).cpu()
+    runner.free_request("w")
+    runner.add_request("c")
+    rows, q = [], 0
+    for mlen in (9, 1, 1, 20, 2, 17):
+        rows.append(runner.step([StepEntry("c", ids[q:q + mlen], list(range(mlen)))]).cpu()); q += mlen
+    assert torch.allclose(torch.cat(rows), whole, rtol=1e-4, atol=1e-5)
+
+    # the same formulas, plainly, from the model's own tensors
+    att, moe = model.blocks[0].mixer, model.blocks[0].ffn
+    x = model.embedding.table.double().cpu()[ids]
+    pos = torch.arange(50, dtype=torch.float64)
+    h = pm.rms_norm(x, model.blocks[0].norm_in.weight.double().cpu(), 1e-5)
+    qkv = h @ att.w_qkv.double().cpu().t() + att.b_qkv.double().cpu()
+    qq = qkv[:, : nH * d].view(50, nH, d) * (1 + pos / 100)[:, None, None]
+    kk = qkv[:, nH * d: (nH + 1) * d].view(50, 1, d) / (1 + pos / 50)[:, None, None]
+    vv = qkv[:, (nH + 1) * d:].view(50, 1, d)
+    x = x + pm.attention(qq, kk, vv).reshape(50, nH * d) @ att.w_o.double().cpu().t()
+    h = pm.rms_norm(x, model.blocks[0].norm_post.weight.double().cpu(), 1e-5)
+    choice = (h @ moe.router.double().cpu().t()).argmax(-1)
+    y = torch.stack([torch.tanh(h[i] @ moe.experts[int(choice[i])].double().cpu().t()) for i in range(50)])
+    x = x + y
+    want = pm.rms_norm(x, model.final_norm.weight.double().cpu(), 1e-5) @ model.head.weight.double().cpu().t()
+    assert torch.allclose(whole.double(), want, rtol=1e-3, atol=1e-4)
