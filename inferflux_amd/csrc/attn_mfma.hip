@@ -167,7 +167,7 @@ __device__ __forceinline__ void use_row_block(const RowBlock& b, const RowArgs& 
   }
 }
 
-__global__ __launch_bounds__(WAVE) void attn_rows_kernel(RowArgs a) {
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_rows_kernel(RowArgs a) {
   const int split = blockIdx.x, kvh = blockIdx.y, ri = blockIdx.z;
   const int lane = threadIdx.x, col = lane & 15, g4 = lane >> 4;
   const int row = a.rows ? a.rows[ri] : ri;
@@ -450,7 +450,9 @@ __device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, 
   }
 }
 
-__global__ __launch_bounds__(256) void attn_tiles_kernel(TileArgs a) {
+// Three waves per SIMD: the kernel waits on LDS and on the matrix pipe, so one more wave to switch to
+// is worth more than the registers it costs (the compiler fits 162 without spilling).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_tiles_kernel(TileArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t k_s[TK * KPAD];
   __shared__ __attribute__((aligned(16))) bf16_t v_s[D * VPAD];
   const int tid = threadIdx.x, wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g4 = lane >> 4;
