@@ -1,6 +1,8 @@
 """Loading a model folder into a runner: the one path every entry point takes."""
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from ..config.registry import load_config
@@ -25,7 +27,34 @@ def load_model(folder: str, dtype: torch.dtype = torch.bfloat16, device=None) ->
     return Model(config).load_folder(folder, dtype, device)
 
 
-def load_runner(folder: str, dtype: torch.dtype = torch.bfloat16, num_pages: int = 256, page_size: int = 16,
-                max_requests: int = 64, device=None) -> ModelRunner:
-    return ModelRunner(load_model(folder, dtype, device), num_pages=num_pages, page_size=page_size,
-                       max_requests=max_requests)
+def plan_kv_pages(model: Model, page_size: int, wanted_tokens: int, memory_fraction: float = 0.8) -> int:
+    """Pages for ``wanted_tokens`` of cache, cut down to what ``memory_fraction`` of the free device
+    memory holds.  bytes per token = 2 * sum over caching layers of kv heads * head size * element
+    size, the reference's planner's arithmetic (runtime/backends/cuda/native/kv_cache_planner.h:22-37),
+    which gives the cache 20 % of free memory (native_bootstrap_config.h:20); here the weights are
+    already resident when this is called, so most of what is left can go to the cache."""
+    per_token = 0
+    esz = 2 if model.dtype == torch.bfloat16 else 4
+    for e, mixer in zip(model.plan.schedule, model.schedule_mixers()):
+        spec = mixer.cache_spec()
+        if spec is not None and e.cache_from is None:
+            per_token += 2 * spec.n_kv_heads * spec.head_dim * esz
+    want = max(1, -(-wanted_tokens // page_size))
+    if per_token == 0:
+        return want
+    free, _ = torch.cuda.mem_get_info(model.device)
+    fit = int(free * memory_fraction) // (per_token * page_size)
+    if fit < 1:
+        raise RuntimeError(f"no device memory left for the cache ({free} bytes free, a page needs {per_token * page_size})")
+    return min(want, fit)
+
+
+def load_runner(folder: str, dtype: torch.dtype = torch.bfloat16, num_pages: Optional[int] = 256, page_size: int = 16,
+                max_requests: int = 64, device=None, cache_tokens: Optional[int] = None,
+                phase_timing: bool = False) -> ModelRunner:
+    """``num_pages`` None: as many pages as ``cache_tokens`` need, within the free device memory."""
+    model = load_model(folder, dtype, device)
+    if num_pages is None:
+        num_pages = plan_kv_pages(model, page_size, cache_tokens or 4096 * max_requests)
+    return ModelRunner(model, num_pages=num_pages, page_size=page_size, max_requests=max_requests,
+                       phase_timing=phase_timing)

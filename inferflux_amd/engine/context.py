@@ -38,6 +38,7 @@ class StepContext:
     def __init__(self, entries: Sequence[StepEntry], manager, act_dtype: torch.dtype, device,
                  width_multiple: int = 8, slab: torch.Tensor = None, pinned: torch.Tensor = None, upload: bool = True):
         self.act_dtype, self.device = act_dtype, device
+        self.timer = None              # a tracing.PhaseTimer while per-phase timing is on
         self.entries = list(entries)
         R = self.n_requests = len(self.entries)
         P = manager.page_size

@@ -90,11 +90,28 @@ class Model:
     # ---- forward ------------------------------------------------------------------
     def forward(self, ctx, storage) -> torch.Tensor:
         """float32 logits [len(ctx.logit_rows), vocab] for the step ``ctx`` describes."""
+        t = ctx.timer
+        if t is not None:
+            t.begin()
+            t.enter("embed")
         residual = self.embedding.forward(ctx.token_ids)
+        if t is not None:
+            t.mark("embed")
         pending = None
         for i, e in enumerate(self.plan.schedule):
             residual, pending = self.blocks[e.layer].forward(residual, pending, ctx, storage.binding(i))
         if ctx.n_logit_rows == 0:
-            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=residual.device)
-        h = self.final_norm.forward(residual, pending, ctx.act_dtype, rows=ctx.logit_rows)
-        return self.head.forward(h)
+            logits = torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=residual.device)
+        else:
+            if t is not None:
+                t.enter("final_norm")
+            h = self.final_norm.forward(residual, pending, ctx.act_dtype, rows=ctx.logit_rows)
+            if t is not None:
+                t.mark("final_norm")
+                t.enter("lm_head")
+            logits = self.head.forward(h)
+            if t is not None:
+                t.mark("lm_head")
+        if t is not None:
+            t.end(len(self.plan.schedule), ctx.n_tokens)
+        return logits

@@ -13,6 +13,7 @@ raises before it touches the cache.
 """
 from __future__ import annotations
 
+import os
 from typing import Hashable, List, Optional, Sequence
 
 import torch
@@ -41,7 +42,7 @@ class ModelRunner:
     MAX_GRAPHS = 12
 
     def __init__(self, model: Model, num_pages: int, page_size: int = 16, max_requests: int = 64,
-                 decode_graphs: bool = True):
+                 decode_graphs: bool = True, phase_timing: bool = False):
         if model.device is None:
             raise ValueError("the model has no weights yet (load_folder / init_random first)")
         if model.device.type != "cuda":
@@ -58,7 +59,11 @@ class ModelRunner:
         # (batch size, wanted rows, block-table width), and replayed: a decode step is some 250
         # launches, which the host cannot issue as fast as the GPU runs them.  The reference does the
         # same per batch size (runtime/backends/cuda/native/transformer_forward.cu:3068-3117).
-        self.decode_graphs = decode_graphs and model.graph_safe
+        self.timer = None
+        if phase_timing or os.environ.get("INFERFLUX_PHASE_TIMING", "") == "1":
+            from .tracing import PhaseTimer
+            self.timer = PhaseTimer()
+        self.decode_graphs = decode_graphs and model.graph_safe and self.timer is None
         self._graphs = {}
 
     # ---- requests -----------------------------------------------------------------
@@ -115,6 +120,7 @@ class ModelRunner:
             logits = self._decode_step(entries)
         else:
             ctx = StepContext(entries, self.manager, self.dtype, self.device)
+            ctx.timer = self.timer
             logits = self.model.forward(ctx, self.storage)
         for rid, n in needs:
             self.manager.commit(rid, n)

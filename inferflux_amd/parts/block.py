@@ -27,7 +27,14 @@ class PreNormBlock(Block):
         return (self.norm_in, self.mixer, self.norm_post, self.ffn)
 
     def forward(self, residual, pending, ctx, binding: MixerBinding):
-        h = self.norm_in.forward(residual, pending, ctx.act_dtype)
-        delta = self.mixer.forward(h, ctx, binding)
-        h = self.norm_post.forward(residual, delta, ctx.act_dtype)
-        return residual, self.ffn.forward(h, ctx)
+        t = ctx.timer
+        if t is None:
+            h = self.norm_in.forward(residual, pending, ctx.act_dtype)
+            delta = self.mixer.forward(h, ctx, binding)
+            h = self.norm_post.forward(residual, delta, ctx.act_dtype)
+            return residual, self.ffn.forward(h, ctx)
+        t.enter("norm"); h = self.norm_in.forward(residual, pending, ctx.act_dtype); t.mark("norm")
+        t.enter("mixer"); delta = self.mixer.forward(h, ctx, binding); t.mark("mixer")
+        t.enter("norm"); h = self.norm_post.forward(residual, delta, ctx.act_dtype); t.mark("norm")
+        t.enter("ffn"); out = self.ffn.forward(h, ctx); t.mark("ffn")
+        return residual, out

@@ -117,3 +117,18 @@ def test_command_line(model_folders):
     assert [l["token"] for l in lines if "token" in l] == want           # streamed one by one
     final = [l for l in lines if "token_ids" in l][0]
     assert final["token_ids"] == want and final["finish_reason"] == "length" and final["prompt_tokens"] == 11
+
+
+def test_phase_timing_and_cache_planning(model_folders, capfd):
+    folder = model_folders["C"]
+    prompt = seeded_ids(97, 20, 777)
+    plain = Engine.load(folder, dtype="float32", kv_pages=32, max_batch_size=2)
+    want = plain.generate([prompt], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0].token_ids
+    timed = Engine.load(folder, dtype="float32", max_batch_size=2, ctx_size=256, phase_timing=True)   # cache sized by the planner
+    assert [p.num_pages for p in timed.runner.manager.pools] == [32, 32] and not timed.runner.decode_graphs
+    got = timed.generate([prompt], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0].token_ids
+    assert got == want
+    err = capfd.readouterr().err
+    assert "[phase_timing] #1 L=4 tokens=20" in err and "mixer=" in err and "lm_head=" in err
+    t = timed.runner.timer
+    assert t.forwards == 5 and all(t.totals[k] > 0 for k in ("embed", "norm", "mixer", "ffn", "final_norm", "lm_head"))
