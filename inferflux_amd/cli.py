@@ -60,7 +60,7 @@ def cmd_completion(args) -> int:
                             frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
                             repetition_penalty=args.repetition_penalty, penalty_last_n=args.penalty_last_n,
                             seed=args.seed if args.seed is not None else 0xFFFFFFFF, max_tokens=args.max_tokens,
-                            ignore_eos=args.ignore_eos)
+                            ignore_eos=args.ignore_eos, logprobs=args.top_n)
     tok = _tokenizer(args.model)
 
     def on_token(rid, t):
@@ -71,6 +71,9 @@ def cmd_completion(args) -> int:
     for o in outs:
         rec = {"model": args.model, "request": o.request_id, "prompt_tokens": len(o.prompt_token_ids),
                "completion_tokens": len(o.token_ids), "token_ids": o.token_ids, "finish_reason": o.finish_reason}
+        if o.logprobs is not None:
+            rec["logprobs"] = [{"token": l.token_id, "logprob": round(l.logprob, 6),
+                                "top_logprobs": [[t, round(v, 6)] for t, v in l.top_logprobs]} for l in o.logprobs]
         if tok:
             rec["completion"] = tok.decode(o.token_ids)
         print(json.dumps(rec), flush=True)
@@ -126,6 +129,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     c.add_argument("--penalty-last-n", type=int, default=64)
     c.add_argument("--seed", type=int, default=None)
     c.add_argument("--ignore-eos", action="store_true")
+    c.add_argument("--top-n", type=int, default=None,
+                   help="report each token's log-probability with the N most probable alternatives (0: the token's only)")
     c.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     c.add_argument("--ctx-size", type=int, default=4096, help="tokens of context per sequence the cache is sized for")
     c.add_argument("--batch-size", type=int, default=16384, help="most tokens in one step (max_batch_tokens)")

@@ -300,3 +300,67 @@ extern "C" int ifx_sample(const float* logits, float* weights, const float* temp
   hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, a);
   IFX_LAUNCH_CHECK();
 }
+
+
+// ---------------------------------------------------------------------------------------
+// Log-probabilities for reporting: lp[r] = logits[r, chosen[r]] - logsumexp(logits[r]) (the
+// log-softmax the reference reports per sampled token, runtime/logprob.h:11-18), and the top_n
+// most probable tokens of the row with theirs, in descending order (lowest index first among
+// equals).  The k-th is found as the largest element that comes after the (k-1)-th in that
+// order, so the logits are not modified.
+#define MAX_TOP_LOGPROBS 20
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void logprobs_kernel(const float* __restrict__ logits, const int* __restrict__ chosen,
+                                                                 int V, int top_n, float* __restrict__ lp,
+                                                                 int* __restrict__ top_ids, float* __restrict__ top_lp) {
+  __shared__ float red_f[16];
+  __shared__ float red_v[16];
+  __shared__ int red_i[16];
+  const int r = blockIdx.x;
+  const float* row = logits + (size_t)r * V;
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i]);
+  mx = block_max(mx, red_f);
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) sum += expf(row[i] - mx);
+  sum = block_sum(sum, red_f);
+  const float lse = mx + logf(sum);
+  if (threadIdx.x == 0) lp[r] = row[chosen[r]] - lse;
+  float last_v = INFINITY;
+  int last_i = -1;
+  for (int k = 0; k < top_n; ++k) {
+    float bv = -INFINITY;
+    int bi = V;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      const float x = row[i];
+      const bool after = x < last_v || (x == last_v && i > last_i);   // not yet reported
+      if (after && (x > bv || (x == bv && i < bi))) { bv = x; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, WAVE);
+      const int oi = __shfl_xor(bi, o, WAVE);
+      argmax_merge(bv, bi, ov, oi);
+    }
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, nw = blockDim.x / WAVE;
+    __syncthreads();
+    if (lane == 0) { red_v[wid] = bv; red_i[wid] = bi; }
+    __syncthreads();
+    bv = red_v[0]; bi = red_i[0];
+    for (int w = 1; w < nw; ++w) argmax_merge(bv, bi, red_v[w], red_i[w]);
+    if (threadIdx.x == 0) {
+      top_ids[r * top_n + k] = bi < V ? bi : -1;
+      top_lp[r * top_n + k] = bi < V ? bv - lse : -INFINITY;
+    }
+    last_v = bv; last_i = bi;
+  }
+}
+
+extern "C" int ifx_logprobs(const float* logits, const int* chosen, int R, int V, int top_n, float* lp, int* top_ids,
+                            float* top_lp, void* stream) {
+  IFX_REQUIRE(R >= 0 && V > 0 && top_n >= 0 && top_n <= MAX_TOP_LOGPROBS, "logprobs: bad sizes R=%d V=%d top_n=%d (at most %d)", R, V, top_n, MAX_TOP_LOGPROBS);
+  if (R == 0) return 0;
+  hipLaunchKernelGGL(logprobs_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, logits, chosen, V, top_n, lp,
+                     top_ids, top_lp);
+  IFX_LAUNCH_CHECK();
+}

@@ -31,6 +31,7 @@ class RequestOutput:
     token_ids: List[int]
     finish_reason: Optional[str] = None      # "stop" (eos or a stop token), "length", "abort"; None while running
     preemptions: int = 0
+    logprobs: Optional[List] = None          # one sampler.TokenLogprob per generated token, when asked for
 
     @property
     def finished(self) -> bool:
@@ -148,7 +149,8 @@ class Engine:
             if reason is not None:
                 self.scheduler.finish(i.seq)
                 del self._live[i.seq.rid]
-                done.append(RequestOutput(i.seq.rid, live.prompt, list(i.seq.generated), reason, i.seq.preemptions))
+                done.append(RequestOutput(i.seq.rid, live.prompt, list(i.seq.generated), reason, i.seq.preemptions,
+                                          list(live.sampling.logprobs) if live.params.logprobs is not None else None))
         return done
 
     def generate(self, prompts: Sequence[Sequence[int]], params=None,

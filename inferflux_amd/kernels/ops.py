@@ -455,3 +455,17 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
           logits.data_ptr(), weights.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
           min_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), R, V, _stream())
     return out
+
+
+def logprobs(logits: torch.Tensor, chosen: torch.Tensor, top_n: int):
+    """log-softmax of the chosen token of each row and the row's ``top_n`` (<= 20) most probable tokens:
+    (lp [R], top_ids [R, top_n] int32, top_lp [R, top_n]), descending, lowest index first among equals."""
+    _check(logits, "logits", (None, None), torch.float32)
+    R, V = logits.shape
+    _check(chosen, "chosen", (R,), torch.int32)
+    lp = torch.empty((R,), dtype=torch.float32, device=logits.device)
+    top_ids = torch.empty((R, top_n), dtype=torch.int32, device=logits.device)
+    top_lp = torch.empty((R, top_n), dtype=torch.float32, device=logits.device)
+    _call(load_module("sampling"), "ifx_logprobs", (P, P, I, I, I, P, P, P, P),
+          logits.data_ptr(), chosen.data_ptr(), R, V, top_n, lp.data_ptr(), top_ids.data_ptr(), top_lp.data_ptr(), _stream())
+    return lp, top_ids, top_lp

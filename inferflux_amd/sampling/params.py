@@ -36,6 +36,9 @@ class SamplingParams:
     max_tokens: int = 16
     stop_token_ids: Sequence[int] = ()
     ignore_eos: bool = False
+    # None: no log-probabilities; 0: the sampled token's; N (at most 20): with the N most probable
+    # alternatives (the reference's collect_logprobs / logprob_top_n, scheduler/request_batch.h:258-265)
+    logprobs: Optional[int] = None
 
     def validate(self) -> None:
         if self.temperature < 0:
@@ -48,6 +51,8 @@ class SamplingParams:
             raise ValueError("repetition_penalty must be positive (1.0 = off)")
         if self.penalty_last_n < 0 or self.max_tokens < 1:
             raise ValueError("penalty_last_n must be >= 0 and max_tokens >= 1")
+        if self.logprobs is not None and not (0 <= self.logprobs <= 20):
+            raise ValueError("logprobs must be None or between 0 and 20")
 
     @property
     def greedy(self) -> bool:

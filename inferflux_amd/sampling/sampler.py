@@ -18,12 +18,23 @@ from .params import UNSEEDED, SamplingParams, fresh_seed, philox_uniform
 
 
 @dataclasses.dataclass
+class TokenLogprob:
+    """The sampled token's log-probability (log-softmax of the logits after penalties and bias, before
+    temperature) and the most probable alternatives [(token id, log-probability)], as the reference
+    reports them (runtime/logprob.h:11-18; token ids here, the engine has no text)."""
+    token_id: int
+    logprob: float
+    top_logprobs: List = dataclasses.field(default_factory=list)
+
+
+@dataclasses.dataclass
 class SamplingState:
     """What sampling remembers of a request between steps."""
     params: SamplingParams
     seed: int = 0
     draws: int = 0                      # stochastic draws so far: the generator's counter
     history: List[int] = dataclasses.field(default_factory=list)   # sampled tokens, oldest first
+    logprobs: List[TokenLogprob] = dataclasses.field(default_factory=list)
 
     @classmethod
     def start(cls, params: SamplingParams) -> "SamplingState":
@@ -71,15 +82,24 @@ class Sampler:
         if brow:
             ops.add_logit_bias(logits, self._dev(brow, torch.int32), self._dev(bid, torch.int32), self._dev(bval, torch.float32))
         if all(s.params.greedy for s in states):
-            tokens = ops.argmax(logits).cpu().tolist()
+            chosen = ops.argmax(logits)
         else:
             u = philox_uniform(np.array([s.seed for s in states]), np.array([s.draws for s in states]))
-            tokens = ops.sample(logits,
+            chosen = ops.sample(logits,
                                 self._dev([s.params.temperature for s in states], torch.float32),
                                 self._dev([s.params.top_k for s in states], torch.int32),
                                 self._dev([s.params.top_p for s in states], torch.float32),
                                 self._dev([s.params.min_p for s in states], torch.float32),
-                                torch.from_numpy(u).to(self.device)).cpu().tolist()
+                                torch.from_numpy(u).to(self.device))
+        top_n = max((s.params.logprobs for s in states if s.params.logprobs is not None), default=None)
+        if top_n is not None:
+            lp, top_ids, top_lp = (t.cpu() for t in ops.logprobs(logits, chosen, top_n))
+        tokens = chosen.cpu().tolist()
+        for r, (st, t) in enumerate(zip(states, tokens)):
+            if st.params.logprobs is not None:
+                n = st.params.logprobs
+                st.logprobs.append(TokenLogprob(int(t), float(lp[r]),
+                                                list(zip(top_ids[r, :n].tolist(), top_lp[r, :n].tolist()))))
         for st, t in zip(states, tokens):
             if not st.params.greedy:
                 st.draws += 1

@@ -132,3 +132,18 @@ def test_phase_timing_and_cache_planning(model_folders, capfd):
     assert "[phase_timing] #1 L=4 tokens=20" in err and "mixer=" in err and "lm_head=" in err
     t = timed.runner.timer
     assert t.forwards == 5 and all(t.totals[k] > 0 for k in ("embed", "norm", "mixer", "ffn", "final_norm", "lm_head"))
+
+
+def test_logprobs_through_the_engine(model_folders):
+    folder = model_folders["A"]
+    cfg, W = pm.load_folder(folder, torch.float64)
+    prompt = seeded_ids(98, 10, 512)
+    engine = Engine.load(folder, dtype="float32", kv_pages=16)
+    out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, logprobs=3))[0]
+    assert len(out.logprobs) == 6 and [l.token_id for l in out.logprobs] == out.token_ids
+    for step, l in enumerate(out.logprobs):
+        want = torch.log_softmax(pm.forward(cfg, W, prompt + out.token_ids[:step])[-1], -1)
+        assert abs(l.logprob - float(want[l.token_id])) < 1e-4
+        assert l.top_logprobs[0][0] == l.token_id and len(l.top_logprobs) == 3          # greedy: the sampled token is the top one
+        assert all(abs(v - float(want[t])) < 1e-4 for t, v in l.top_logprobs)
+    assert engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))[0].logprobs is None

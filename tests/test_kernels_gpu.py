@@ -426,3 +426,20 @@ def test_staged_gemm_swiglu_pairs_and_unrolls():
     for unroll in (2, 4, 6):
         got = ops.staged_gemm(x.to(DEV), pairs.to(DEV), BF16, unroll=unroll, swiglu_pairs=True).cpu().double()
         assert got.shape == (40, I) and torch.allclose(got, want, rtol=2e-2, atol=2e-2)
+
+
+def test_logprobs_against_log_softmax_and_topk():
+    g = gen(17)
+    R, V = 5, 3000
+    logits = 2.0 * torch.randn(R, V, generator=g)
+    logits[1, 100] = logits[1, 7] = logits[1].max() + 1.0          # a tie at the top: index 7 first
+    chosen = torch.tensor([0, 100, 5, 2999, 17], dtype=torch.int32)
+    lp, ids, tlp = (t.cpu() for t in ops.logprobs(logits.to(DEV), chosen.to(DEV), 6))
+    want = torch.log_softmax(logits.double(), -1)
+    assert torch.allclose(lp.double(), want[torch.arange(R), chosen.long()], atol=1e-4)
+    for r in range(R):
+        order = sorted(range(V), key=lambda i: (-float(logits[r, i]), i))[:6]
+        assert ids[r].tolist() == order
+        assert torch.allclose(tlp[r].double(), want[r, order], atol=1e-4)
+    assert ids[1, :2].tolist() == [7, 100]
+    assert ops.logprobs(logits.to(DEV), chosen.to(DEV), 0)[1].shape == (R, 0)
