@@ -334,3 +334,26 @@ def test_toy_position_encoding_and_routed_feed_forward(tmp_path):
     x = x + y
     want = pm.rms_norm(x, model.final_norm.weight.double().cpu(), 1e-5) @ model.head.weight.double().cpu().t()
     assert torch.allclose(whole.double(), want, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [32, 64])
+def test_other_page_sizes(page_size, dtype, sharp_folders):
+    """Pages of 32 and 64 tokens (trace_run's rounding unit): mixed steps over a pool that is used again."""
+    import traces
+    folder = sharp_folders["C", dtype]
+    seqs = {f"r{i}": seeded_ids(500 + i, n, 777) for i, n in enumerate([70, 130, 45, 200, 64])}
+    steps, expected = traces.mixed(seqs, seed=page_size)
+    runner = load_runner(folder, DT[dtype], num_pages=traces.peak_tokens(steps, page_size) // page_size, page_size=page_size)
+    for s in steps:
+        for e in s["entries"]:
+            if not runner.has_request(e["id"]):
+                runner.add_request(e["id"])
+        got = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).cpu()
+        if s["step"] in expected:
+            want = torch.stack([plain_logits(folder, seqs[rid])[p] for rid, p in expected[s["step"]]])
+            assert rel_err(got, want) < REL_TOL[dtype], s["step"]
+        for rid in s["end"]:
+            runner.free_request(rid)
+        runner.manager.check()
+    assert runner.manager.free_pages() == [p.num_pages for p in runner.manager.pools]
