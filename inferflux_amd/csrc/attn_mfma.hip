@@ -300,7 +300,12 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
 // =======================================================================================
 // tiles
 // =======================================================================================
-constexpr int TQ = 64;            // query rows per workgroup (16 per wave)
+#ifndef TILE_QT
+#define TILE_QT 2
+#endif
+constexpr int QT = TILE_QT;       // 16-row query tiles per wave: each K and V operand read from LDS feeds QT products
+constexpr int TQ = 64 * QT;       // query rows per workgroup (4 waves)
+extern "C" int ifx_attn_tile_rows() { return TQ; }
 constexpr int TK = 64;            // keys per staged tile
 constexpr int KPAD = D + 8;       // bf16 elements per K row in LDS
 constexpr int VPAD = TK + 8;      // bf16 elements per V^T row in LDS
@@ -392,67 +397,95 @@ __device__ __forceinline__ void stage_tile(const TileRegs& r, bf16_t* k_s, bf16_
   }
 }
 
-// One staged tile of 64 keys against a wave's 16 query rows: scores, running softmax, output.
-// Scores stay unscaled; the scale (with log2 e) enters the exponent through one fused multiply-add.
-// MASKED adds the causal / window / row-validity test per score.
+// One staged tile of 64 keys against a wave's QT tiles of 16 query rows: scores, running softmax,
+// output.  Scores stay unscaled; the scale (with log2 e) enters the exponent through one fused
+// multiply-add.  MASKED adds the causal / window / row-validity test per score.
+struct QueryTile {
+  bf16x8 qop[KS];
+  floatx4 o[DT];
+  float m, l;
+  int pos, lo;     // this lane's query: its position and the first position it sees
+  bool ok;
+};
+
 template <bool MASKED>
-__device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, const bf16x8* qop, floatx4* o, float& m,
-                                          float& l, float c_log2e, int j0, int my_pos, int my_lo, bool q_ok, int col, int g4) {
-  floatx4 s[4];
-  float mb = -INFINITY;
+__device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, QueryTile* q, float c_log2e, int j0, int col,
+                                          int g4) {
+  floatx4 s[QT][4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int c = 32 * ks + 8 * g4;
       const bf16x8 kop = c < D ? *(const bf16x8*)(k_s + (16 * t + col) * KPAD + c) : zero8();
-      s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[ks], s[t], 0, 0, 0);
-    }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      if (MASKED) {
-        const int key = j0 + 16 * t + 4 * g4 + r;
-        const bool vis = q_ok && key <= my_pos && key >= my_lo;
-        s[t][r] = vis ? s[t][r] : -INFINITY;
-      }
-      mb = fmaxf(mb, s[t][r]);
+      for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, q[qt].qop[ks], s[qt][t], 0, 0, 0);
     }
   }
-  const float m_new = fmaxf(m, col_max(mb));
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = fast_exp2((m - m_safe) * c_log2e);
-  const float ms = m_safe * c_log2e;
-  float psum = 0.f;
-  bf16x4 pb[4];
+  bf16x8 pop[QT][2];
+  float alpha[QT];
+  bool rescale = false;
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int qt = 0; qt < QT; ++qt) {
+    float mb = -INFINITY;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float p = fast_exp2(fmaf(s[t][r], c_log2e, -ms));
-      psum += p;
-      pb[t][r] = (__bf16)p;
-    }
-  l = l * alpha + psum;
-  m = m_new;
-  const bf16x8 pop0 = join4(pb[0], pb[1]), pop1 = join4(pb[2], pb[3]);
-  const bool rescale = __any(alpha != 1.0f);   // once the running maxima have settled nothing is rescaled
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (MASKED) {
+          const int key = j0 + 16 * t + 4 * g4 + r;
+          const bool vis = q[qt].ok && key <= q[qt].pos && key >= q[qt].lo;
+          s[qt][t][r] = vis ? s[qt][t][r] : -INFINITY;
+        }
+        mb = fmaxf(mb, s[qt][t][r]);
+      }
+    const float m_new = fmaxf(q[qt].m, col_max(mb));
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    alpha[qt] = fast_exp2((q[qt].m - m_safe) * c_log2e);
+    const float ms = m_safe * c_log2e;
+    float psum = 0.f;
+    bf16x4 pb[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = fast_exp2(fmaf(s[qt][t][r], c_log2e, -ms));
+        psum += p;
+        pb[t][r] = (__bf16)p;
+      }
+    q[qt].l = q[qt].l * alpha[qt] + psum;
+    q[qt].m = m_new;
+    pop[qt][0] = join4(pb[0], pb[1]);
+    pop[qt][1] = join4(pb[2], pb[3]);
+    rescale = rescale || __any(alpha[qt] != 1.0f);   // once the running maxima have settled nothing is rescaled
+  }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 8 * g4;
     const bf16x8 vop0 = *(const bf16x8*)(vr), vop1 = *(const bf16x8*)(vr + 32);
-    if (rescale) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+    for (int qt = 0; qt < QT; ++qt) {
+      if (rescale) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q[qt].o[dt][r] *= alpha[qt];
+      }
+      q[qt].o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop[qt][0], q[qt].o[dt], 0, 0, 0);
+      q[qt].o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop[qt][1], q[qt].o[dt], 0, 0, 0);
     }
-    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop0, o[dt], 0, 0, 0);
-    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop1, o[dt], 0, 0, 0);
   }
 }
 
-// Three waves per SIMD: the kernel waits on LDS and on the matrix pipe, so one more wave to switch to
-// is worth more than the registers it costs (the compiler fits 162 without spilling).
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_tiles_kernel(TileArgs a) {
+// The kernel waits on LDS and on the matrix pipe, so waves to switch to are worth more than the
+// registers they cost: 3 waves per SIMD with one query tile per wave (162 registers, no spill), 2 with two.
+#if TILE_QT == 1
+#define TILE_WAVES_PER_SIMD 3
+#else
+#define TILE_WAVES_PER_SIMD 2
+#endif
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TILE_WAVES_PER_SIMD, TILE_WAVES_PER_SIMD)))
+void attn_tiles_kernel(TileArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t k_s[TK * KPAD];
   __shared__ __attribute__((aligned(16))) bf16_t v_s[D * VPAD];
   const int tid = threadIdx.x, wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g4 = lane >> 4;
@@ -474,25 +507,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   const int pos_first = start + q0, pos_last = pos_first + rows_here - 1;
   const int lo_wg = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
 
-  const int my_q = q0 + 16 * wid + col;                 // this lane's query column, as a row of the request
-  const bool q_ok = my_q < qlen;
-  const int my_pos = start + my_q;
-  const int my_lo = a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
-  const size_t my_row = (size_t)a.q_start[req] + my_q;
-  // the keys this wave's 16 rows can see at all: tiles outside are skipped by the whole wave
-  const int wave_first = pos_first + 16 * wid;
-  const int wave_hi = min(pos_last, pos_first + 16 * wid + 15);
-  const int wave_lo = a.window > 0 ? max(0, pos_first + 16 * wid - a.window + 1) : 0;
-  bf16x8 qop[KS];
+  // this wave's rows: QT tiles of 16, lane `col` of tile qt holds row 16 * QT * wid + 16 * qt + col of the tile
+  const int wave_q = q0 + 16 * QT * wid;
+  const size_t row0 = (size_t)a.q_start[req];
+  QueryTile q[QT];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int c = 32 * ks + 8 * g4;
-    qop[ks] = (q_ok && c < D) ? *(const bf16x8*)(a.q + (my_row * a.nH + head) * D + c) : zero8();
+  for (int qt = 0; qt < QT; ++qt) {
+    const int my_q = wave_q + 16 * qt + col;
+    q[qt].ok = my_q < qlen;
+    q[qt].pos = start + my_q;
+    q[qt].lo = a.window > 0 ? max(0, q[qt].pos - a.window + 1) : 0;
+    q[qt].m = -INFINITY;
+    q[qt].l = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = 32 * ks + 8 * g4;
+      q[qt].qop[ks] = (q[qt].ok && c < D) ? *(const bf16x8*)(a.q + ((row0 + my_q) * a.nH + head) * D + c) : zero8();
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) q[qt].o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
-  floatx4 o[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  // the keys this wave's rows can see at all: tiles outside are skipped by the whole wave
+  const int wave_first = start + wave_q;
+  const int wave_hi = min(pos_last, wave_first + 16 * QT - 1);
+  const int wave_lo = a.window > 0 ? max(0, wave_first - a.window + 1) : 0;
 
   TileRegs regs;
   int pg[TK / 16];
@@ -512,19 +550,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
     // A tile every key of which every row of this wave sees needs no mask: the common case.
     const bool full = j0 + TK - 1 <= wave_first && (a.window <= 0 || j0 >= wave_hi - a.window + 1);
-    if (full) tile_math<false>(k_s, v_s, qop, o, m, l, a.scale_log2e, j0, my_pos, my_lo, q_ok, col, g4);
-    else tile_math<true>(k_s, v_s, qop, o, m, l, a.scale_log2e, j0, my_pos, my_lo, q_ok, col, g4);
+    if (full) tile_math<false>(k_s, v_s, q, a.scale_log2e, j0, col, g4);
+    else tile_math<true>(k_s, v_s, q, a.scale_log2e, j0, col, g4);
   }
-  l = col_sum(l);
-  if (q_ok) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    bf16_t* orow = a.out + (my_row * a.nH + head) * D;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      bf16x4 w;
+  for (int qt = 0; qt < QT; ++qt) {
+    const float l = col_sum(q[qt].l);
+    if (q[qt].ok) {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      bf16_t* orow = a.out + ((row0 + wave_q + 16 * qt + col) * a.nH + head) * D;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) w[r] = (__bf16)(o[dt][r] * inv);
-      *(bf16x4*)(orow + 16 * dt + 4 * g4) = w;
+      for (int dt = 0; dt < DT; ++dt) {
+        bf16x4 w;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w[r] = (__bf16)(q[qt].o[dt][r] * inv);
+        *(bf16x4*)(orow + 16 * dt + 4 * g4) = w;
+      }
     }
   }
 }

@@ -3,7 +3,7 @@
 Every choice computes the same function (causal, optionally windowed, grouped-query attention
 over the paged cache); they differ in speed and in which sizes they accept.  In bfloat16 with a
 head size the matrix-core module takes, requests that bring at least TILE_MIN rows go to the
-tile kernel and all other rows (decode tokens, short portions) to the row kernel; everything
+tile kernel (tiles of as many rows as the compiled module says) and all other rows (decode tokens, short portions) to the row kernel; everything
 else (float32, other head sizes) goes to the plain kernel.
 """
 from __future__ import annotations
@@ -16,20 +16,20 @@ import torch
 from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
-TILE_ROWS = 64      # rows per tile of the tile kernel
+TILE_QT2_MIN_WORKGROUPS = 512   # the chip holds 2 workgroups of the tile kernel on each of its 256 CUs
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 64  # and until a row has at most this many splits
 
 
-def _work_lists(ctx, ctx_kv_heads):
+def _work_lists(ctx, ctx_kv_heads, tile_rows):
     """What the kernels need beyond the step's own arrays, computed once per step (and per number of
     kv heads, which decides how many waves a launch has)."""
     q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
     tiled = q_len >= TILE_MIN
     tile_req, tile_q0 = [], []
     for r in np.nonzero(tiled)[0]:
-        for q0 in range(0, int(q_len[r]), TILE_ROWS):
+        for q0 in range(0, int(q_len[r]), tile_rows):
             tile_req.append(r); tile_q0.append(q0)
     row_mask = ~tiled[ctx.h_row_req] if ctx.n_tokens else np.zeros(0, bool)
     rows = np.nonzero(row_mask)[0].astype(np.int32)
@@ -57,11 +57,16 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
     n_kv = cache.k.shape[1]
-    w = ctx.derived(("attention_work_lists", n_kv), lambda: _work_lists(ctx, n_kv))
+    # two query tiles per wave when that still leaves enough workgroups to fill the chip
+    big = ops.attention_tile_rows(d, 2)
+    n_big = sum(-(-int(n) // big) for n in ctx.h_q_len if n >= TILE_MIN)
+    qt = 2 if n_big * nH >= TILE_QT2_MIN_WORKGROUPS else 1
+    tile_rows = ops.attention_tile_rows(d, qt)
+    w = ctx.derived(("attention_work_lists", n_kv, tile_rows), lambda: _work_lists(ctx, n_kv, tile_rows))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
-                            table, window, scale)
+                            table, window, scale, qt)
     if w["n_rows"]:
         ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
                            window, scale, w["chunk"], w["max_splits"])

@@ -28,6 +28,10 @@ ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
 # first runs; these sizes are compiled ahead by build_all().
 MFMA_HEAD_DIMS_PREBUILT = (16, 32, 64, 128)
 MFMA_MAX_HEAD_DIM = 128
+# Query tiles of 16 rows per wave in the tile kernel: 2 (128 rows per workgroup) reuses each key and
+# value operand twice and is faster once there are enough workgroups to fill the chip; 1 (64 rows)
+# gives twice as many workgroups for short portions.
+TILE_QTS = (1, 2)
 
 
 class KernelError(RuntimeError):
@@ -41,7 +45,8 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("sampling", ())
     yield ("gemm_bf16", ())
     for d in MFMA_HEAD_DIMS_PREBUILT:
-        yield ("attn_mfma", (("HEAD_DIM", d),))
+        for qt in TILE_QTS:
+            yield ("attn_mfma", (("HEAD_DIM", d), ("TILE_QT", qt)))
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -347,7 +352,7 @@ def mfma_attention_supported(dtype: torch.dtype, head_dim: int, page_size: int) 
             and page_size >= 16 and page_size & (page_size - 1) == 0)
 
 
-def _attn_common(q, k_cache, v_cache):
+def _attn_common(q, k_cache, v_cache, qt=1):
     _check(q, "q", (None, None, None), torch.bfloat16)
     T, nH, d = q.shape
     _check(k_cache, "k_cache", (None, None, None, d), torch.bfloat16)
@@ -356,7 +361,7 @@ def _attn_common(q, k_cache, v_cache):
     if not mfma_attention_supported(q.dtype, d, page_size):
         raise KernelError(f"matrix-core attention needs bfloat16, head_dim a multiple of 16 up to {MFMA_MAX_HEAD_DIM} and "
                           f"page_size a power of two from 16; got head_dim {d}, page_size {page_size}")
-    return T, nH, d, nKV, page_size, load_module("attn_mfma", (("HEAD_DIM", d),))
+    return T, nH, d, nKV, page_size, load_module("attn_mfma", (("HEAD_DIM", d), ("TILE_QT", qt)))
 
 
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -382,12 +387,21 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
           int(window or 0), chunk, max_splits, float(scale), part_o.data_ptr(), part_ml.data_ptr(), _stream())
 
 
+def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
+    """Rows per tile of the tile kernel compiled for ``head_dim`` with ``qt`` query tiles per wave."""
+    mod = load_module("attn_mfma", (("HEAD_DIM", head_dim), ("TILE_QT", qt)))
+    f = mod.lib.ifx_attn_tile_rows
+    f.restype = ctypes.c_int
+    return int(f())
+
+
 def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                     tile_req: torch.Tensor, tile_q0: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-                    kv_len: torch.Tensor, block_table: torch.Tensor, window: Optional[int], scale: float) -> None:
-    """Attention of tiles of 64 consecutive rows of one request each (tile t: request tile_req[t], rows
-    from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d]."""
-    T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache)
+                    kv_len: torch.Tensor, block_table: torch.Tensor, window: Optional[int], scale: float,
+                    qt: int = 1) -> None:
+    """Attention of tiles of ``attention_tile_rows(d, qt)`` consecutive rows of one request each (tile t:
+    request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d]."""
+    T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt)
     _check(out, "out", (T, nH * d), torch.bfloat16)
     n_tiles = tile_req.shape[0]
     _check(tile_req, "tile_req", (n_tiles,), torch.int32)

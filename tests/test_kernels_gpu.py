@@ -326,18 +326,19 @@ def test_attention_rows_subset_leaves_other_rows_alone():
     assert torch.all(out[rest] == 0)
 
 
+@pytest.mark.parametrize("qt", [1, 2])
 @pytest.mark.parametrize("case", MFMA_CASES)
-def test_attention_tiles(case):
+def test_attention_tiles(case, qt):
     lens_q, lens_past, nH, nKV, d, P, window, sharp = case
     (q, kc, vc, row_req, positions, table), want, info = paged_case(7, lens_q, lens_past, nH, nKV, d, P, BF16, window, sharp=sharp)
     T = q.shape[0]
     out = torch.zeros(T, nH * d, dtype=BF16, device=DEV)
     q_len = torch.tensor(info["q_lens"], dtype=torch.int32)
     q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
-    tiles = [(r, q0) for r, n in enumerate(info["q_lens"]) for q0 in range(0, n, 64)]
+    tiles = [(r, q0) for r, n in enumerate(info["q_lens"]) for q0 in range(0, n, ops.attention_tile_rows(d, qt))]
     dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     ops.attention_tiles(q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV),
-                        q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d))
+                        q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt)
     out = out.cpu().double()
     assert torch.isfinite(out).all()
     assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
