@@ -55,7 +55,8 @@ def cmd_completion(args) -> int:
     prompts = _read_ids(args)
     engine = Engine.load(args.model, dtype=args.dtype, kv_pages=args.kv_pages, ctx_size=args.ctx_size,
                          max_batch_size=args.max_parallel_sequences, max_batch_tokens=args.batch_size,
-                         chunked_prefill_tokens=args.chunked_prefill_tokens, phase_timing=args.phase_timing)
+                         chunked_prefill_tokens=args.chunked_prefill_tokens, phase_timing=args.phase_timing,
+                         decode_weight_copy=not args.no_decode_weight_copy)
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p,
                             frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
                             repetition_penalty=args.repetition_penalty, penalty_last_n=args.penalty_last_n,
@@ -137,6 +138,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     c.add_argument("--max-parallel-sequences", type=int, default=32, help="most requests in one step (max_batch_size)")
     c.add_argument("--chunked-prefill-tokens", type=int, default=512)
     c.add_argument("--kv-pages", type=int, default=None, help="pages of 16 tokens in the cache (overrides --ctx-size)")
+    c.add_argument("--no-decode-weight-copy", action="store_true",
+                   help="keep one copy of the weights only (saves their size in memory, decoding is slower)")
     c.add_argument("--phase-timing", action="store_true",
                    help="print per-phase times of every forward pass (synchronises after each phase: slow)")
     c.set_defaults(fn=cmd_completion)

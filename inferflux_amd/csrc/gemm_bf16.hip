@@ -10,6 +10,13 @@
 // their accumulators through LDS in a fixed order, so the result does not depend on timing.
 // U blocks are loaded before the first is consumed, to keep enough bytes in flight.
 //
+// The weight may also come pre-tiled for exactly this walk (TILED): tile (t, kt) holds the 16 rows
+// 16 t .. 16 t + 15 at k = 32 kt .. 32 kt + 31 as 64 pieces of 16 bytes, piece 16 g + col = row
+// 16 t + col at k = 32 kt + 8 g; tiles follow each other along k, then along t, and the tensor is
+// padded with zeros to whole tiles and to an even number of tiles along k.  A wave's load then
+// covers 1 KB of contiguous memory instead of 16 half-used lines, and x is read in runs of 64
+// contiguous bytes per row; measured on 7B shapes this takes 15-25 % off the time.
+//
 // The reference sends these products to cuBLAS (runtime/backends/cuda/native/cublas_gemm.cpp:
 // 99-117) and measured 30-44 % of its roofline there (docs/benchmarks.md:180-183).
 #include "common.h"
@@ -28,9 +35,9 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // EPI 0: out[m, n] = acc.  EPI 1: the rows of W alternate gate, up, gate, up ...; a lane holds two
 // such pairs of one output row and writes silu(gate) * up to out[m, n / 2] (out is [M, N / 2]).
-template <int MT, int NT, int U, typename TO, int EPI>
+template <int MT, int NT, int U, typename TO, int EPI, bool TILED>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out,
-                                   int M, int N, int K) {
+                                   int M, int N, int K, int k_tiles) {
   extern __shared__ float red[];  // [(waves - 1)][NT * MT][64 lanes][4]
   const int wid = threadIdx.x / WAVE, nw = blockDim.x / WAVE, lane = threadIdx.x % WAVE;
   const int col = lane & 15, g = lane >> 4;
@@ -41,9 +48,11 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const bf16_t* wrow[NT];
+  const bf16_t* wrow[NT];  // rows (tiles) past N are read again, never stored
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) wrow[nt] = W + (size_t)min(n_base + 16 * nt + col, N - 1) * K;  // rows past N are read again, never stored
+  for (int nt = 0; nt < NT; ++nt)
+    wrow[nt] = TILED ? W + ((size_t)min(n_base / 16 + nt, (N - 1) / 16) * k_tiles * WAVE + lane) * 8
+                     : W + (size_t)min(n_base + 16 * nt + col, N - 1) * K;
   const bf16_t* xrow[MT];
   bool xok[MT];
 #pragma unroll
@@ -57,14 +66,21 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
     bf16x8 wa[U][NT][2], xa[U][MT][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = (kb0 + u) * 64 + 16 * g;
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const bool kok = kb0 + u < nkb && k + 8 * h < K;
+        // the lane's 8 k-values of step h of block kb0 + u, and where its piece of W lies
+        const int k = TILED ? (kb0 + u) * 64 + 32 * h + 8 * g : (kb0 + u) * 64 + 16 * g + 8 * h;
+        const size_t w_off = TILED ? (size_t)(2 * (kb0 + u) + h) * WAVE * 8 : (size_t)k;
+        const bool blk = kb0 + u < nkb, kok = blk && k < K;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wa[u][nt][h] = kok ? *(const bf16x8*)(wrow[nt] + k + 8 * h) : zero8();
+        for (int nt = 0; nt < NT; ++nt) {
+          // Tiles are read once, in whole lines: a streaming load keeps them from pushing x out of the L2.
+          // (Rows are read in half lines by two loads; there the hint costs more than it gives.)
+          const bf16x8* wp = (const bf16x8*)(wrow[nt] + w_off);
+          wa[u][nt][h] = TILED ? (blk ? __builtin_nontemporal_load(wp) : zero8()) : (kok ? *wp : zero8());
+        }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xa[u][mt][h] = (kok && xok[mt]) ? *(const bf16x8*)(xrow[mt] + k + 8 * h) : zero8();
+        for (int mt = 0; mt < MT; ++mt) xa[u][mt][h] = (kok && xok[mt]) ? *(const bf16x8*)(xrow[mt] + k) : zero8();
       }
     }
 #pragma unroll
@@ -122,14 +138,15 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
     }
 }
 
-template <int MT, int NT, int U>
-static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int waves, int epi, hipStream_t s) {
+template <int MT, int NT, int U, bool TILED>
+static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int k_tiles, int waves, int epi,
+                  hipStream_t s) {
   const int groups = (N + 16 * NT - 1) / (16 * NT);
   const size_t lds = (size_t)(waves - 1) * NT * MT * WAVE * 4 * sizeof(float);
   IFX_REQUIRE(lds <= 64 * 1024, "skinny_gemm: %d waves of %dx%d tiles need %zu bytes of LDS", waves, NT, MT, lds);
 #define GO(TO_, EPI_)                                                                                              \
-  hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, TO_, EPI_>), dim3(groups), dim3(waves * WAVE), lds, s,         \
-                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K)
+  hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, TO_, EPI_, TILED>), dim3(groups), dim3(waves * WAVE), lds, s,  \
+                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles)
   if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
   else if (out_dtype == DT_BF16) GO(bf16_t, 1);
   else if (epi == 0) GO(float, 0);
@@ -138,10 +155,34 @@ static int launch(const void* x, const void* W, void* out, int out_dtype, int M,
   IFX_LAUNCH_CHECK();
 }
 
+// Rows and k-values of the tiled form of an [N, K] weight: whole tiles, an even number along k.
+extern "C" int ifx_tiled_rows(int N) { return (N + 15) / 16 * 16; }
+extern "C" int ifx_tiled_cols(int K) { return (K + 63) / 64 * 64; }
+
+__global__ void tile_weights_kernel(const bf16_t* __restrict__ W, bf16_t* __restrict__ Wt, int N, int K, int k_tiles, size_t pieces) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // piece number: ((t * k_tiles + kt) * 64 + 16 g + col)
+  if (i >= pieces) return;
+  const int lane = (int)(i % WAVE), col = lane & 15, g = lane >> 4;
+  const size_t tile = i / WAVE;
+  const int kt = (int)(tile % k_tiles), n = (int)(tile / k_tiles) * 16 + col, k = 32 * kt + 8 * g;
+  *(bf16x8*)(Wt + i * 8) = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero8();
+}
+
+// Wt [ifx_tiled_rows(N) * ifx_tiled_cols(K)] = the tiled form of W [N, K] (K a multiple of 8).
+extern "C" int ifx_tile_weights(const void* W, void* Wt, int N, int K, void* stream) {
+  IFX_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "tile_weights: N=%d K=%d (K must be a multiple of 8)", N, K);
+  const int k_tiles = ifx_tiled_cols(K) / 32;
+  const size_t pieces = (size_t)(ifx_tiled_rows(N) / 16) * k_tiles * WAVE;
+  hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)W, (bf16_t*)Wt, N, K, k_tiles, pieces);
+  IFX_LAUNCH_CHECK();
+}
+
 // nt, waves, unroll = 0: chosen here from the shape.
 // epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2].
+// tiled 1: W is the tiled form written by ifx_tile_weights.
 extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int nt,
-                               int waves, int unroll, int epi, void* stream) {
+                               int waves, int unroll, int epi, int tiled, void* stream) {
   IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "skinny_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "skinny_gemm: K=%d must be a multiple of 8", K);
@@ -151,6 +192,23 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   const int nkb = (K + 63) / 64;
   // Choices measured on the 7B shapes at 1-16 rows: two row tiles per wave pay off only for very tall
   // weights; deeper unrolling than 4 blocks spills; about 1500-2500 waves fill the chip.
+  if (tiled && mt == 1) {
+    // Measured on the tiled copy (7B shapes, 1-16 rows): two row tiles per wave halve the reads of x and
+    // win wherever they leave 128 workgroups or more, except for the tallest weights at 1-4 rows; tall
+    // weights want 8 waves per workgroup up to 8 rows of x and one beyond; the others enough waves to
+    // reach about a thousand.
+    const bool tall = N >= 32768;
+    if (nt == 0) nt = tall ? (M <= 4 ? 1 : 2) : ((N + 31) / 32 >= 128 ? 2 : 1);
+    if (unroll == 0) unroll = (nt == 1 && M <= 4) ? 4 : 2;
+    if (waves == 0) {
+      const int groups = (N + 16 * nt - 1) / (16 * nt);
+      waves = 1;
+      if (tall) waves = M <= 8 ? 8 : 1;
+      else
+        while (waves < 16 && groups * waves < 1024) waves *= 2;
+      while (waves > 1 && nkb < waves * 2) waves /= 2;
+    }
+  }
   if (nt == 0) nt = (N >= 32768 && mt <= 2) ? 2 : 1;
   if (unroll == 0) unroll = (mt * nt >= 2) ? 2 : 4;
   if (waves == 0) {
@@ -158,11 +216,15 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
     waves = 1;
     if (groups < 1024)
       while (waves < 16 && groups * waves < 1536 && nkb >= waves * 2) waves *= 2;
-    while (waves > 1 && (size_t)(waves - 1) * nt * mt * WAVE * 16 > 64 * 1024) waves /= 2;
   }
+  while (waves > 1 && (size_t)(waves - 1) * nt * mt * WAVE * 16 > 64 * 1024) waves /= 2;
   IFX_REQUIRE(waves >= 1 && waves <= 16, "skinny_gemm: waves=%d outside 1..16", waves);
   hipStream_t s = (hipStream_t)stream;
-#define CASE(MT_, NT_, U_) if (mt == MT_ && nt == NT_ && unroll == U_) return launch<MT_, NT_, U_>(x, W, out, out_dtype, M, N, K, waves, epi, s)
+  const int k_tiles = ifx_tiled_cols(K) / 32;
+#define CASE(MT_, NT_, U_)                                                                                  \
+  if (mt == MT_ && nt == NT_ && unroll == U_)                                                               \
+    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, s)        \
+                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, s)
   CASE(1, 1, 4); CASE(1, 2, 4); CASE(1, 1, 2); CASE(1, 2, 2); CASE(1, 1, 8); CASE(1, 2, 8);
   CASE(2, 1, 4); CASE(2, 2, 2); CASE(2, 1, 2); CASE(2, 2, 4);
   CASE(3, 1, 2); CASE(3, 2, 2); CASE(3, 1, 4);

@@ -6,6 +6,7 @@ from typing import Optional
 import torch
 
 from ..config.registry import load_config
+from ..kernels import ops
 from .model import Model
 from .runner import ModelRunner
 
@@ -16,15 +17,22 @@ def require_gpu() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device())
 
 
-def load_model(folder: str, dtype: torch.dtype = torch.bfloat16, device=None) -> Model:
-    """The model class is chosen by config.json; weights are read by tensor name."""
+def load_model(folder: str, dtype: torch.dtype = torch.bfloat16, device=None, decode_weight_copy: bool = True) -> Model:
+    """The model class is chosen by config.json; weights are read by tensor name.  With
+    ``decode_weight_copy`` every bfloat16 projection also keeps the tiled copy that products with few
+    rows stream from (twice the weights' memory for about a fifth off a decode step)."""
     device = device or require_gpu()
     if dtype == torch.float32:
         # The 32-bit path never uses a reduced-precision matrix mode; the engine's own float32
         # kernels do not consult these switches, they are set for any library call a part makes.
         torch.backends.cuda.matmul.allow_tf32 = False
     config = load_config(folder)
-    return Model(config).load_folder(folder, dtype, device)
+    before = ops.decode_weight_copy
+    ops.decode_weight_copy = bool(decode_weight_copy)
+    try:
+        return Model(config).load_folder(folder, dtype, device)
+    finally:
+        ops.decode_weight_copy = before
 
 
 def plan_kv_pages(model: Model, page_size: int, wanted_tokens: int, memory_fraction: float = 0.8) -> int:
@@ -51,9 +59,9 @@ def plan_kv_pages(model: Model, page_size: int, wanted_tokens: int, memory_fract
 
 def load_runner(folder: str, dtype: torch.dtype = torch.bfloat16, num_pages: Optional[int] = 256, page_size: int = 16,
                 max_requests: int = 64, device=None, cache_tokens: Optional[int] = None,
-                phase_timing: bool = False) -> ModelRunner:
+                phase_timing: bool = False, decode_weight_copy: bool = True) -> ModelRunner:
     """``num_pages`` None: as many pages as ``cache_tokens`` need, within the free device memory."""
-    model = load_model(folder, dtype, device)
+    model = load_model(folder, dtype, device, decode_weight_copy)
     if num_pages is None:
         num_pages = plan_kv_pages(model, page_size, cache_tokens or 4096 * max_requests)
     return ModelRunner(model, num_pages=num_pages, page_size=page_size, max_requests=max_requests,

@@ -69,12 +69,14 @@ class Engine:
     @classmethod
     def load(cls, model: str, dtype: str = "bfloat16", kv_pages: Optional[int] = None, page_size: int = 16,
              max_batch_size: int = 32, max_batch_tokens: int = 16384, chunked_prefill_tokens: int = 512,
-             ctx_size: int = 4096, phase_timing: bool = False) -> "Engine":
+             ctx_size: int = 4096, phase_timing: bool = False, decode_weight_copy: bool = True) -> "Engine":
         """``kv_pages`` None sizes the cache for ``ctx_size`` tokens for each of ``max_batch_size``
-        requests, within the device memory that is free once the weights are loaded."""
+        requests, within the device memory that is free once the weights are loaded.
+        ``decode_weight_copy`` False saves the second, tiled copy of the weights at the price of slower decoding."""
         dt = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}[dtype]
         runner = load_runner(model, dt, num_pages=kv_pages, page_size=page_size, max_requests=max_batch_size,
-                             cache_tokens=ctx_size * max_batch_size, phase_timing=phase_timing)
+                             cache_tokens=ctx_size * max_batch_size, phase_timing=phase_timing,
+                             decode_weight_copy=decode_weight_copy)
         log.info("engine", "model loaded", model=model, dtype=dtype, kv_pages=runner.manager.pools[0].num_pages
                  if runner.manager.pools else 0, page_size=page_size, max_batch_size=max_batch_size)
         return cls(runner, SchedulerConfig(max_batch_size, max_batch_tokens, chunked_prefill_tokens))

@@ -12,6 +12,7 @@ from typing import Iterable, Optional, Tuple
 
 import torch
 
+from .. import log
 from .library import KernelModule, Variant, load_module
 
 P = ctypes.c_void_p
@@ -230,23 +231,81 @@ def pause_library_gemm_tuning(paused: bool) -> None:
         tunable.tuning_enable(not paused)
 
 
+def tile_weights(weight: torch.Tensor) -> torch.Tensor:
+    """The tiled form of a bfloat16 ``weight`` [N, K] that the weight-streaming product reads in
+    contiguous kilobytes: a flat tensor of rows16(N) * cols64(K) elements (zeros in the padding)."""
+    _check(weight, "weight", (None, None), torch.bfloat16)
+    N, K = weight.shape
+    if K % 8:
+        raise KernelError(f"tile_weights: K={K} must be a multiple of 8")
+    mod = load_module("gemm_bf16")
+    size = mod.fn("ifx_tiled_rows", (I,))(N) * mod.fn("ifx_tiled_cols", (I,))(K)
+    out = torch.empty((size,), dtype=torch.bfloat16, device=weight.device)
+    _call(mod, "ifx_tile_weights", (P, P, I, I, P), weight.data_ptr(), out.data_ptr(), N, K, _stream())
+    return out
+
+
+class LinearWeight:
+    """A projection's weight as the products want it: ``rows`` [N, K] as the model file has it, and for
+    bfloat16 weights ``tiled``, the copy that products with few rows of x (decoding) stream from.  The
+    copy doubles the weight's memory; it is left out when ``decode_weight_copy`` is off or when the
+    card has no room for it, and products with few rows then read ``rows``."""
+
+    __slots__ = ("rows", "tiled")
+
+    def __init__(self, rows: torch.Tensor, tiled: Optional[torch.Tensor] = None):
+        self.rows, self.tiled = rows, tiled
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+
+# Whether prepare_linear makes tiled copies, and how much memory it leaves free when it does.
+decode_weight_copy = True
+DECODE_COPY_RESERVE_BYTES = 8 << 30
+
+
+def prepare_linear(weight: torch.Tensor) -> LinearWeight:
+    """Wrap a projection's weight for ``linear`` / ``linear_swiglu``, with the tiled copy if wanted and possible."""
+    tiled = None
+    if (decode_weight_copy and weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2
+            and weight.shape[1] % 8 == 0):
+        free, _ = torch.cuda.mem_get_info(weight.device)
+        if free >= weight.numel() * 2 + DECODE_COPY_RESERVE_BYTES:
+            tiled = tile_weights(weight.contiguous())
+        else:
+            log.warn("kernels", f"no room for the decode copy of a {tuple(weight.shape)} weight "
+                                f"({free / 2**30:.1f} GiB free): decoding reads the plain rows")
+    return LinearWeight(weight, tiled)
+
+
 def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
+                nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False,
+                tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
     accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose.
-    With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2]."""
+    With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2].
+    With ``tiled`` (``tile_weights(weight)``) the kernel streams that copy instead of the rows."""
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     _check(weight, "weight", (None, K), torch.bfloat16)
     N = weight.shape[0]
+    if tiled is not None:
+        mod = load_module("gemm_bf16")
+        _check(tiled, "tiled", (mod.fn("ifx_tiled_rows", (I,))(N) * mod.fn("ifx_tiled_cols", (I,))(K),), torch.bfloat16)
     if M > SKINNY_MAX_M or K % 8:
         raise KernelError(f"skinny_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
     if swiglu_pairs and N % 2:
         raise KernelError("skinny_gemm: gate/up pairs need an even number of weight rows")
     out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
-    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, I, P),
-          x.data_ptr(), weight.data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves, unroll,
-          1 if swiglu_pairs else 0, _stream())
+    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, I, I, P),
+          x.data_ptr(), (weight if tiled is None else tiled).data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves,
+          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else 1, _stream())
     return out
 
 
@@ -272,8 +331,9 @@ def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """x [M, K] times ``weight`` [N, K] transposed, chosen by the weight's type and by M.
+def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x [M, K] times ``weight`` [N, K] transposed (a tensor or a ``LinearWeight``), chosen by the weight's
+    type and by M.
 
     A float32 weight takes the true 32-bit kernel whatever the activation's type.  A bfloat16
     weight with bfloat16 activations takes the weight-streaming kernel for up to 64 rows and the
@@ -281,6 +341,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     projection (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).  float32 output (logits)
     always comes from float accumulators, never through a bfloat16 rounding.
     """
+    tiled = None
+    if isinstance(weight, LinearWeight):
+        weight, tiled = weight.rows, weight.tiled
     if weight.dtype == torch.float32:
         return gemm_f32(x, weight, None, out_dtype or x.dtype)
     if weight.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
@@ -289,9 +352,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     _check(weight, "weight", (None, None))
     out_dtype = out_dtype or torch.bfloat16
     M, K = x.shape
-    kind = _small_m_kernel(M, weight.shape[0], K)
+    kind = _small_m_kernel(M, weight.shape[0], K, tiled is not None)
     if kind == "skinny":
-        return skinny_gemm(x, weight, out_dtype)
+        return skinny_gemm(x, weight, out_dtype, tiled=tiled)
     if kind == "staged":
         return staged_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:
@@ -299,7 +362,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     return torch.matmul(x, weight.t())
 
 
-def _small_m_kernel(M: int, N: int, K: int) -> Optional[str]:
+def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional[str]:
     """Which of the two streaming kernels takes a bfloat16 product of this shape, or None for the
     library.  Measured on the 7B shapes: streaming wins up to 16 rows everywhere (with x staged in LDS
     for very tall weights such as the head's) and up to 32 rows on the narrow products; beyond that
@@ -307,23 +370,25 @@ def _small_m_kernel(M: int, N: int, K: int) -> Optional[str]:
     if K % 8:
         return None
     if M <= 16:
-        return "staged" if N >= 65536 else "skinny"
+        return "staged" if N >= 65536 and not has_tiled else "skinny"
     if M <= 32 and N <= 4096:
         return "skinny"
     return None
 
 
-def linear_swiglu(x: torch.Tensor, weight_pairs: torch.Tensor) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) where ``weight_pairs`` [2I, K] alternates the rows of Wg and Wu.
-    For few rows the activation is the product's epilogue; otherwise a second kernel applies it."""
+def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) where ``weight_pairs`` [2I, K] (a tensor or a ``LinearWeight``) alternates the
+    rows of Wg and Wu.  For few rows the activation is the product's epilogue; otherwise a second kernel
+    applies it."""
     M, K = x.shape
-    if weight_pairs.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-        kind = _small_m_kernel(M, weight_pairs.shape[0], K)
+    rows, tiled = (weight_pairs.rows, weight_pairs.tiled) if isinstance(weight_pairs, LinearWeight) else (weight_pairs, None)
+    if rows.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
+        kind = _small_m_kernel(M, rows.shape[0], K, tiled is not None)
         if kind == "skinny":
-            return skinny_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
+            return skinny_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, tiled=tiled)
         if kind == "staged":
-            return staged_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
-    return swiglu(linear(x, weight_pairs), interleaved=True)
+            return staged_gemm(x, rows, torch.bfloat16, swiglu_pairs=True)
+    return swiglu(linear(x, rows), interleaved=True)
 
 
 # ----------------------------------------------------------------------------------------

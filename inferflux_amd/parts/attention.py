@@ -40,7 +40,7 @@ class PagedAttention(Mixer):
         self.bias, self.window, self.init_std = bool(bias), (int(window) if window else None), init_std
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = build_part("position", position)
-        self.w_qkv = self.b_qkv = self.w_o = None
+        self.w_qkv = self.b_qkv = self.w_o = self._w_q = None
 
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(self.n_kv_heads, self.head_dim, self.window)
@@ -61,9 +61,10 @@ class PagedAttention(Mixer):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         n = self.name
-        self.w_qkv = concat_weights([tensors[f"{n}.{p}_proj.weight"] for p in "qkv"])
+        self.w_qkv = ops.prepare_linear(concat_weights([tensors[f"{n}.{p}_proj.weight"] for p in "qkv"]))
         self.b_qkv = concat_weights([tensors[f"{n}.{p}_proj.bias"] for p in "qkv"]) if self.bias else None
-        self.w_o = tensors[f"{n}.o_proj.weight"]
+        self.w_o = ops.prepare_linear(tensors[f"{n}.o_proj.weight"])
+        self._w_q = None
 
     def forward(self, h: torch.Tensor, ctx, binding: MixerBinding) -> torch.Tensor:
         cache = binding.cache
@@ -73,7 +74,9 @@ class PagedAttention(Mixer):
         style, rotary_dim, cos, sin = self.position.kernel_args(ctx)
         w, b = self.w_qkv, self.b_qkv
         if not binding.writes_cache:  # only the queries: the first nH*d rows of the fused matrix
-            w, b = w[:width], (b[:width] if b is not None else None)
+            if self._w_q is None:
+                self._w_q = ops.prepare_linear(w.rows[:width])
+            w, b = self._w_q, (b[:width] if b is not None else None)
         qkv = ops.linear(h, w)
         if self.position.needs_apply:
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None

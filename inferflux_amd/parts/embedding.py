@@ -44,7 +44,7 @@ class LinearHead(Part):
 
     def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, init_std: float = 0.02):
         self.name, self.vocab_size, self.hidden_size, self.tied_to, self.init_std = name, int(vocab_size), int(hidden_size), tied_to, init_std
-        self.weight: Optional[torch.Tensor] = None
+        self.weight: Optional[ops.LinearWeight] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         if self.tied_to:
@@ -52,7 +52,7 @@ class LinearHead(Part):
         return {f"{self.name}.weight": ParamSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.tied_to or f"{self.name}.weight"]
+        self.weight = ops.prepare_linear(tensors[self.tied_to or f"{self.name}.weight"])
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return ops.linear(h, self.weight, out_dtype=torch.float32)

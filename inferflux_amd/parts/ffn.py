@@ -48,8 +48,9 @@ class SwiGLU(FeedForward):
         g, u = tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
-        self.w_down = tensors[f"{self.name}.down_proj.weight"]
+        self.w_gate_up = ops.prepare_linear(
+            torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous())
+        self.w_down = ops.prepare_linear(tensors[f"{self.name}.down_proj.weight"])
 
     def forward(self, h, ctx):
         return ops.linear(ops.linear_swiglu(h, self.w_gate_up), self.w_down)

@@ -323,16 +323,16 @@ def test_toy_position_encoding_and_routed_feed_forward(tmp_path):
     x = model.embedding.table.double().cpu()[ids]
     pos = torch.arange(50, dtype=torch.float64)
     h = pm.rms_norm(x, model.blocks[0].norm_in.weight.double().cpu(), 1e-5)
-    qkv = h @ att.w_qkv.double().cpu().t() + att.b_qkv.double().cpu()
+    qkv = h @ att.w_qkv.rows.double().cpu().t() + att.b_qkv.double().cpu()
     qq = qkv[:, : nH * d].view(50, nH, d) * (1 + pos / 100)[:, None, None]
     kk = qkv[:, nH * d: (nH + 1) * d].view(50, 1, d) / (1 + pos / 50)[:, None, None]
     vv = qkv[:, (nH + 1) * d:].view(50, 1, d)
-    x = x + pm.attention(qq, kk, vv).reshape(50, nH * d) @ att.w_o.double().cpu().t()
+    x = x + pm.attention(qq, kk, vv).reshape(50, nH * d) @ att.w_o.rows.double().cpu().t()
     h = pm.rms_norm(x, model.blocks[0].norm_post.weight.double().cpu(), 1e-5)
     choice = (h @ moe.router.double().cpu().t()).argmax(-1)
     y = torch.stack([torch.tanh(h[i] @ moe.experts[int(choice[i])].double().cpu().t()) for i in range(50)])
     x = x + y
-    want = pm.rms_norm(x, model.final_norm.weight.double().cpu(), 1e-5) @ model.head.weight.double().cpu().t()
+    want = pm.rms_norm(x, model.final_norm.weight.double().cpu(), 1e-5) @ model.head.weight.rows.double().cpu().t()
     assert torch.allclose(whole.double(), want, rtol=1e-3, atol=1e-4)
 
 

@@ -377,6 +377,59 @@ def test_skinny_gemm_every_launch_shape_gives_the_same_product(nt, waves, unroll
     assert torch.allclose(out, want, rtol=1e-4, atol=3e-3)
 
 
+def test_tile_weights_layout():
+    """Piece (tile t, k-tile kt, 16 g + col) of the tiled copy is row 16 t + col at k = 32 kt + 8 g; padding is zero."""
+    g = gen(15)
+    N, K = 37, 72                                      # 3 row tiles (11 padded rows), 4 k-tiles (56 padded values)
+    w = torch.randn(N, K, generator=g).to(BF16)
+    t = ops.tile_weights(w.to(DEV)).cpu().float().view(3, 4, 4, 16, 8)      # [t, kt, g, col, 8]
+    want = torch.zeros(48, 128)
+    want[:N, :K] = w.float()
+    want = want.view(3, 16, 4, 4, 8).permute(0, 2, 3, 1, 4)                 # [t, col, kt, g, 8] -> [t, kt, g, col, 8]
+    assert torch.equal(t, want)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(50, 64), (3, 8), (130, 200), (577, 1000), (4608, 3584)])
+def test_skinny_gemm_from_the_tiled_copy_equals_from_rows(M, N, K):
+    g = gen(16)
+    x = torch.randn(M, K, generator=g).to(BF16).to(DEV)
+    w = torch.randn(N, K, generator=g).to(BF16).to(DEV)
+    tiled = ops.tile_weights(w)
+    want = x.double().cpu() @ w.double().cpu().t()
+    out = ops.skinny_gemm(x, w, F32, tiled=tiled).cpu().double()
+    assert torch.allclose(out, want, rtol=1e-4, atol=1e-4 * math.sqrt(K)), float((out - want).abs().max())
+    for nt, waves, unroll in [(1, 1, 4), (2, 4, 2), (1, 16, 2)]:
+        if M > 32 and nt == 2 and unroll == 4:
+            continue
+        a = ops.skinny_gemm(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled).cpu().double()
+        assert torch.allclose(a, want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
+
+
+def test_linear_weight_uses_the_copy_for_few_rows_and_the_rows_beyond():
+    g = gen(17)
+    w = torch.randn(200, 136, generator=g).to(BF16).to(DEV)
+    lw = ops.prepare_linear(w)
+    assert lw.tiled is not None and lw.rows is w
+    lw.rows = torch.zeros_like(w)                      # few rows must not read this; many rows must
+    x = torch.randn(5, 136, generator=g).to(BF16).to(DEV)
+    want = x.double().cpu() @ w.double().cpu().t()
+    assert torch.allclose(ops.linear(x, lw, out_dtype=F32).cpu().double(), want, rtol=1e-4, atol=2e-3)
+    big = torch.randn(100, 136, generator=g).to(BF16).to(DEV)
+    assert torch.all(ops.linear(big, lw) == 0)
+    pairs = ops.prepare_linear(w)
+    got = ops.linear_swiglu(x, pairs).cpu().double()
+    gt, up = want[:, 0::2], want[:, 1::2]
+    assert torch.allclose(got, gt / (1 + torch.exp(-gt)) * up, rtol=2e-2, atol=2e-2)
+    old = ops.decode_weight_copy
+    try:
+        ops.decode_weight_copy = False
+        assert ops.prepare_linear(w).tiled is None
+    finally:
+        ops.decode_weight_copy = old
+    assert ops.prepare_linear(w.float()).tiled is None  # a 32-bit weight has no copy
+
+
 def test_linear_picks_by_weight_type_and_rows():
     g = gen(13)
     w = torch.randn(96, 72, generator=g)
