@@ -46,8 +46,11 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
-    ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
-                    help="decode: the headline measurement; mixed3b / long14b: whole workloads through the scheduler")
+    ap.add_argument("--workload", choices=["decode", "prefill", *WORKLOADS], default="decode",
+                    help="decode: the headline measurement; prefill: only the 2,048-token prefill, --steps times "
+                         "(for profiles); mixed3b / long14b: whole workloads through the scheduler")
+    ap.add_argument("--no-decode-weight-copy", action="store_true",
+                    help="decode from the weights' plain rows instead of the tiled copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -71,7 +74,8 @@ def main() -> int:
 
     def note(msg):
         print(f"[bench] {msg}", file=sys.stderr, flush=True)
-    if args.workload != "decode":
+    ops.decode_weight_copy = not args.no_decode_weight_copy
+    if args.workload in WORKLOADS:
         return run_workload(args, WORKLOADS[args.workload])
     shape = dict(SHAPE_7B)
     layers_full = shape["num_hidden_layers"]
@@ -147,6 +151,15 @@ def main() -> int:
         attn = 4.0 * L * nH * d * tokens * (tokens + 1) / 2
         return tokens / best, best * 1e3, (linear + attn) / best / 1e12 / PEAK_TFLOPS[args.dtype]
 
+    if args.workload == "prefill":
+        ptps, pms, pfrac = prefill_rate(PROMPT, reps=args.steps)
+        print(json.dumps({"metric": f"prefill tok/s, {PROMPT} tokens (Qwen2.5-7B shape, {args.dtype}, random weights)",
+                          "value": round(ptps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": 1,
+                          "ms_per_step": round(pms, 3), "higher_is_better": True, "dtype": args.dtype,
+                          "config": {"model": "Qwen2.5-7B shape", "num_hidden_layers": layers_full, "layers_run": L,
+                                     "prompt_len": PROMPT, "library_gemm_tuning": not args.no_gemm_tuning},
+                          "frac_of_peak": round(pfrac, 4)}), flush=True)
+        return 0
     tps, ms, kv_mean = decode_rate(args.batch, args.steps, max(args.warmup, 1))
     note(f"batch {args.batch}: {tps:.0f} tokens/s")
     step_bytes = weight_bytes + args.batch * kv_mean * kv_bytes_per_token
@@ -160,7 +173,8 @@ def main() -> int:
                    "num_hidden_layers": layers_full, "layers_run": L, "hidden_size": H, "num_attention_heads": nH,
                    "num_key_value_heads": nKV, "head_dim": d, "intermediate_size": I, "vocab_size": V,
                    "prompt_len": PROMPT, "decode_kv_start": DECODE_KV_START, "kv_page_size": PAGE,
-                   "tie_word_embeddings": False, "library_gemm_tuning": not args.no_gemm_tuning},
+                   "tie_word_embeddings": False, "library_gemm_tuning": not args.no_gemm_tuning,
+                   "decode_weight_copy": not args.no_decode_weight_copy},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
     }

@@ -65,3 +65,42 @@ class PhaseTimer:
             parts = " ".join(f"{k}={v:.2f}" for k, v in self.step.items())
             print(f"[phase_timing] #{self.forwards} L={n_layers} tokens={n_tokens} {parts} "
                   f"total={sum(self.step.values()):.2f} ms", file=sys.stderr, flush=True)
+
+
+def kernel_trace_summary(csv_path: str, n_steps: int = 16, end_marker: str = "argmax_final") -> str:
+    """Per-kernel time per engine step from a ``rocprofv3 --kernel-trace --output-format csv`` file.
+
+    A step ends with the kernel whose name contains ``end_marker`` (the sampler's last kernel); the
+    last ``n_steps`` complete steps are averaged.  Returns the text of the table: kernels per step,
+    busy time (sum of kernel durations) and span (first start to last end) per step, then one line
+    per kernel name.
+    """
+    import collections
+    import csv
+    with open(csv_path, newline="") as f:
+        rows = sorted(csv.DictReader(f), key=lambda r: int(r["Start_Timestamp"]))
+    ends = [i for i, r in enumerate(rows) if end_marker in r["Kernel_Name"]]
+    if len(ends) < n_steps + 1:
+        raise ValueError(f"{csv_path}: {len(ends)} kernels named *{end_marker}*, need {n_steps + 1}")
+    steps = [rows[ends[k - 1] + 1: ends[k] + 1] for k in range(len(ends) - n_steps, len(ends))]
+    agg = collections.defaultdict(lambda: [0, 0])
+    span = 0
+    for st in steps:
+        span += int(st[-1]["End_Timestamp"]) - int(st[0]["Start_Timestamp"])
+        for r in st:
+            a = agg[r["Kernel_Name"][:72]]
+            a[0] += int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+            a[1] += 1
+    n = len(steps)
+    busy = sum(v[0] for v in agg.values())
+    lines = [f"steps {n}  kernels/step {sum(v[1] for v in agg.values()) / n:.0f}  busy/step {busy / n / 1e3:.1f} us  "
+             f"span/step {span / n / 1e3:.1f} us"]
+    for name, (t, c) in sorted(agg.items(), key=lambda kv: -kv[1][0]):
+        lines.append(f"{t / n / 1e3:9.1f} us/step  {c / n:6.1f} calls  {t / c / 1e3:8.2f} us each  {name}")
+    return "\n".join(lines)
+
+
+if __name__ == "__main__":
+    # python -m inferflux_amd.engine.tracing <kernel_trace.csv> [steps] [end marker]
+    print(kernel_trace_summary(sys.argv[1], int(sys.argv[2]) if len(sys.argv) > 2 else 16,
+                               sys.argv[3] if len(sys.argv) > 3 else "argmax_final"))
