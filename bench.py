@@ -218,16 +218,24 @@ def run_workload(args, w) -> int:
         if rid not in first:
             first[rid] = time.perf_counter() - t0
 
+    sp = SamplingParams(temperature=0.0, max_tokens=w["new"], ignore_eos=True)
+    if args.warmup > 0:
+        # One untimed pass of the same workload: the library loads a kernel the first time a shape asks
+        # for it, which costs up to a second per shape and has nothing to do with the steady state.
+        eng.generate(prompts, SamplingParams(**vars(sp)))
+        eng.stats = type(eng.stats)()
+        print("[bench] warm-up pass done", file=sys.stderr, flush=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=w["new"], ignore_eos=True), on_token)
+    outs = eng.generate(prompts, sp, on_token)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     n_gen = sum(len(o.token_ids) for o in outs)
     ttft = sorted(first.values())
     out = {
         "metric": f"generated tok/s, {w['requests']} requests, prompts {lo}-{hi}, {w['new']} new tokens each ({w['name']}, {args.dtype}, random weights)",
-        "value": round(n_gen / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": eng.stats.steps, "warmup": 0,
+        "value": round(n_gen / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": eng.stats.steps,
+        "warmup": 1 if args.warmup > 0 else 0,
         "ms_per_step": round(dt / eng.stats.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (uniform random token ids, seeded N(0,0.02) weights)",
         "config": {"model": w["name"], "global_batch": w["requests"], "seq_len": hi + w["new"], "parallelism": "1 GPU",
