@@ -66,16 +66,27 @@ __device__ __forceinline__ bf16x4 zero4() {
 // normal float may flush to zero, which a softmax weight of that size may.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// max over the four lanes that hold the same query column (lane, lane^16, lane^32, lane^48)
+// The four lanes that hold the same query column are lane, lane^16, lane^32, lane^48: one lane of each
+// row of 16.  gfx950 exchanges rows between two registers in one VALU instruction (permlane16_swap: odd
+// rows of the first with even rows of the second; permlane32_swap: rows 2, 3 of the first with rows 0, 1
+// of the second); given the same value twice, the two results hold v and v from the partner lane.
+__device__ __forceinline__ void swap16(float v, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void swap32(float v, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+}
 __device__ __forceinline__ float col_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, WAVE));
-  v = fmaxf(v, __shfl_xor(v, 32, WAVE));
-  return v;
+  float a, b;
+  swap16(v, a, b); v = fmaxf(a, b);
+  swap32(v, a, b); return fmaxf(a, b);
 }
 __device__ __forceinline__ float col_sum(float v) {
-  v += __shfl_xor(v, 16, WAVE);
-  v += __shfl_xor(v, 32, WAVE);
-  return v;
+  float a, b;
+  swap16(v, a, b); v = a + b;
+  swap32(v, a, b); return a + b;
 }
 
 // =======================================================================================
@@ -461,16 +472,23 @@ __device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, 
     pop[qt][1] = join4(pb[2], pb[3]);
     rescale = rescale || __any(alpha[qt] != 1.0f);   // once the running maxima have settled nothing is rescaled
   }
+  if (rescale) {
+    // The empty statement keeps this a branch the whole wave takes or skips: as straight-line code
+    // (multiply and select per element) it would be nearly half of the tile's vector instructions.
+    asm volatile("");
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q[qt].o[dt][r] *= alpha[qt];
+  }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const bf16_t* vr = v_s + (16 * dt + col) * VPAD + 8 * g4;
     const bf16x8 vop0 = *(const bf16x8*)(vr), vop1 = *(const bf16x8*)(vr + 32);
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
-      if (rescale) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) q[qt].o[dt][r] *= alpha[qt];
-      }
       q[qt].o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0, pop[qt][0], q[qt].o[dt], 0, 0, 0);
       q[qt].o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1, pop[qt][1], q[qt].o[dt], 0, 0, 0);
     }

@@ -16,7 +16,6 @@ import torch
 from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
-TILE_QT2_MIN_WORKGROUPS = 512   # the chip holds 2 workgroups of the tile kernel on each of its 256 CUs
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 64  # and until a row has at most this many splits
@@ -57,10 +56,10 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
     n_kv = cache.k.shape[1]
-    # two query tiles per wave when that still leaves enough workgroups to fill the chip
-    big = ops.attention_tile_rows(d, 2)
-    n_big = sum(-(-int(n) // big) for n in ctx.h_q_len if n >= TILE_MIN)
-    qt = 2 if n_big * nH >= TILE_QT2_MIN_WORKGROUPS else 1
+    # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often
+    # and were faster at every length measured (256 to 8,192 rows, 28 heads); one tile per wave only
+    # when no request brings more rows than one such workgroup's half.
+    qt = 2 if int(ctx.h_q_len.max(initial=0)) > ops.attention_tile_rows(d, 1) else 1
     tile_rows = ops.attention_tile_rows(d, qt)
     w = ctx.derived(("attention_work_lists", n_kv, tile_rows), lambda: _work_lists(ctx, n_kv, tile_rows))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
