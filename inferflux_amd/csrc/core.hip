@@ -283,6 +283,84 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   }
 }
 
+// The common case in 16-byte pieces: bfloat16, split-half pairs over the whole head, head size a
+// multiple of 16, bias bfloat16 or none.  The first n_qk_blocks blocks rotate q and k: a thread takes 8
+// consecutive dimensions of the first half of a head and their 8 partners in the second.  The other
+// blocks append v: a thread takes one dimension of one kv head for 8 consecutive tokens and, when
+// their slots are 8 consecutive offsets of one page starting at a multiple of 8, writes them as one
+// piece of the transposed page; otherwise element by element.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 rope_bf16x8;
+
+__global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T, int n_qk_blocks) {
+  const int d = a.d, half = d / 2;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
+  const bf16_t* qkv = (const bf16_t*)a.qkv;
+  const bf16_t* bias = (const bf16_t*)a.bias;
+  if ((int)blockIdx.x < n_qk_blocks) {
+    const int per_head = d / 16, heads = a.nH + (a.slots ? a.nKV : 0);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)T * heads * per_head) return;
+    const int j = (int)(idx % per_head), head = (int)(idx / per_head % heads), t = (int)(idx / per_head / heads);
+    const int col = head * d + 8 * j;
+    const bf16_t* row = qkv + (size_t)t * row_width + col;
+    rope_bf16x8 x0 = *(const rope_bf16x8*)row, x1 = *(const rope_bf16x8*)(row + half);
+    float f0[8], f1[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { f0[e] = (float)x0[e]; f1[e] = (float)x1[e]; }
+    if (bias) {
+      const rope_bf16x8 b0 = *(const rope_bf16x8*)(bias + col), b1 = *(const rope_bf16x8*)(bias + col + half);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { f0[e] += (float)b0[e]; f1[e] += (float)b1[e]; }
+    }
+    const float* cs = a.cs + (size_t)t * half + 8 * j;
+    const float* sn = a.sn + (size_t)t * half + 8 * j;
+    rope_bf16x8 y0, y1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      y0[e] = (__bf16)(f0[e] * cs[e] - f1[e] * sn[e]);
+      y1[e] = (__bf16)(f0[e] * sn[e] + f1[e] * cs[e]);
+    }
+    bf16_t* dst;
+    if (head < a.nH) {
+      dst = (bf16_t*)a.q_out + (size_t)t * q_width + col;
+    } else {
+      const int slot = a.slots[t];
+      if (slot < 0) return;
+      const int page = slot / a.page_size, off = slot % a.page_size;
+      dst = (bf16_t*)a.k_cache + (((size_t)page * a.nKV + (head - a.nH)) * a.page_size + off) * d + 8 * j;
+    }
+    *(rope_bf16x8*)dst = y0;
+    *(rope_bf16x8*)(dst + half) = y1;
+    return;
+  }
+  // v: (group of 8 tokens, kv head, dimension)
+  const size_t idx = (size_t)(blockIdx.x - n_qk_blocks) * 256 + threadIdx.x;
+  const int groups = (T + 7) / 8;
+  if (idx >= (size_t)groups * a.nKV * d) return;
+  const int e = (int)(idx % d), kh = (int)(idx / d % a.nKV), t0 = (int)(idx / d / a.nKV) * 8;
+  const int col = q_width + kv_width + kh * d + e;
+  const float b = bias ? (float)bias[col] : 0.f;
+  const int n = min(8, T - t0);
+  const int s0 = a.slots[t0];
+  bool run = n == 8 && s0 >= 0 && s0 % 8 == 0;
+  for (int k = 1; k < 8 && run; ++k) run = a.slots[t0 + k] == s0 + k;
+  if (run) {
+    rope_bf16x8 v;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = (__bf16)((float)qkv[(size_t)(t0 + k) * row_width + col] + b);
+    const int page = s0 / a.page_size, off = s0 % a.page_size;
+    *(rope_bf16x8*)((bf16_t*)a.v_cache + (((size_t)page * a.nKV + kh) * d + e) * a.page_size + off) = v;
+  } else {
+    for (int k = 0; k < n; ++k) {
+      const int slot = a.slots[t0 + k];
+      if (slot < 0) continue;
+      const int page = slot / a.page_size, off = slot % a.page_size;
+      ((bf16_t*)a.v_cache)[(((size_t)page * a.nKV + kh) * d + e) * a.page_size + off] =
+          (__bf16)((float)qkv[(size_t)(t0 + k) * row_width + col] + b);
+    }
+  }
+}
+
 extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const int* slots,
                                const float* cs, const float* sn, int rope_style, int rotary_dim, int T, int nH,
                                int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, void* stream) {
@@ -295,6 +373,15 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   if (T == 0) return 0;
   RopeArgs a{qkv, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
   hipStream_t s = (hipStream_t)stream;
+  // (a few tokens are quicker with one small block per token and head: nothing waits on a loop over tokens)
+  if (T >= 64 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
+      (!slots || page_size % 8 == 0)) {
+    const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
+    const size_t v_threads = slots ? (size_t)((T + 7) / 8) * nKV * d : 0;
+    const unsigned qk_blocks = (unsigned)((qk_threads + 255) / 256), v_blocks = (unsigned)((v_threads + 255) / 256);
+    hipLaunchKernelGGL(rope_append_vec_kernel, dim3(qk_blocks + v_blocks), dim3(256), 0, s, a, T, (int)qk_blocks);
+    IFX_LAUNCH_CHECK();
+  }
   const dim3 grid(T, nH + 2 * nKV);
   if (dtype == DT_F32) hipLaunchKernelGGL(rope_append_kernel<float>, grid, dim3(64), 0, s, a);
   else if (dtype == DT_BF16) hipLaunchKernelGGL(rope_append_kernel<bf16_t>, grid, dim3(64), 0, s, a);

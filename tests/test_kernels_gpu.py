@@ -111,6 +111,39 @@ def test_rope_append(dtype, style, rot, bias):
     assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P, -1)[~written] == 0)
 
 
+@pytest.mark.parametrize("d,nH,nKV", [(16, 3, 1), (32, 4, 2), (128, 7, 1)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_rope_append_in_pieces(d, nH, nKV, bias):
+    """bfloat16, split-half over the whole head, head size a multiple of 16: the kernel's 16-byte path.  Slots:
+    an aligned run of 16 (written as pieces of the transposed page), a run that starts at an odd offset, scattered
+    ones, one token without a slot."""
+    g = gen(31)
+    T, P, pages, theta = 69, 16, 12, 1e4
+    width = (nH + 2 * nKV) * d
+    qkv = torch.randn(T, width, generator=g).to(BF16)
+    b = (0.5 * torch.randn(width, generator=g)).to(BF16) if bias else None
+    positions = torch.cat([torch.arange(100, 116), torch.arange(3, 11), torch.randint(0, 2000, (45,), generator=g)]).to(torch.int32)
+    scattered = (48 + torch.randperm(pages * P - 48, generator=g)[:45]).tolist()
+    slots = torch.tensor(list(range(32, 48)) + list(range(3, 11)) + scattered, dtype=torch.int32)
+    slots[30] = -1
+    kc = torch.zeros(pages, nKV, P, d, dtype=BF16, device=DEV)
+    vc = torch.zeros(pages, nKV, d, P, dtype=BF16, device=DEV)
+    inv_freq = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64), 2.0 * torch.arange(d // 2, dtype=torch.float64) / d)).float()
+    cs, sn = ops.rope_table(positions.to(DEV), inv_freq.to(DEV))
+    q = ops.rope_append(qkv.to(DEV), b.to(DEV) if bias else None, slots.to(DEV), cs, sn, ops.ROPE_SPLIT_HALF, d, nH, nKV, d, kc, vc, P)
+    x = qkv.double() + (b.double() if bias else 0)
+    xq, xk, xv = x[:, : nH * d].view(T, nH, d), x[:, nH * d: (nH + nKV) * d].view(T, nKV, d), x[:, (nH + nKV) * d:].view(T, nKV, d)
+    t = dict(rtol=tol(BF16)["rtol"], atol=tol(BF16)["atol"] + 2e-4)
+    assert torch.allclose(q.cpu().double(), pm.rope_split_half(xq, positions.tolist(), theta), **t)
+    live = slots >= 0
+    k_got, v_got = cache_rows(kc.cpu(), vc.cpu(), slots[live], P)
+    assert torch.allclose(k_got.double(), pm.rope_split_half(xk, positions.tolist(), theta)[live], **t)
+    assert torch.allclose(v_got.double(), xv[live], **tol(BF16))
+    written = torch.zeros(pages * P, dtype=torch.bool); written[slots[live].long()] = True
+    assert torch.all(kc.cpu().permute(0, 2, 1, 3).reshape(pages * P, -1)[~written] == 0)   # nothing else touched
+    assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P, -1)[~written] == 0)
+
+
 def test_rope_queries_only():
     g = gen(4)
     T, nH, d = 4, 3, 16
