@@ -340,23 +340,29 @@ __global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T,
   const int e = (int)(idx % d), kh = (int)(idx / d % a.nKV), t0 = (int)(idx / d / a.nKV) * 8;
   const int col = q_width + kv_width + kh * d + e;
   const float b = bias ? (float)bias[col] : 0.f;
-  const int n = min(8, T - t0);
-  const int s0 = a.slots[t0];
-  bool run = n == 8 && s0 >= 0 && s0 % 8 == 0;
-  for (int k = 1; k < 8 && run; ++k) run = a.slots[t0 + k] == s0 + k;
+  int slot[8];
+  float x[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {   // all loads of the group are independent: they go out together
+    slot[k] = t0 + k < T ? a.slots[t0 + k] : -1;
+    x[k] = t0 + k < T ? (float)qkv[(size_t)(t0 + k) * row_width + col] + b : 0.f;
+  }
+  bool run = slot[0] >= 0 && slot[0] % 8 == 0;
+#pragma unroll
+  for (int k = 1; k < 8; ++k) run = run && slot[k] == slot[0] + k;
+  bf16_t* vc = (bf16_t*)a.v_cache;
   if (run) {
     rope_bf16x8 v;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] = (__bf16)((float)qkv[(size_t)(t0 + k) * row_width + col] + b);
-    const int page = s0 / a.page_size, off = s0 % a.page_size;
-    *(rope_bf16x8*)((bf16_t*)a.v_cache + (((size_t)page * a.nKV + kh) * d + e) * a.page_size + off) = v;
+    for (int k = 0; k < 8; ++k) v[k] = (__bf16)x[k];
+    const int page = slot[0] / a.page_size, off = slot[0] % a.page_size;
+    *(rope_bf16x8*)(vc + (((size_t)page * a.nKV + kh) * d + e) * a.page_size + off) = v;
   } else {
-    for (int k = 0; k < n; ++k) {
-      const int slot = a.slots[t0 + k];
-      if (slot < 0) continue;
-      const int page = slot / a.page_size, off = slot % a.page_size;
-      ((bf16_t*)a.v_cache)[(((size_t)page * a.nKV + kh) * d + e) * a.page_size + off] =
-          (__bf16)((float)qkv[(size_t)(t0 + k) * row_width + col] + b);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (slot[k] < 0) continue;
+      const int page = slot[k] / a.page_size, off = slot[k] % a.page_size;
+      vc[(((size_t)page * a.nKV + kh) * d + e) * a.page_size + off] = (__bf16)x[k];
     }
   }
 }
