@@ -16,6 +16,7 @@ import torch
 from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
+TILE_QT2_MIN_WORKGROUPS = 512   # two workgroups of the tile kernel for each of the 256 compute units
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 64  # and until a row has at most this many splits
@@ -56,10 +57,12 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
     n_kv = cache.k.shape[1]
-    # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often
-    # and were faster at every length measured (256 to 8,192 rows, 28 heads); one tile per wave only
-    # when no request brings more rows than one such workgroup's half.
-    qt = 2 if int(ctx.h_q_len.max(initial=0)) > ops.attention_tile_rows(d, 1) else 1
+    # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often;
+    # they win once they still give two workgroups for each compute unit (measured with 28 heads: equal
+    # at 2,048 rows, 5 % faster at 4,096, 30 % at 8,192; one tile per wave is ahead below).
+    big = ops.attention_tile_rows(d, 2)
+    n_big = sum(-(-int(n) // big) for n in ctx.h_q_len if n >= TILE_MIN)
+    qt = 2 if n_big * nH >= TILE_QT2_MIN_WORKGROUPS else 1
     tile_rows = ops.attention_tile_rows(d, qt)
     w = ctx.derived(("attention_work_lists", n_kv, tile_rows), lambda: _work_lists(ctx, n_kv, tile_rows))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)

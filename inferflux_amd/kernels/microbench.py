@@ -1,0 +1,122 @@
+"""Timings of single kernels at chosen sizes, for profiles and for tuning launch shapes.
+
+    python -m inferflux_amd.kernels.microbench attention-tiles --rows 8192 [--query-tiles 2]
+    python -m inferflux_amd.kernels.microbench attention-rows --batch 64 --context 3072 [--chunk 512]
+    python -m inferflux_amd.kernels.microbench gemm --rows 8 [--shape gate_up]
+
+Sizes default to the Qwen2.5-7B shape (28 query heads, 4 kv heads, head size 128, hidden 3584,
+intermediate 18944).  Times are averages of back-to-back launches between two events and include what
+the Python wrapper costs per call (10-15 us): for kernels that short, read the kernel's own time from
+``rocprofv3 --kernel-trace`` around this program instead.  Products rotate through enough copies of the
+weight that no launch finds it in a cache.
+"""
+from __future__ import annotations
+
+import argparse
+import math
+import sys
+
+import torch
+
+from . import ops
+
+GEMM_SHAPES = {"qkv": (4608, 3584), "o": (3584, 3584), "gate_up": (37888, 3584), "down": (3584, 18944),
+               "lm_head": (152064, 3584)}
+
+
+def _time_us(fn, iters: int) -> float:
+    for i in range(3):
+        fn(i)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(iters):
+        fn(i + 3)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters * 1e3
+
+
+def attention_tiles(args) -> None:
+    dev, T, nH, nKV, d, P = "cuda", args.rows, args.heads, args.kv_heads, args.head_dim, args.page_size
+    q = torch.randn(T, nH, d, device=dev, dtype=torch.bfloat16)
+    nb = -(-T // P)
+    kc = torch.randn(nb, nKV, P, d, device=dev, dtype=torch.bfloat16)
+    vc = torch.randn(nb, nKV, d, P, device=dev, dtype=torch.bfloat16)
+    table = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    for qt in ([args.query_tiles] if args.query_tiles else list(ops.TILE_QTS)):
+        tiles = list(range(0, T, ops.attention_tile_rows(d, qt)))
+        out = torch.empty(T, nH * d, device=dev, dtype=torch.bfloat16)
+        call = (q, kc, vc, out, i32([0] * len(tiles)), i32(tiles), i32([0]), i32([T]), i32([T]), table, None, 1 / math.sqrt(d), qt)
+        t = _time_us(lambda i: ops.attention_tiles(*call), args.iters)
+        flops = 4.0 * nH * d * T * (T + 1) / 2
+        print(f"attention-tiles rows={T} query_tiles={qt}: {t:9.1f} us  {flops / t / 1e6:7.1f} TFLOP/s (causal half only)", flush=True)
+
+
+def attention_rows(args) -> None:
+    dev, B, kv, nH, nKV, d, P = "cuda", args.batch, args.context, args.heads, args.kv_heads, args.head_dim, args.page_size
+    nb = -(-kv // P)
+    kc = torch.randn(B * nb, nKV, P, d, device=dev, dtype=torch.bfloat16)
+    vc = torch.randn(B * nb, nKV, d, P, device=dev, dtype=torch.bfloat16)
+    table = torch.randperm(B * nb, device=dev).to(torch.int32).view(B, nb).contiguous()
+    q = torch.randn(B, nH, d, device=dev, dtype=torch.bfloat16)
+    out = torch.empty(B, nH * d, device=dev, dtype=torch.bfloat16)
+    row_req = torch.arange(B, dtype=torch.int32, device=dev)
+    pos = torch.full((B,), kv - 1, dtype=torch.int32, device=dev)
+    for chunk in ([args.chunk] if args.chunk else [128, 256, 512, 1024]):
+        splits = -(-kv // chunk)
+        t = _time_us(lambda i: ops.attention_rows(q, kc, vc, out, None, B, row_req, pos, table, None, 1 / math.sqrt(d), chunk, splits),
+                     args.iters)
+        gb = B * kv * nKV * d * 2 * 2 / 1e9
+        print(f"attention-rows batch={B} context={kv} chunk={chunk} splits={splits}: {t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache "
+              f"(row kernel + merge)", flush=True)
+
+
+def gemm(args) -> None:
+    dev, M = "cuda", args.rows
+    for name in ([args.shape] if args.shape else list(GEMM_SHAPES)):
+        N, K = GEMM_SHAPES[name]
+        copies = max(2, min(24, int(3e9 // (N * K * 2))))
+        ws = [ops.prepare_linear(torch.randn(N, K, device=dev, dtype=torch.bfloat16)) for _ in range(copies)]
+        x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+        gb = N * K * 2 / 1e9
+        t = _time_us(lambda i: ops.linear(x, ws[i % copies]), args.iters)
+        t_lib = _time_us(lambda i: torch.matmul(x, ws[i % copies].rows.t()), args.iters)
+        print(f"gemm {name:8s} rows={M:3d} [{N} x {K}]: engine's choice {t:8.1f} us ({gb / t * 1e3:5.2f} TB/s of weights)   "
+              f"library {t_lib:8.1f} us", flush=True)
+        del ws
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="python -m inferflux_amd.kernels.microbench")
+    sub = ap.add_subparsers(dest="what", required=True)
+    for name, fn in (("attention-tiles", attention_tiles), ("attention-rows", attention_rows), ("gemm", gemm)):
+        p = sub.add_parser(name)
+        p.set_defaults(fn=fn)
+        p.add_argument("--iters", type=int, default=10)
+        if name.startswith("attention"):
+            p.add_argument("--heads", type=int, default=28)
+            p.add_argument("--kv-heads", type=int, default=4)
+            p.add_argument("--head-dim", type=int, default=128)
+            p.add_argument("--page-size", type=int, default=16)
+        if name == "attention-tiles":
+            p.add_argument("--rows", type=int, default=2048, help="rows of one request in one step, no past")
+            p.add_argument("--query-tiles", type=int, default=0, help="1 or 2 query tiles per wave (0: both)")
+        if name == "attention-rows":
+            p.add_argument("--batch", type=int, default=8)
+            p.add_argument("--context", type=int, default=3072)
+            p.add_argument("--chunk", type=int, default=0, help="keys per split (0: 128, 256, 512 and 1024)")
+        if name == "gemm":
+            p.add_argument("--rows", type=int, default=8, help="rows of x")
+            p.add_argument("--shape", choices=list(GEMM_SHAPES), default=None)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        print("microbench: no GPU", file=sys.stderr)
+        return 2
+    args.fn(args)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -30,7 +30,8 @@ ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
 MFMA_HEAD_DIMS_PREBUILT = (16, 32, 64, 128)
 MFMA_MAX_HEAD_DIM = 128
 # Query tiles of 16 rows per wave in the tile kernel: 2 (128 rows per workgroup) reuses each key and
-# value operand twice; 1 (64 rows) for portions that would leave half of such a workgroup empty.
+# value operand twice and is faster once there are enough workgroups to fill the chip; 1 (64 rows)
+# gives twice as many workgroups for short portions.
 TILE_QTS = (1, 2)
 
 
