@@ -400,7 +400,7 @@ def test_skinny_gemm(M, N, K, out_dtype):
     assert torch.allclose(out, want, **t), float((out - want).abs().max())
 
 
-@pytest.mark.parametrize("nt,waves,unroll", [(1, 1, 4), (2, 4, 2), (1, 16, 2), (2, 8, 4), (1, 3, 8)])
+@pytest.mark.parametrize("nt,waves,unroll", [(1, 1, 4), (2, 4, 2), (1, 16, 2), (2, 8, 4), (1, 3, 4)])
 def test_skinny_gemm_every_launch_shape_gives_the_same_product(nt, waves, unroll):
     g = gen(12)
     x = torch.randn(9, 1096, generator=g).to(BF16)
@@ -432,8 +432,11 @@ def test_skinny_gemm_from_the_tiled_copy_equals_from_rows(M, N, K):
     want = x.double().cpu() @ w.double().cpu().t()
     out = ops.skinny_gemm(x, w, F32, tiled=tiled).cpu().double()
     assert torch.allclose(out, want, rtol=1e-4, atol=1e-4 * math.sqrt(K)), float((out - want).abs().max())
+    mt = (M + 15) // 16
     for nt, waves, unroll in [(1, 1, 4), (2, 4, 2), (1, 16, 2)]:
-        if M > 32 and nt == 2 and unroll == 4:
+        if (mt >= 3 and unroll == 4) or (mt == 4 and nt == 2):     # shapes the kernel is not built for
+            with pytest.raises(ops.KernelError, match="no kernel"):
+                ops.skinny_gemm(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled)
             continue
         a = ops.skinny_gemm(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled).cpu().double()
         assert torch.allclose(a, want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
