@@ -105,6 +105,7 @@ struct RowArgs {
   bf16_t* out;            // [T, nH * D]
   int max_blocks, n_rows, nH, nKV, P, window, chunk, max_splits;
   float scale_log2e;
+  int part_by_row;        // partial results lie at the batch row's number (the tile kernel's), not at its place in ``rows``
 };
 
 // The operands of one block of 32 keys (two pages' worth of 16): loaded together, K and V at once,
@@ -239,8 +240,9 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
   const int pos = a.positions[row];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int s0 = lo / a.chunk, s1 = pos / a.chunk;  // first and last split that hold a visible key
-  const float* po = a.part_o + ((size_t)ri * a.nH + head) * a.max_splits * D;
-  const float* pml = a.part_ml + ((size_t)ri * a.nH + head) * a.max_splits * 2;
+  const size_t pi = a.part_by_row ? row : ri;
+  const float* po = a.part_o + (pi * a.nH + head) * a.max_splits * D;
+  const float* pml = a.part_ml + (pi * a.nH + head) * a.max_splits * 2;
   float acc[(D + WAVE - 1) / WAVE];
 #pragma unroll
   for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = 0.f;
@@ -301,7 +303,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   if (n_rows == 0) return 0;
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-            scale * 1.4426950408889634f};
+            scale * 1.4426950408889634f, 0};
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(attn_rows_kernel, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
   hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, a);
@@ -338,7 +340,13 @@ struct TileArgs {
   int max_blocks, nH, nKV, P, window;
   float scale_log2e;
   int page_shift;         // log2(P): the tile kernel takes power-of-two pages and splits positions by shift and mask
-  int n_tiles, per_xcd;   // work items are (tile, head); per_xcd = ceil(n_tiles * nH / 8)
+  int n_tiles, per_xcd;   // work items are (tile, head, split); per_xcd = ceil(n_tiles * nH * max_splits / 8)
+  // With max_splits > 1 a workgroup takes only the keys [split * chunk, (split + 1) * chunk) (chunk a multiple of
+  // 64) and writes unnormalised partial results in the row kernel's format, at the batch row's number; the
+  // row kernel's merge finishes them.  For portions of prompts with a long past: few tiles, many keys.
+  int chunk, max_splits;
+  float* part_o;          // [T, nH, max_splits, D]
+  float* part_ml;         // [T, nH, max_splits, 2]
 };
 
 constexpr int N_PIECES = TK * (D / 8);                // 16-byte pieces of a K tile, and as many of a V^T tile
@@ -516,8 +524,9 @@ void attn_tiles_kernel(TileArgs a) {
   // workgroups that read one kv head's keys and values share an L2 instead of filling all eight with
   // everything; within a run the tiles with the most keys (the latest rows) come first.
   const int ratio = a.nH / a.nKV;
-  const int item = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
-  if (blockIdx.x / 8 >= a.per_xcd || item >= a.n_tiles * a.nH) return;   // the whole workgroup leaves together
+  const int work = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
+  if (blockIdx.x / 8 >= a.per_xcd || work >= a.n_tiles * a.nH * a.max_splits) return;   // the whole workgroup leaves together
+  const int item = work / a.max_splits, split = work % a.max_splits;
   const int per_kv = ratio * a.n_tiles;
   const int kvh = item / per_kv, rem = item % per_kv;
   const int head = kvh * ratio + rem / a.n_tiles, ti = a.n_tiles - 1 - rem % a.n_tiles;
@@ -526,8 +535,10 @@ void attn_tiles_kernel(TileArgs a) {
   const int start = kvlen - qlen;                       // position of the request's first row in this step
   const int* table = a.block_table + (size_t)req * a.max_blocks;
   const int rows_here = min(TQ, qlen - q0);
-  const int pos_first = start + q0, pos_last = pos_first + rows_here - 1;
-  const int lo_wg = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+  const int pos_first = start + q0, row_last = pos_first + rows_here - 1;
+  // the keys of this workgroup: what its rows can see, cut to its split
+  const int lo_wg = max(a.window > 0 ? max(0, pos_first - a.window + 1) : 0, a.max_splits > 1 ? split * a.chunk : 0);
+  const int pos_last = a.max_splits > 1 ? min(row_last, (split + 1) * a.chunk - 1) : row_last;
 
   // this wave's rows: QT tiles of 16, lane `col` of tile qt holds row 16 * QT * wid + 16 * qt + col of the tile
   const int wave_q = q0 + 16 * QT * wid;
@@ -551,7 +562,7 @@ void attn_tiles_kernel(TileArgs a) {
   }
   // the keys this wave's rows can see at all: tiles outside are skipped by the whole wave
   const int wave_first = start + wave_q;
-  const int wave_hi = min(pos_last, wave_first + 16 * QT - 1);
+  const int wave_hi = min(row_last, wave_first + 16 * QT - 1);
   const int wave_lo = a.window > 0 ? max(0, wave_first - a.window + 1) : 0;
 
   TileRegs regs;
@@ -577,9 +588,17 @@ void attn_tiles_kernel(TileArgs a) {
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const float l = col_sum(q[qt].l);
-    if (q[qt].ok) {
+    if (!q[qt].ok) continue;
+    const size_t row = row0 + wave_q + 16 * qt + col;
+    if (a.max_splits > 1) {
+      float* po = a.part_o + ((row * a.nH + head) * a.max_splits + split) * D;
+      float* pml = a.part_ml + ((row * a.nH + head) * a.max_splits + split) * 2;
+      if (g4 == 0) { pml[0] = q[qt].m * a.scale_log2e; pml[1] = l; }   // -inf stays -inf: nothing of this split was visible
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = q[qt].o[dt];
+    } else {
       const float inv = l > 0.f ? 1.f / l : 0.f;
-      bf16_t* orow = a.out + ((row0 + wave_q + 16 * qt + col) * a.nH + head) * D;
+      bf16_t* orow = a.out + (row * a.nH + head) * D;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         bf16x4 w;
@@ -591,24 +610,41 @@ void attn_tiles_kernel(TileArgs a) {
   }
 }
 
+// chunk / max_splits / part_o / part_ml / rows / n_rows / positions: with max_splits > 1 the keys are cut into
+// splits of ``chunk`` (a multiple of 64; max_splits * chunk reaches past the largest position), the partial
+// results go to part_o [T, nH, max_splits, D] and part_ml [T, nH, max_splits, 2], and the rows named by ``rows``
+// (every row of every tiled request, n_rows of them) are merged into ``out`` at the end.
 extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_cache, void* out,
                               const int* tile_req, const int* tile_q0, int n_tiles, const int* q_start,
                               const int* q_len, const int* kv_len, const int* block_table, int max_blocks,
-                              int nH, int nKV, int d, int page_size, int window, float scale, void* stream) {
+                              int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
+                              float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
+                              const int* positions, void* stream) {
   IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_tiles: page_size %d must be a multiple of 16", page_size);
   IFX_REQUIRE(nH <= 65535, "attn_tiles: too many heads for one launch");
   IFX_REQUIRE((page_size & (page_size - 1)) == 0, "attn_tiles: page_size %d must be a power of two", page_size);
+  IFX_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attn_tiles: bad number of splits %d", max_splits);
+  IFX_REQUIRE(max_splits == 1 || (chunk > 0 && chunk % TK == 0 && part_o && part_ml && rows && positions && row_req && n_rows > 0),
+              "attn_tiles: %d splits need a chunk that is a multiple of %d (got %d), scratch, and the rows to merge", max_splits,
+              TK, chunk);
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   if (n_tiles == 0) return 0;
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
-             n_tiles, 0};
-  const long long items = (long long)n_tiles * nH;
+             n_tiles, 0, chunk, max_splits, part_o, part_ml};
+  const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
   a.per_xcd = (int)((items + 7) / 8);
-  hipLaunchKernelGGL(attn_tiles_kernel, dim3(8 * a.per_xcd), dim3(256), 0, (hipStream_t)stream, a);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(attn_tiles_kernel, dim3(8 * a.per_xcd), dim3(256), 0, s, a);
+  if (max_splits > 1) {
+    RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
+              part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
+              scale * 1.4426950408889634f, 1};
+    hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, m);
+  }
   IFX_LAUNCH_CHECK();
 }

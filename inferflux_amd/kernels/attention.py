@@ -17,12 +17,16 @@ from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
 TILE_QT2_MIN_WORKGROUPS = 512   # two workgroups of the tile kernel for each of the 256 compute units
+TILE_SPLIT_BELOW = 256          # fewer workgroups than compute units: the tile kernel splits the keys
+TILE_SPLIT_TARGET = 512         # ... aiming at this many workgroups,
+TILE_SPLIT_MIN_KEYS = 256       # with at least this many keys to a split
+TILE_MAX_SPLITS = 16
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 64  # and until a row has at most this many splits
 
 
-def _work_lists(ctx, ctx_kv_heads, tile_rows):
+def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads):
     """What the kernels need beyond the step's own arrays, computed once per step (and per number of
     kv heads, which decides how many waves a launch has)."""
     q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
@@ -33,10 +37,21 @@ def _work_lists(ctx, ctx_kv_heads, tile_rows):
             tile_req.append(r); tile_q0.append(q0)
     row_mask = ~tiled[ctx.h_row_req] if ctx.n_tokens else np.zeros(0, bool)
     rows = np.nonzero(row_mask)[0].astype(np.int32)
-    out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1}
+    out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1,
+           "tile_splits": 1, "tile_chunk": 0, "tile_row_list": None}
     if tile_req:
         out["tile_req"] = ctx.upload(np.asarray(tile_req, np.int32))
         out["tile_q0"] = ctx.upload(np.asarray(tile_q0, np.int32))
+        # Few tiles with many keys each (portions of prompts with a long past) leave most of the chip idle
+        # and each workgroup walking its keys alone: cut the keys into splits that run side by side.
+        groups = len(tile_req) * n_heads
+        longest = int(kv_len[tiled].max())
+        if groups < TILE_SPLIT_BELOW and longest >= 2 * TILE_SPLIT_MIN_KEYS:
+            want = min(-(-TILE_SPLIT_TARGET // groups), longest // TILE_SPLIT_MIN_KEYS, TILE_MAX_SPLITS)
+            chunk = (-(-longest // want) + 63) // 64 * 64
+            out["tile_splits"], out["tile_chunk"] = -(-longest // chunk), chunk
+            if out["tile_splits"] > 1:
+                out["tile_row_list"] = ctx.upload(np.nonzero(~row_mask)[0].astype(np.int32))
     if rows.size:
         if rows.size != ctx.n_tokens:
             out["rows"] = ctx.upload(rows)
@@ -64,11 +79,12 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     n_big = sum(-(-int(n) // big) for n in ctx.h_q_len if n >= TILE_MIN)
     qt = 2 if n_big * nH >= TILE_QT2_MIN_WORKGROUPS else 1
     tile_rows = ops.attention_tile_rows(d, qt)
-    w = ctx.derived(("attention_work_lists", n_kv, tile_rows), lambda: _work_lists(ctx, n_kv, tile_rows))
+    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH), lambda: _work_lists(ctx, n_kv, tile_rows, nH))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
-                            table, window, scale, qt)
+                            table, window, scale, qt, w["tile_chunk"], w["tile_splits"], w["tile_row_list"], ctx.row_req,
+                            ctx.positions)
     if w["n_rows"]:
         ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
                            window, scale, w["chunk"], w["max_splits"])

@@ -58,17 +58,25 @@ def _dt(t: torch.Tensor) -> int:
 
 
 def _check(t: torch.Tensor, name: str, shape=None, dtype=None) -> None:
-    if not isinstance(t, torch.Tensor):
-        raise KernelError(f"{name}: not a tensor")
-    if not t.is_cuda:
-        raise KernelError(f"{name}: tensor is on {t.device}; the kernels run on the GPU only")
-    if not t.is_contiguous():
+    # on every launch: written for the case that nothing is wrong
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous()):
+        if not isinstance(t, torch.Tensor):
+            raise KernelError(f"{name}: not a tensor")
+        if not t.is_cuda:
+            raise KernelError(f"{name}: tensor is on {t.device}; the kernels run on the GPU only")
         raise KernelError(f"{name}: tensor is not contiguous")
     if dtype is not None and t.dtype != dtype:
         raise KernelError(f"{name}: element type {t.dtype}, expected {dtype}")
     if shape is not None:
-        if len(shape) != t.dim() or any(s is not None and s != ts for s, ts in zip(shape, t.shape)):
-            raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        ts = t.shape
+        ok = len(shape) == len(ts)
+        if ok:
+            for want, got in zip(shape, ts):
+                if want is not None and want != got:
+                    ok = False
+                    break
+        if not ok:
+            raise KernelError(f"{name}: shape {tuple(ts)}, expected {tuple(shape)}")
 
 
 def _ptr(t: Optional[torch.Tensor]) -> int:
@@ -76,7 +84,14 @@ def _ptr(t: Optional[torch.Tensor]) -> int:
 
 
 def _stream() -> int:
+    # torch's current stream as a raw handle; the accessor that skips building a Stream object is used
+    # where this torch has it (it is called once per launch)
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _call(mod: KernelModule, fname: str, argtypes, *args) -> None:
@@ -463,9 +478,15 @@ def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
 def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                     tile_req: torch.Tensor, tile_q0: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                     kv_len: torch.Tensor, block_table: torch.Tensor, window: Optional[int], scale: float,
-                    qt: int = 1) -> None:
+                    qt: int = 1, chunk: int = 0, max_splits: int = 1, rows: Optional[torch.Tensor] = None,
+                    row_req: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
     """Attention of tiles of ``attention_tile_rows(d, qt)`` consecutive rows of one request each (tile t:
-    request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d]."""
+    request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d].
+
+    With ``max_splits`` > 1 every tile's keys are cut into splits of ``chunk`` keys (a multiple of 64;
+    ``max_splits`` * chunk must reach past the largest position) that run as workgroups of their own, and
+    the rows named by ``rows`` (int32: every row of every tiled request) are merged at the end; this
+    needs the step's ``row_req`` and ``positions`` [T]."""
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt)
     _check(out, "out", (T, nH * d), torch.bfloat16)
     n_tiles = tile_req.shape[0]
@@ -475,10 +496,24 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (kv_len, "kv_len")):
         _check(t, nm, (R,), torch.int32)
     _check(block_table, "block_table", (R, None), torch.int32)
-    _call(mod, "ifx_attn_tiles", (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, P),
+    part_o = part_ml = None
+    n_rows = 0
+    if max_splits > 1:
+        if chunk <= 0 or chunk % 64:
+            raise KernelError(f"attention_tiles: splits need a chunk that is a multiple of 64, got {chunk}")
+        if rows is None or row_req is None or positions is None:
+            raise KernelError("attention_tiles: splits need the rows to merge, row_req and positions")
+        n_rows = rows.shape[0]
+        _check(rows, "rows", (n_rows,), torch.int32)
+        _check(row_req, "row_req", (T,), torch.int32)
+        _check(positions, "positions", (T,), torch.int32)
+        part_o = torch.empty((T, nH, max_splits, d), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nH, max_splits, 2), dtype=torch.float32, device=q.device)
+    _call(mod, "ifx_attn_tiles", (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
           n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
-          block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), _stream())
+          block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), int(chunk), int(max_splits),
+          _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _stream())
 
 
 # ----------------------------------------------------------------------------------------

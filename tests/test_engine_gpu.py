@@ -357,3 +357,26 @@ def test_other_page_sizes(page_size, dtype, sharp_folders):
             runner.free_request(rid)
         runner.manager.check()
     assert runner.manager.free_pages() == [p.num_pages for p in runner.manager.pools]
+
+
+def test_prompt_portions_with_a_long_past_split_their_keys(sharp_folders, monkeypatch):
+    """Portions of a prompt late in a long context: few tiles, many keys, which the tile kernel cuts into splits.
+    The thresholds are lowered so that the tiny models' 250 and 380 tokens qualify."""
+    from inferflux_amd.kernels import attention
+    monkeypatch.setattr(attention, "TILE_SPLIT_MIN_KEYS", 64)
+    calls = []
+    real = attention.ops.attention_tiles
+    monkeypatch.setattr(attention.ops, "attention_tiles", lambda *a, **k: (calls.append(a[14] if len(a) > 14 else 1), real(*a, **k))[1])
+    for name, portions in (("A", (100, 90, 17, 43)), ("C", (150, 100, 17, 113))):
+        folder = sharp_folders[name, "bfloat16"]
+        runner = load_runner(folder, torch.bfloat16, num_pages=40)
+        ids = seeded_ids(77, sum(portions), TINY[name]["vocab_size"])
+        want = plain_logits(folder, ids)
+        runner.add_request("p")
+        pos = 0
+        for n in portions:
+            got = runner.step([StepEntry("p", ids[pos:pos + n], list(range(n)))]).cpu()
+            assert rel_err(got, want[pos:pos + n]) < REL_TOL["bfloat16"], (name, pos)
+            pos += n
+        runner.free_request("p")
+    assert max(calls) > 1      # some portion did run in splits

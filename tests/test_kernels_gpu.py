@@ -360,8 +360,10 @@ def test_attention_rows_subset_leaves_other_rows_alone():
 
 
 @pytest.mark.parametrize("qt", [1, 2])
+@pytest.mark.parametrize("split_chunk", [0, 64, 192])
 @pytest.mark.parametrize("case", MFMA_CASES)
-def test_attention_tiles(case, qt):
+def test_attention_tiles(case, qt, split_chunk):
+    """``split_chunk``: the keys cut into splits of that many, run as workgroups of their own and merged."""
     lens_q, lens_past, nH, nKV, d, P, window, sharp = case
     (q, kc, vc, row_req, positions, table), want, info = paged_case(7, lens_q, lens_past, nH, nKV, d, P, BF16, window, sharp=sharp)
     T = q.shape[0]
@@ -370,11 +372,25 @@ def test_attention_tiles(case, qt):
     q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
     tiles = [(r, q0) for r, n in enumerate(info["q_lens"]) for q0 in range(0, n, ops.attention_tile_rows(d, qt))]
     dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    splits = {}
+    if split_chunk:
+        splits = dict(chunk=split_chunk, max_splits=-(-max(info["kv_lens"]) // split_chunk),
+                      rows=torch.arange(T, dtype=torch.int32, device=DEV), row_req=row_req, positions=positions)
     ops.attention_tiles(q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV),
-                        q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt)
+                        q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt, **splits)
     out = out.cpu().double()
     assert torch.isfinite(out).all()
     assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
+
+
+def test_attention_tiles_refuses_splits_it_cannot_merge():
+    (q, kc, vc, row_req, positions, table), _, info = paged_case(7, [64], [100], 4, 2, 16, 16, BF16, None)
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    args = (q, kc, vc, torch.zeros(64, 64, dtype=BF16, device=DEV), dev([0]), dev([0]), dev([0]), dev([64]), dev([164]), table, None, 0.25, 1)
+    with pytest.raises(ops.KernelError, match="multiple of 64"):
+        ops.attention_tiles(*args, chunk=100, max_splits=2, rows=dev(list(range(64))), row_req=row_req, positions=positions)
+    with pytest.raises(ops.KernelError, match="rows to merge"):
+        ops.attention_tiles(*args, chunk=128, max_splits=2)
 
 
 def test_mfma_attention_refuses_what_it_cannot_do():
