@@ -3,8 +3,9 @@
 Every choice computes the same function (causal, optionally windowed, grouped-query attention
 over the paged cache); they differ in speed and in which sizes they accept.  In bfloat16 with a
 head size the matrix-core module takes, requests that bring at least TILE_MIN rows go to the
-tile kernel (tiles of as many rows as the compiled module says) and all other rows (decode tokens, short portions) to the row kernel; everything
-else (float32, other head sizes) goes to the plain kernel.
+tile kernel (tiles of as many rows as the compiled module says; keys in splits when the tiles are
+few and their pasts long) and all other rows (decode tokens, short portions) to the row kernel;
+everything else (float32, other head sizes) goes to the plain kernel.
 """
 from __future__ import annotations
 
