@@ -378,39 +378,89 @@ __device__ __forceinline__ int pick_page(const TilePages& pg, int sub) {
   return sub == 0 ? pg.p0 : sub == 1 ? pg.p1 : sub == 2 ? pg.p2 : pg.p3;
 }
 
+// Pieces are numbered run by run (a run = 16 keys = one page or part of one): piece c of a tile belongs
+// to run c / (2 D); a run's K pieces are (key in run, 8 dims), its V^T pieces (dim, half of the run).
+// With 2 D a multiple of 256 (head sizes 128 and 256) a thread's i-th piece lies in a run known at
+// compile time, so the run's page and base address stay in scalar registers and a piece costs two or
+// three vector instructions of address arithmetic; smaller heads select per lane.
+constexpr int RUN_PIECES = 2 * D;
+constexpr bool STATIC_RUN = RUN_PIECES % 256 == 0;
+
+struct PieceAt { int run, within; bool live; };
+__device__ __forceinline__ PieceAt piece_at(int i, int tid) {
+  const int c = tid + 256 * i;
+  if (STATIC_RUN) return PieceAt{(256 * i) / RUN_PIECES, tid + (256 * i) % RUN_PIECES, true};
+  return PieceAt{c / RUN_PIECES, c % RUN_PIECES, c < N_PIECES};
+}
+
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+// A buffer descriptor over ``bytes`` at ``p``: loads through it return zeros beyond its end, so a run
+// without a page gets a descriptor of no bytes instead of a branch around its loads.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t run_buffer(const bf16_t* p, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, bytes, 0x00020000);   // raw 32-bit data format of gfx9
+}
+__device__ __forceinline__ bf16x8 buffer_load8(__amdgpu_buffer_rsrc_t rs, int byte_offset) {
+  const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, byte_offset, 0, 0);
+  return *(const bf16x8*)&v;
+}
+
 __device__ __forceinline__ void fetch_tile(TileRegs& r, const TileArgs& a, const TilePages& pg, int kvh, int j0, int tid) {
   const int P = a.P;
+  if (STATIC_RUN) {
+    // Every piece's run is known here: one descriptor per run for K (the run's 16 rows are contiguous) and
+    // one for V^T (D rows of P, of which the run takes 16 keys), built from scalars; a piece is one load
+    // at an offset that depends on the thread alone.
+#pragma unroll
+    for (int i = 0; i < K_PIECES; ++i) {
+      const PieceAt at = piece_at(i, tid);
+      const int page = pick_page(pg, at.run), pos0 = (j0 + 16 * at.run) & (P - 1);
+      const bf16_t* base = a.k_cache + (((size_t)max(page, 0) * a.nKV + kvh) * P + pos0) * D;
+      r.k[i] = buffer_load8(run_buffer(base, page >= 0 ? 16 * D * 2 : 0), at.within * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < V_PIECES; ++i) {
+      const PieceAt at = piece_at(i, tid);
+      const int page = pick_page(pg, at.run), pos0 = (j0 + 16 * at.run) & (P - 1);
+      const bf16_t* base = a.v_cache + ((size_t)max(page, 0) * a.nKV + kvh) * D * P + pos0;
+      r.v[i] = buffer_load8(run_buffer(base, page >= 0 ? ((D - 1) * P + 16) * 2 : 0), ((at.within / 2) * P + 8 * (at.within % 2)) * 2);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < K_PIECES; ++i) {
-    const int c = tid + 256 * i;
-    const int key = c / (D / 8), c8 = c % (D / 8);
-    const int page = c < N_PIECES ? pick_page(pg, key >> 4) : -1;
-    r.k[i] = page >= 0 ? *(const bf16x8*)(a.k_cache + (((size_t)page * a.nKV + kvh) * P + ((j0 + key) & (P - 1))) * D + 8 * c8) : zero8();
+    const PieceAt at = piece_at(i, tid);
+    const int key = at.within / (D / 8), c8 = at.within % (D / 8);
+    const int page = at.live ? pick_page(pg, at.run) : -1;
+    const bf16_t* base = a.k_cache + ((size_t)max(page, 0) * a.nKV + kvh) * P * D;
+    r.k[i] = page >= 0 ? *(const bf16x8*)(base + ((j0 + 16 * at.run + key) & (P - 1)) * D + 8 * c8) : zero8();
   }
 #pragma unroll
   for (int i = 0; i < V_PIECES; ++i) {
-    const int c = tid + 256 * i;
-    const int dim = c / (TK / 8), k8 = c % (TK / 8);  // 8 keys never straddle a page
-    const int page = c < N_PIECES ? pick_page(pg, k8 >> 1) : -1;
-    r.v[i] = page >= 0 ? *(const bf16x8*)(a.v_cache + (((size_t)page * a.nKV + kvh) * D + dim) * P + ((j0 + 8 * k8) & (P - 1))) : zero8();
+    const PieceAt at = piece_at(i, tid);
+    const int dim = at.within / 2, half = at.within % 2;   // 8 keys never straddle a page
+    const int page = at.live ? pick_page(pg, at.run) : -1;
+    const bf16_t* base = a.v_cache + ((size_t)max(page, 0) * a.nKV + kvh) * D * P;
+    r.v[i] = page >= 0 ? *(const bf16x8*)(base + dim * P + ((j0 + 16 * at.run + 8 * half) & (P - 1))) : zero8();
   }
 }
 
 __device__ __forceinline__ void stage_tile(const TileRegs& r, bf16_t* k_s, bf16_t* v_s, int tid) {
 #pragma unroll
   for (int i = 0; i < K_PIECES; ++i) {
-    const int c = tid + 256 * i;
-    if (c < N_PIECES) *(bf16x8*)(k_s + (c / (D / 8)) * KPAD + 8 * (c % (D / 8))) = r.k[i];
+    const PieceAt at = piece_at(i, tid);
+    if (at.live) *(bf16x8*)(k_s + (16 * at.run + at.within / (D / 8)) * KPAD + 8 * (at.within % (D / 8))) = r.k[i];
   }
 #pragma unroll
   for (int i = 0; i < V_PIECES; ++i) {
-    const int c = tid + 256 * i;
-    if (c < N_PIECES) {
+    const PieceAt at = piece_at(i, tid);
+    if (at.live) {
       // Keys are stored in the order the second product consumes them: within each run of 32 keys,
       // position 8 g + 4 h + r holds key 16 h + 4 g + r, so that one 16-byte read gives a lane its
-      // four keys of both 16-key score tiles.  A piece of 8 consecutive keys lands as two halves.
-      const int dim = c / (TK / 8), k8 = c % (TK / 8);
-      bf16_t* dst = v_s + dim * VPAD + 32 * (k8 / 4) + 16 * (k8 % 2) + 4 * ((k8 % 4) / 2);
+      // four keys of both 16-key score tiles.  A piece of 8 consecutive keys (half a run of 16: keys
+      // 16 run + 8 half ...) lands as two halves.
+      const int dim = at.within / 2, half = at.within % 2;
+      bf16_t* dst = v_s + dim * VPAD + 32 * (at.run / 2) + 16 * half + 4 * (at.run % 2);
       bf16x4 lo, hi;
 #pragma unroll
       for (int e = 0; e < 4; ++e) { lo[e] = r.v[i][e]; hi[e] = r.v[i][e + 4]; }
