@@ -380,7 +380,7 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   RopeArgs a{qkv, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
   hipStream_t s = (hipStream_t)stream;
   // (a few tokens are quicker with one small block per token and head: nothing waits on a loop over tokens)
-  if (T >= 64 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
+  if (T >= 128 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
       (!slots || page_size % 8 == 0)) {
     const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
     const size_t v_threads = slots ? (size_t)((T + 7) / 8) * nKV * d : 0;

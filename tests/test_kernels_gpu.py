@@ -118,12 +118,12 @@ def test_rope_append_in_pieces(d, nH, nKV, bias):
     an aligned run of 16 (written as pieces of the transposed page), a run that starts at an odd offset, scattered
     ones, one token without a slot."""
     g = gen(31)
-    T, P, pages, theta = 69, 16, 12, 1e4
+    T, P, pages, theta = 133, 16, 16, 1e4
     width = (nH + 2 * nKV) * d
     qkv = torch.randn(T, width, generator=g).to(BF16)
     b = (0.5 * torch.randn(width, generator=g)).to(BF16) if bias else None
-    positions = torch.cat([torch.arange(100, 116), torch.arange(3, 11), torch.randint(0, 2000, (45,), generator=g)]).to(torch.int32)
-    scattered = (48 + torch.randperm(pages * P - 48, generator=g)[:45]).tolist()
+    positions = torch.cat([torch.arange(100, 116), torch.arange(3, 11), torch.randint(0, 2000, (109,), generator=g)]).to(torch.int32)
+    scattered = (48 + torch.randperm(pages * P - 48, generator=g)[:109]).tolist()
     slots = torch.tensor(list(range(32, 48)) + list(range(3, 11)) + scattered, dtype=torch.int32)
     slots[30] = -1
     kc = torch.zeros(pages, nKV, P, d, dtype=BF16, device=DEV)
