@@ -10,9 +10,11 @@
 //          all of them (any group size; more than 16 heads take several passes).  Partial
 //          results (max, sum, unnormalised output) go to scratch and a second kernel merges
 //          the splits.  For decode tokens and short portions.
-//   tiles  one workgroup of 4 waves per (64 consecutive rows of one request, query head): key
-//          and value tiles of 64 positions are staged in LDS and shared by the 4 waves.  For
-//          long portions of prompts.
+//   tiles  one workgroup of 4 waves per (64 or 128 consecutive rows of one request, query head;
+//          -DTILE_QT=1 or 2 tiles of 16 rows per wave): key and value tiles of 64 positions are
+//          staged in LDS and shared by the 4 waves.  For long portions of prompts.  The keys can
+//          be cut into splits that run as workgroups of their own and are merged like the row
+//          kernel's (portions late in a long context: few tiles, many keys).
 //
 // Both work on transposed tiles so that no register shuffle is needed between the two matrix
 // products: S^T[key, q] = K Q^T leaves each lane holding four consecutive keys of one query
