@@ -249,28 +249,36 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
 #pragma unroll
   for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = 0.f;
   float L = 0.f;
-  // The launcher bounds the splits of a row by 64 per round; rounds handle longer rows.
-  float M = -INFINITY;
+  // Lane s of a round holds split sb + s; rows with more than 64 splits take further rounds.  The first
+  // round's maxima and sums are kept from the pass that finds the maximum (the usual case is one round).
+  float M = -INFINITY, m_first = -INFINITY, l_first = 0.f;
   for (int sb = s0; sb <= s1; sb += WAVE) {
     const int s = sb + lane;
-    M = fmaxf(M, s <= s1 ? pml[2 * s] : -INFINITY);
+    const float2 ml = s <= s1 ? *(const float2*)(pml + 2 * s) : float2{-INFINITY, 0.f};
+    if (sb == s0) { m_first = ml.x; l_first = ml.y; }
+    M = fmaxf(M, ml.x);
   }
   M = wave_max(M);
   for (int sb = s0; sb <= s1; sb += WAVE) {
     const int s = sb + lane;
-    const float ms = s <= s1 ? pml[2 * s] : -INFINITY;
+    float ms = m_first, ls = l_first;
+    if (sb != s0) {
+      const float2 ml = s <= s1 ? *(const float2*)(pml + 2 * s) : float2{-INFINITY, 0.f};
+      ms = ml.x; ls = ml.y;
+    }
     const float w = ms == -INFINITY ? 0.f : exp2f(ms - M);
-    L += s <= s1 ? w * pml[2 * s + 1] : 0.f;
+    L += w * ls;
     __syncthreads();
     w_s[lane] = w;
     __syncthreads();
     const int n = min(WAVE, s1 - sb + 1);
-    // four splits at a time, so that their loads are in flight together; an empty split (weight 0) is
-    // never read, its scratch may hold anything
-    for (int i = 0; i < n; i += 4) {
-      float wi[4], val[4][(D + WAVE - 1) / WAVE];
+    // sixteen splits at a time, so that their loads are in flight together (a step of a loop that waits
+    // for its own loads costs a trip to the L2 each); an empty split (weight 0) is never read, its
+    // scratch may hold anything
+    for (int i = 0; i < n; i += 16) {
+      float wi[16], val[16][(D + WAVE - 1) / WAVE];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < 16; ++u) {
         wi[u] = i + u < n ? w_s[i + u] : 0.f;
 #pragma unroll
         for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
@@ -279,7 +287,7 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
         }
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 16; ++u)
 #pragma unroll
         for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = fmaf(wi[u], val[u][c], acc[c]);
     }
