@@ -33,16 +33,14 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-// EPI 0: out[m, n] = acc.  EPI 1: the rows of W alternate gate, up, gate, up ...; a lane holds two
-// such pairs of one output row and writes silu(gate) * up to out[m, n / 2] (out is [M, N / 2]).
-template <int MT, int NT, int U, typename TO, int EPI, bool TILED>
-__global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out,
-                                   int M, int N, int K, int k_tiles) {
-  extern __shared__ float red[];  // [(waves - 1)][NT * MT][64 lanes][4]
+// The sums of one workgroup: acc[nt][mt] = W tile (first_tile + nt) times x rows 16 mt ..., K split over
+// the workgroup's waves and added through LDS in wave order.  Returns true in the wave that holds the
+// sums (wave 0); the others are done.
+template <int MT, int NT, int U, bool TILED>
+__device__ __forceinline__ bool skinny_accumulate(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, int M, int N,
+                                                  int K, int k_tiles, int first_tile, floatx4 (&acc)[NT][MT], float* red) {
   const int wid = threadIdx.x / WAVE, nw = blockDim.x / WAVE, lane = threadIdx.x % WAVE;
   const int col = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.x * 16 * NT;
-  floatx4 acc[NT][MT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -51,8 +49,8 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
   const bf16_t* wrow[NT];  // rows (tiles) past N are read again, never stored
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
-    wrow[nt] = TILED ? W + ((size_t)min(n_base / 16 + nt, (N - 1) / 16) * k_tiles * WAVE + lane) * 8
-                     : W + (size_t)min(n_base + 16 * nt + col, N - 1) * K;
+    wrow[nt] = TILED ? W + ((size_t)min(first_tile + nt, (N - 1) / 16) * k_tiles * WAVE + lane) * 8
+                     : W + (size_t)min(16 * (first_tile + nt) + col, N - 1) * K;
   const bf16_t* xrow[MT];
   bool xok[MT];
 #pragma unroll
@@ -103,7 +101,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
           *(floatx4*)(red + ((size_t)((wid - 1) * NT * MT + nt * MT + mt) * WAVE + lane) * 4) = acc[nt][mt];
     }
     __syncthreads();
-    if (wid > 0) return;
+    if (wid > 0) return false;
     for (int w = 1; w < nw; ++w)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
@@ -114,9 +112,25 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
           for (int r = 0; r < 4; ++r) acc[nt][mt][r] += o[r];
         }
   }
-  // acc[nt][mt][r] = out[m = 16 mt + col][n = n_base + 16 nt + 4 g + r]
+  return true;
+}
+
+// EPI 0: out[m, n] = acc.  EPI 1: the rows of W alternate gate, up, gate, up ...; a lane holds two
+// such pairs of one output row and writes silu(gate) * up to out[m, n / 2] (out is [M, N / 2]).
+// ``order`` (tiled copies only): tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
+template <int MT, int NT, int U, typename TO, int EPI, bool TILED>
+__global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out,
+                                   int M, int N, int K, int k_tiles, const int* __restrict__ order) {
+  extern __shared__ float red[];  // [(waves - 1)][NT * MT][64 lanes][4]
+  const int lane = threadIdx.x % WAVE, col = lane & 15, g = lane >> 4;
+  const int first_tile = blockIdx.x * NT, n_tiles = (N + 15) / 16;
+  floatx4 acc[NT][MT];
+  if (!skinny_accumulate<MT, NT, U, TILED>(x, W, M, N, K, k_tiles, first_tile, acc, red)) return;
+  // acc[nt][mt][r] = out[m = 16 mt + col][n = 16 (row tile of the weight) + 4 g + r]
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
+  for (int nt = 0; nt < NT; ++nt) {
+    if (first_tile + nt >= n_tiles) continue;
+    const int n0 = 16 * ((TILED && order) ? order[first_tile + nt] : first_tile + nt);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = 16 * mt + col;
@@ -124,29 +138,106 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
       if (EPI == 0) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int n = n_base + 16 * nt + 4 * g + r;
+          const int n = n0 + 4 * g + r;
           if (n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r]);
         }
       } else {
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
-          const int n = n_base + 16 * nt + 4 * g + r;  // even: gate at n, up at n + 1
+          const int n = n0 + 4 * g + r;  // even: gate at n, up at n + 1
           const float gt = acc[nt][mt][r], up = acc[nt][mt][r + 1];
           if (n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
         }
       }
     }
+  }
+}
+
+// The q/k/v projection of up to 16 tokens with what follows it as the epilogue: bias, rotation of q and
+// k by the token's position (split-half pairs over the whole head), q to q_out, k and v into the paged
+// cache at the token's slot.  The tiled copy is ordered so that consecutive tiles hold the two halves of
+// 16 rotation pairs: tile 2 w is rows h d + 16 j ... of head h, tile 2 w + 1 rows h d + d/2 + 16 j ...,
+// with w = h (d / 32) + j; a lane then holds both elements of its four pairs.  Heads are numbered over
+// the concatenated weight: q heads, then k heads, then v heads.
+struct QkvArgs {
+  const void* bias;       // [(nH + 2 nKV) d] or null
+  int bias_dtype;
+  const int* slots;       // [M] page * page_size + offset, < 0: nothing is written; null: queries only
+  const float* cs;        // [M, d / 2]
+  const float* sn;
+  bf16_t* q_out;          // [M, nH * d]
+  bf16_t* k_cache;        // [pages, nKV, P, d]
+  bf16_t* v_cache;        // [pages, nKV, d, P]
+  int nH, nKV, d, P;
+};
+
+template <int U>
+__global__ void qkv_rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, int M, int N, int K, int k_tiles,
+                                QkvArgs a) {
+  extern __shared__ float red[];
+  const int lane = threadIdx.x % WAVE, col = lane & 15, g = lane >> 4;
+  floatx4 acc[2][1];
+  if (!skinny_accumulate<1, 2, U, true>(x, W, M, N, K, k_tiles, 2 * blockIdx.x, acc, red)) return;
+  const int m = col;
+  if (m >= M) return;
+  const int d = a.d, half = d / 2, per_head = d / 32;
+  const int head = blockIdx.x / per_head, i0 = 16 * (blockIdx.x % per_head) + 4 * g;   // the lane's pairs: i0 + r and i0 + r + half
+  float x0[4], x1[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    x0[r] = acc[0][0][r];
+    x1[r] = acc[1][0][r];
+    if (a.bias) {
+      x0[r] += load_dyn(a.bias, a.bias_dtype, (size_t)head * d + i0 + r);
+      x1[r] += load_dyn(a.bias, a.bias_dtype, (size_t)head * d + half + i0 + r);
+    }
+  }
+  const bool is_v = head >= a.nH + a.nKV;
+  if (!is_v) {
+    const floatx4 cs = *(const floatx4*)(a.cs + (size_t)m * half + i0), sn = *(const floatx4*)(a.sn + (size_t)m * half + i0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float y0 = x0[r] * cs[r] - x1[r] * sn[r], y1 = x0[r] * sn[r] + x1[r] * cs[r];
+      x0[r] = y0;
+      x1[r] = y1;
+    }
+  }
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+  bf16x4 lo, hi;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) { lo[r] = (__bf16)x0[r]; hi[r] = (__bf16)x1[r]; }
+  if (head < a.nH) {
+    bf16_t* dst = a.q_out + ((size_t)m * a.nH + head) * d + i0;
+    *(bf16x4*)dst = lo;
+    *(bf16x4*)(dst + half) = hi;
+    return;
+  }
+  const int slot = a.slots ? a.slots[m] : -1;
+  if (slot < 0) return;
+  const int page = slot / a.P, off = slot % a.P;
+  if (!is_v) {
+    bf16_t* dst = a.k_cache + (((size_t)page * a.nKV + (head - a.nH)) * a.P + off) * d + i0;
+    *(bf16x4*)dst = lo;
+    *(bf16x4*)(dst + half) = hi;
+  } else {
+    bf16_t* dst = a.v_cache + (((size_t)page * a.nKV + (head - a.nH - a.nKV)) * d + i0) * a.P + off;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      dst[(size_t)r * a.P] = lo[r];
+      dst[(size_t)(half + r) * a.P] = hi[r];
+    }
+  }
 }
 
 template <int MT, int NT, int U, bool TILED>
 static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int k_tiles, int waves, int epi,
-                  hipStream_t s) {
+                  const int* order, hipStream_t s) {
   const int groups = (N + 16 * NT - 1) / (16 * NT);
   const size_t lds = (size_t)(waves - 1) * NT * MT * WAVE * 4 * sizeof(float);
   IFX_REQUIRE(lds <= 64 * 1024, "skinny_gemm: %d waves of %dx%d tiles need %zu bytes of LDS", waves, NT, MT, lds);
 #define GO(TO_, EPI_)                                                                                              \
   hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, TO_, EPI_, TILED>), dim3(groups), dim3(waves * WAVE), lds, s,  \
-                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles)
+                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles, order)
   if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
   else if (out_dtype == DT_BF16) GO(bf16_t, 1);
   else if (epi == 0) GO(float, 0);
@@ -159,30 +250,65 @@ static int launch(const void* x, const void* W, void* out, int out_dtype, int M,
 extern "C" int ifx_tiled_rows(int N) { return (N + 15) / 16 * 16; }
 extern "C" int ifx_tiled_cols(int K) { return (K + 63) / 64 * 64; }
 
-__global__ void tile_weights_kernel(const bf16_t* __restrict__ W, bf16_t* __restrict__ Wt, int N, int K, int k_tiles, size_t pieces) {
+__global__ void tile_weights_kernel(const bf16_t* __restrict__ W, bf16_t* __restrict__ Wt, int N, int K, int k_tiles, size_t pieces,
+                                    const int* __restrict__ order) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // piece number: ((t * k_tiles + kt) * 64 + 16 g + col)
   if (i >= pieces) return;
   const int lane = (int)(i % WAVE), col = lane & 15, g = lane >> 4;
   const size_t tile = i / WAVE;
-  const int kt = (int)(tile % k_tiles), n = (int)(tile / k_tiles) * 16 + col, k = 32 * kt + 8 * g;
+  const int t = (int)(tile / k_tiles), kt = (int)(tile % k_tiles);
+  const int n = (order ? order[t] : t) * 16 + col, k = 32 * kt + 8 * g;
   *(bf16x8*)(Wt + i * 8) = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero8();
 }
 
-// Wt [ifx_tiled_rows(N) * ifx_tiled_cols(K)] = the tiled form of W [N, K] (K a multiple of 8).
-extern "C" int ifx_tile_weights(const void* W, void* Wt, int N, int K, void* stream) {
+// Wt [ifx_tiled_rows(N) * ifx_tiled_cols(K)] = the tiled form of W [N, K] (K a multiple of 8).  ``order``
+// [ifx_tiled_rows(N) / 16] (or null): row tile t of the copy is row tile order[t] of W (a permutation,
+// checked by the caller).
+extern "C" int ifx_tile_weights(const void* W, void* Wt, int N, int K, const int* order, void* stream) {
   IFX_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "tile_weights: N=%d K=%d (K must be a multiple of 8)", N, K);
   const int k_tiles = ifx_tiled_cols(K) / 32;
   const size_t pieces = (size_t)(ifx_tiled_rows(N) / 16) * k_tiles * WAVE;
   hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)W, (bf16_t*)Wt, N, K, k_tiles, pieces);
+                     (const bf16_t*)W, (bf16_t*)Wt, N, K, k_tiles, pieces, order);
+  IFX_LAUNCH_CHECK();
+}
+
+// The q/k/v projection of M <= 16 tokens from the pair-ordered tiled copy Wt of the concatenated weight
+// [(nH + 2 nKV) d, K], with bias, rotation and the cache write as its epilogue (see qkv_rope_kernel).
+// With slots null only the nH query heads are projected (the copy then holds those rows only).
+extern "C" int ifx_qkv_rope(const void* x, const void* Wt, int M, int K, const void* bias, int bias_dtype, const int* slots,
+                            const float* cs, const float* sn, int nH, int nKV, int d, int page_size, void* q_out,
+                            void* k_cache, void* v_cache, int waves, int unroll, void* stream) {
+  IFX_REQUIRE(M >= 0 && M <= 16 && K > 0 && K % 8 == 0, "qkv_rope: M=%d must be at most 16, K=%d a multiple of 8", M, K);
+  IFX_REQUIRE(nH > 0 && nKV >= 0 && d > 0 && d % 32 == 0, "qkv_rope: head size %d must be a multiple of 32 (nH=%d nKV=%d)", d, nH, nKV);
+  IFX_REQUIRE(cs && sn && q_out, "qkv_rope: needs the rotation table and an output");
+  IFX_REQUIRE(!slots || (page_size > 0 && k_cache && v_cache), "qkv_rope: cache write without cache");
+  IFX_REQUIRE(bias_dtype == DT_BF16 || bias_dtype == DT_F32 || !bias, "qkv_rope: unknown bias dtype %d", bias_dtype);
+  if (M == 0) return 0;
+  const int heads = nH + (slots ? 2 * nKV : 0), N = heads * d, groups = N / 32;
+  const int nkb = (K + 63) / 64, k_tiles = ifx_tiled_cols(K) / 32;
+  if (unroll == 0) unroll = 2;
+  if (waves == 0) {
+    waves = 1;
+    while (waves < 16 && groups * waves < 1024) waves *= 2;
+    while (waves > 1 && nkb < waves * 2) waves /= 2;
+  }
+  IFX_REQUIRE(waves >= 1 && waves <= 16 && (unroll == 2 || unroll == 4), "qkv_rope: waves=%d unroll=%d", waves, unroll);
+  const size_t lds = (size_t)(waves - 1) * 2 * WAVE * 4 * sizeof(float);
+  QkvArgs a{bias, bias_dtype, slots, cs, sn, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nH, slots ? nKV : 0, d, page_size};
+  hipStream_t s = (hipStream_t)stream;
+  if (unroll == 2) hipLaunchKernelGGL(qkv_rope_kernel<2>, dim3(groups), dim3(waves * WAVE), lds, s, (const bf16_t*)x, (const bf16_t*)Wt, M, N, K, k_tiles, a);
+  else hipLaunchKernelGGL(qkv_rope_kernel<4>, dim3(groups), dim3(waves * WAVE), lds, s, (const bf16_t*)x, (const bf16_t*)Wt, M, N, K, k_tiles, a);
   IFX_LAUNCH_CHECK();
 }
 
 // nt, waves, unroll = 0: chosen here from the shape.
 // epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2].
-// tiled 1: W is the tiled form written by ifx_tile_weights.
+// tiled 1: W is the tiled form written by ifx_tile_weights, with the row-tile order it was given (or null).
 extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int nt,
-                               int waves, int unroll, int epi, int tiled, void* stream) {
+                               int waves, int unroll, int epi, int tiled, const int* order, void* stream) {
+  IFX_REQUIRE(tiled || !order, "skinny_gemm: a tile order goes with a tiled copy");
+  IFX_REQUIRE(epi == 0 || !order, "skinny_gemm: gate/up pairs with a tile order are not supported");
   IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "skinny_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "skinny_gemm: K=%d must be a multiple of 8", K);
@@ -223,8 +349,8 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   const int k_tiles = ifx_tiled_cols(K) / 32;
 #define CASE(MT_, NT_, U_)                                                                                  \
   if (mt == MT_ && nt == NT_ && unroll == U_)                                                               \
-    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, s)        \
-                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, s)
+    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, s)  \
+                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, s)
   // (the combinations left out need more than the 128 registers a workgroup of 16 waves leaves a lane)
   CASE(1, 1, 4); CASE(1, 2, 4); CASE(1, 1, 2); CASE(1, 2, 2);
   CASE(2, 1, 4); CASE(2, 2, 2); CASE(2, 1, 2);

@@ -246,17 +246,24 @@ def pause_library_gemm_tuning(paused: bool) -> None:
         tunable.tuning_enable(not paused)
 
 
-def tile_weights(weight: torch.Tensor) -> torch.Tensor:
+def tile_weights(weight: torch.Tensor, order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The tiled form of a bfloat16 ``weight`` [N, K] that the weight-streaming product reads in
-    contiguous kilobytes: a flat tensor of rows16(N) * cols64(K) elements (zeros in the padding)."""
+    contiguous kilobytes: a flat tensor of rows16(N) * cols64(K) elements (zeros in the padding).
+    ``order`` (int32, a permutation of the ceil(N / 16) row tiles): tile t of the copy is row tile
+    order[t] of the weight."""
     _check(weight, "weight", (None, None), torch.bfloat16)
     N, K = weight.shape
     if K % 8:
         raise KernelError(f"tile_weights: K={K} must be a multiple of 8")
     mod = load_module("gemm_bf16")
-    size = mod.fn("ifx_tiled_rows", (I,))(N) * mod.fn("ifx_tiled_cols", (I,))(K)
+    rows16 = mod.fn("ifx_tiled_rows", (I,))(N)
+    if order is not None:
+        _check(order, "order", (rows16 // 16,), torch.int32)
+        if sorted(order.tolist()) != list(range(rows16 // 16)):
+            raise KernelError("tile_weights: order is not a permutation of the weight's row tiles")
+    size = rows16 * mod.fn("ifx_tiled_cols", (I,))(K)
     out = torch.empty((size,), dtype=torch.bfloat16, device=weight.device)
-    _call(mod, "ifx_tile_weights", (P, P, I, I, P), weight.data_ptr(), out.data_ptr(), N, K, _stream())
+    _call(mod, "ifx_tile_weights", (P, P, I, I, P, P), weight.data_ptr(), out.data_ptr(), N, K, _ptr(order), _stream())
     return out
 
 
@@ -266,10 +273,10 @@ class LinearWeight:
     copy doubles the weight's memory; it is left out when ``decode_weight_copy`` is off or when the
     card has no room for it, and products with few rows then read ``rows``."""
 
-    __slots__ = ("rows", "tiled")
+    __slots__ = ("rows", "tiled", "order")
 
-    def __init__(self, rows: torch.Tensor, tiled: Optional[torch.Tensor] = None):
-        self.rows, self.tiled = rows, tiled
+    def __init__(self, rows: torch.Tensor, tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None):
+        self.rows, self.tiled, self.order = rows, tiled, order   # order: the copy's row-tile order (see tile_weights)
 
     @property
     def shape(self):
@@ -285,27 +292,67 @@ decode_weight_copy = True
 DECODE_COPY_RESERVE_BYTES = 8 << 30
 
 
-def prepare_linear(weight: torch.Tensor) -> LinearWeight:
-    """Wrap a projection's weight for ``linear`` / ``linear_swiglu``, with the tiled copy if wanted and possible."""
+def prepare_linear(weight: torch.Tensor, order: Optional[torch.Tensor] = None) -> LinearWeight:
+    """Wrap a projection's weight for ``linear`` / ``linear_swiglu``, with the tiled copy if wanted and possible
+    (its row tiles in ``order``, if given)."""
     tiled = None
     if (decode_weight_copy and weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2
             and weight.shape[1] % 8 == 0):
         free, _ = torch.cuda.mem_get_info(weight.device)
         if free >= weight.numel() * 2 + DECODE_COPY_RESERVE_BYTES:
-            tiled = tile_weights(weight.contiguous())
+            tiled = tile_weights(weight.contiguous(), order)
         else:
             log.warn("kernels", f"no room for the decode copy of a {tuple(weight.shape)} weight "
                                 f"({free / 2**30:.1f} GiB free): decoding reads the plain rows")
-    return LinearWeight(weight, tiled)
+    return LinearWeight(weight, tiled, order if tiled is not None else None)
+
+
+def pair_tile_order(n_heads: int, head_dim: int) -> list:
+    """Row-tile order of a projection whose rows are ``n_heads`` heads of ``head_dim`` (a multiple of 32) that
+    puts the two halves of 16 split-half rotation pairs into consecutive tiles: for head h and j < d / 32,
+    tiles h d/16 + j and h d/16 + j + d/32.  What ``qkv_rope_append`` expects of its tiled copy."""
+    per, half = head_dim // 16, head_dim // 32
+    return [h * per + j + s * half for h in range(n_heads) for j in range(half) for s in (0, 1)]
+
+
+def qkv_rope_append(x: torch.Tensor, weight: LinearWeight, bias: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                    cos: torch.Tensor, sin: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int,
+                    waves: int = 0, unroll: int = 0) -> torch.Tensor:
+    """For up to 16 tokens: q, k, v = x W^T + bias from the pair-ordered tiled copy of the concatenated
+    weight, q and k rotated (split-half pairs over the whole head, table cos/sin [M, d/2]), k and v written
+    into the paged cache at ``slots``, q returned [M, nH, d] -- one kernel, the rotation and the cache
+    write being the product's epilogue.  With ``slots`` None the weight holds the query rows only."""
+    _check(x, "x", (None, None), torch.bfloat16)
+    M, K = x.shape
+    heads = n_heads + (2 * n_kv_heads if slots is not None else 0)
+    if weight.tiled is None or weight.order is None or tuple(weight.rows.shape) != (heads * head_dim, K):
+        raise KernelError(f"qkv_rope_append: needs the pair-ordered tiled copy of a [{heads * head_dim}, {K}] weight")
+    if M > 16 or head_dim % 32 or K % 8:
+        raise KernelError(f"qkv_rope_append: M={M} must be <= 16, head_dim={head_dim} a multiple of 32, K={K} of 8")
+    _check(cos, "cos", (M, head_dim // 2), torch.float32)
+    _check(sin, "sin", (M, head_dim // 2), torch.float32)
+    if bias is not None:
+        _check(bias, "bias", (heads * head_dim,))
+    if slots is not None:
+        _check(slots, "slots", (M,), torch.int32)
+        _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), torch.bfloat16)
+        _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, head_dim, page_size), torch.bfloat16)
+    q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=x.device)
+    _call(load_module("gemm_bf16"), "ifx_qkv_rope", (P, P, I, I, P, I, P, P, P, I, I, I, I, P, P, P, I, I, P),
+          x.data_ptr(), weight.tiled.data_ptr(), M, K, _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
+          cos.data_ptr(), sin.data_ptr(), n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache),
+          _ptr(v_cache), waves, unroll, _stream())
+    return q
 
 
 def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                 nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False,
-                tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
+                tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
     accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose.
     With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2].
-    With ``tiled`` (``tile_weights(weight)``) the kernel streams that copy instead of the rows."""
+    With ``tiled`` (``tile_weights(weight, order)``) the kernel streams that copy instead of the rows."""
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     _check(weight, "weight", (None, K), torch.bfloat16)
@@ -318,9 +365,11 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     if swiglu_pairs and N % 2:
         raise KernelError("skinny_gemm: gate/up pairs need an even number of weight rows")
     out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
-    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, I, I, P),
+    if order is not None and (tiled is None or swiglu_pairs):
+        raise KernelError("skinny_gemm: a tile order goes with a tiled copy and a plain product")
+    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, I, I, P, P),
           x.data_ptr(), (weight if tiled is None else tiled).data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves,
-          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else 1, _stream())
+          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else 1, _ptr(order), _stream())
     return out
 
 
@@ -356,9 +405,9 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> 
     projection (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).  float32 output (logits)
     always comes from float accumulators, never through a bfloat16 rounding.
     """
-    tiled = None
+    tiled = order = None
     if isinstance(weight, LinearWeight):
-        weight, tiled = weight.rows, weight.tiled
+        weight, tiled, order = weight.rows, weight.tiled, weight.order
     if weight.dtype == torch.float32:
         return gemm_f32(x, weight, None, out_dtype or x.dtype)
     if weight.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
@@ -369,7 +418,7 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> 
     M, K = x.shape
     kind = _small_m_kernel(M, weight.shape[0], K, tiled is not None)
     if kind == "skinny":
-        return skinny_gemm(x, weight, out_dtype, tiled=tiled)
+        return skinny_gemm(x, weight, out_dtype, tiled=tiled, order=order)
     if kind == "staged":
         return staged_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:
@@ -397,6 +446,8 @@ def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
     applies it."""
     M, K = x.shape
     rows, tiled = (weight_pairs.rows, weight_pairs.tiled) if isinstance(weight_pairs, LinearWeight) else (weight_pairs, None)
+    if isinstance(weight_pairs, LinearWeight) and weight_pairs.order is not None:
+        raise KernelError("linear_swiglu: a tile order is not supported for gate/up pairs")
     if rows.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
         kind = _small_m_kernel(M, rows.shape[0], K, tiled is not None)
         if kind == "skinny":

@@ -61,10 +61,20 @@ class PagedAttention(Mixer):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         n = self.name
-        self.w_qkv = ops.prepare_linear(concat_weights([tensors[f"{n}.{p}_proj.weight"] for p in "qkv"]))
+        self.w_qkv = self._prepare_qkv(concat_weights([tensors[f"{n}.{p}_proj.weight"] for p in "qkv"]),
+                                       self.n_heads + 2 * self.n_kv_heads)
         self.b_qkv = concat_weights([tensors[f"{n}.{p}_proj.bias"] for p in "qkv"]) if self.bias else None
         self.w_o = ops.prepare_linear(tensors[f"{n}.o_proj.weight"])
         self._w_q = None
+
+    def _prepare_qkv(self, weight: torch.Tensor, heads: int):
+        """The projection's weight with its decode copy; for head sizes that are multiples of 32 the copy's
+        row tiles are ordered so that the fused projection + rotation kernel finds both halves of a rotation
+        pair in one lane (plain products read the same copy through the order)."""
+        order = None
+        if self.head_dim % 32 == 0 and weight.is_cuda and weight.dtype == torch.bfloat16:
+            order = torch.tensor(ops.pair_tile_order(heads, self.head_dim), dtype=torch.int32, device=weight.device)
+        return ops.prepare_linear(weight, order)
 
     def forward(self, h: torch.Tensor, ctx, binding: MixerBinding) -> torch.Tensor:
         cache = binding.cache
@@ -75,12 +85,18 @@ class PagedAttention(Mixer):
         w, b = self.w_qkv, self.b_qkv
         if not binding.writes_cache:  # only the queries: the first nH*d rows of the fused matrix
             if self._w_q is None:
-                self._w_q = ops.prepare_linear(w.rows[:width])
+                self._w_q = self._prepare_qkv(w.rows[:width], self.n_heads)
             w, b = self._w_q, (b[:width] if b is not None else None)
+        slots = ctx.write_slots(cache.group) if binding.writes_cache else None
+        if (style == ops.ROPE_SPLIT_HALF and rotary_dim == d and w.order is not None and h.dtype == torch.bfloat16
+                and h.shape[0] <= 16 and not self.position.needs_apply):
+            # few tokens: the rotation and the cache write are the projection's epilogue
+            q = ops.qkv_rope_append(h, w, b, slots, cos, sin, nH, nKV, d, cache.k if slots is not None else None,
+                                    cache.v if slots is not None else None, cache.page_size)
+            return ops.linear(paged_attention(q, cache, ctx, self.window, self.scale), self.w_o)
         qkv = ops.linear(h, w)
         if self.position.needs_apply:
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
-        slots = ctx.write_slots(cache.group) if binding.writes_cache else None
         q = ops.rope_append(qkv, b, slots, cos, sin, style, rotary_dim, nH, nKV, d,
                             cache.k if slots is not None else None, cache.v if slots is not None else None,
                             cache.page_size)

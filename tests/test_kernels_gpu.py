@@ -458,6 +458,69 @@ def test_skinny_gemm_from_the_tiled_copy_equals_from_rows(M, N, K):
         assert torch.allclose(a, want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
 
 
+def test_tiled_copy_in_another_row_tile_order():
+    """A permuted copy gives the same product (the kernel writes tile t to the rows order[t] names) and lays
+    its tiles out as the order says."""
+    g = gen(20)
+    N, K = 150, 136                                    # 10 row tiles, the last with 6 rows
+    w = torch.randn(N, K, generator=g).to(BF16).to(DEV)
+    order = torch.tensor([3, 9, 0, 7, 1, 8, 2, 6, 5, 4], dtype=torch.int32, device=DEV)
+    tiled = ops.tile_weights(w, order)
+    plain = ops.tile_weights(w).view(10, -1)
+    assert torch.equal(tiled.view(10, -1), plain[order.long()])
+    for M in (1, 9, 16, 40):
+        x = torch.randn(M, K, generator=g).to(BF16).to(DEV)
+        want = x.double().cpu() @ w.double().cpu().t()
+        got = ops.skinny_gemm(x, w, F32, tiled=tiled, order=order).cpu().double()
+        assert torch.allclose(got, want, rtol=1e-4, atol=2e-3)
+        assert torch.allclose(ops.linear(x, ops.LinearWeight(w, tiled, order), out_dtype=F32).cpu().double(), want, rtol=1e-4, atol=2e-3)
+    with pytest.raises(ops.KernelError, match="permutation"):
+        ops.tile_weights(w, torch.zeros(10, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("d,nH,nKV,K", [(32, 3, 1, 72), (128, 7, 1, 264), (64, 4, 2, 128)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, nKV, K, bias):
+    """The fused kernel against the product followed by the rotary + append kernel (itself checked against the
+    plain formulas above): same q, same cache, nothing else touched; and queries only."""
+    g = gen(21)
+    P_, pages, theta = 16, 5, 1e4
+    heads = nH + 2 * nKV
+    w = (torch.randn(heads * d, K, generator=g) / math.sqrt(K)).to(BF16).to(DEV)
+    b = (0.5 * torch.randn(heads * d, generator=g)).to(BF16).to(DEV) if bias else None
+    x = torch.randn(M, K, generator=g).to(BF16).to(DEV)
+    positions = torch.randint(0, 3000, (M,), generator=g).to(torch.int32).to(DEV)
+    slots = torch.randperm(pages * P_, generator=g)[:M].to(torch.int32)
+    if M > 2:
+        slots[1] = -1
+    slots = slots.to(DEV)
+    inv_freq = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64), 2.0 * torch.arange(d // 2, dtype=torch.float64) / d)).float()
+    cs, sn = ops.rope_table(positions, inv_freq.to(DEV))
+    lw = ops.prepare_linear(w, torch.tensor(ops.pair_tile_order(heads, d), dtype=torch.int32, device=DEV))
+
+    def caches():
+        return (torch.zeros(pages, nKV, P_, d, dtype=BF16, device=DEV), torch.zeros(pages, nKV, d, P_, dtype=BF16, device=DEV))
+    kc, vc = caches()
+    q = ops.qkv_rope_append(x, lw, b, slots, cs, sn, nH, nKV, d, kc, vc, P_)
+    # the unfused path rounds the product to bf16 before the bias: compare with that path in float, at bf16's rounding
+    qkv32 = ops.skinny_gemm(x, w, F32)
+    kc2f, vc2f = (c.float() for c in caches())
+    q2 = ops.rope_append(qkv32, b.float() if bias else None, slots, cs, sn, ops.ROPE_SPLIT_HALF, d, nH, nKV, d, kc2f, vc2f, P_)
+    t = dict(rtol=1e-2, atol=1e-2)
+    assert torch.allclose(q.float().view(M, -1), q2.view(M, -1), **t)
+    assert torch.allclose(kc.float(), kc2f, **t) and torch.allclose(vc.float(), vc2f, **t)
+    assert torch.equal(kc == 0, kc2f == 0) and torch.equal(vc == 0, vc2f == 0)      # the same elements written
+    for waves, unroll in [(1, 2), (4, 4), (16, 2)]:
+        ka, va = caches()
+        qa = ops.qkv_rope_append(x, lw, b, slots, cs, sn, nH, nKV, d, ka, va, P_, waves=waves, unroll=unroll)
+        assert torch.allclose(qa.float(), q.float(), rtol=1e-2, atol=1e-2) and torch.allclose(ka.float(), kc.float(), rtol=1e-2, atol=1e-2)
+    # queries only: the first nH heads of the weight, no cache
+    lq = ops.prepare_linear(w[: nH * d], torch.tensor(ops.pair_tile_order(nH, d), dtype=torch.int32, device=DEV))
+    qq = ops.qkv_rope_append(x, lq, b[: nH * d] if bias else None, None, cs, sn, nH, 0, d, None, None, P_)
+    assert torch.allclose(qq.float(), q.float(), rtol=1e-2, atol=1e-2)
+
+
 def test_linear_weight_uses_the_copy_for_few_rows_and_the_rows_beyond():
     g = gen(17)
     w = torch.randn(200, 136, generator=g).to(BF16).to(DEV)
