@@ -328,6 +328,8 @@ MFMA_CASES = [c for c in ATTN_CASES if c[4] % 16 == 0 and c[4] <= 128] + [
     ([33], [90], 40, 2, 32, 16, None, 64),                         # 20 query heads per kv head: two passes of 16
     ([2, 70], [9000, 8200], 4, 2, 64, 16, None, 4500),             # long contexts: many splits, planted key mid-way
     ([1, 1], [5000, 300], 2, 1, 128, 64, 1000, None),              # a window inside a long context, pages of 64
+    ([40, 3], [30, 170], 6, 3, 96, 16, None, 20),                  # head sizes between the prebuilt ones
+    ([90], [75], 5, 1, 80, 32, 50, None),
 ]
 
 
