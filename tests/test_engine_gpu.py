@@ -205,6 +205,45 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     assert not torch.allclose(whole[1:], whole[:-1])
 
 
+def test_a_layer_that_reads_another_entries_cache_in_bfloat16():
+    """The schedule runs one attention layer twice, the second time on the first one's cache (queries only).  In
+    bfloat16 with a head size of 32, steps of up to 16 tokens take the fused projection + rotation kernel and longer
+    ones the separate kernels: both must give the same logits within bfloat16's rounding."""
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.parts import LayerSpec, ModelPlan, PartSpec, ScheduleEntry
+
+    H, V = 64, 90
+    p = "twice.layers.0"
+    attn = PartSpec("paged_attention", {"name": f"{p}.attn", "n_heads": 4, "n_kv_heads": 2, "head_dim": 32, "bias": True,
+                                        "position": PartSpec("rotary", {"head_dim": 32, "theta": 1000.0})})
+    layer = LayerSpec(p, PartSpec("prenorm"), PartSpec("rmsnorm", {"name": f"{p}.n1", "eps": 1e-5}), attn,
+                      PartSpec("rmsnorm", {"name": f"{p}.n2", "eps": 1e-5}),
+                      PartSpec("swiglu", {"name": f"{p}.mlp", "intermediate_size": 80}))
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=128,
+                     embedding=PartSpec("token_embedding", {"name": "twice.embed", "vocab_size": V}),
+                     layers=(layer,), schedule=(ScheduleEntry(0), ScheduleEntry(0, cache_from=0)),
+                     final_norm=PartSpec("rmsnorm", {"name": "twice.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "twice.head", "vocab_size": V}))
+    logits = {}
+    for dtype in (torch.float32, torch.bfloat16):
+        model = Model(plan=plan).init_random(5, dtype, "cuda")
+        runner = ModelRunner(model, num_pages=16, max_requests=2)
+        ids = seeded_ids(21, 56, V)
+        runner.add_request("w")
+        whole = runner.step([StepEntry("w", ids, list(range(56)))]).cpu()
+        runner.free_request("w")
+        runner.add_request("c")
+        rows, at = [], 0
+        for m in (1, 2, 16, 5, 16, 16):
+            rows.append(runner.step([StepEntry("c", ids[at:at + m], list(range(m)))]).cpu()); at += m
+        logits[dtype] = (whole, torch.cat(rows))
+    w32, c32 = logits[torch.float32]
+    wb, cb = logits[torch.bfloat16]
+    assert torch.equal(w32, c32)
+    assert rel_err(cb, w32) < REL_TOL["bfloat16"] and rel_err(wb, w32) < REL_TOL["bfloat16"]
+
+
 # ---- captured decode steps ----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C"])
