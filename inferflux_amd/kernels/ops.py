@@ -519,11 +519,10 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
-    """Rows per tile of the tile kernel compiled for ``head_dim`` with ``qt`` query tiles per wave."""
-    mod = load_module("attn_mfma", (("HEAD_DIM", head_dim), ("TILE_QT", qt)))
-    f = mod.lib.ifx_attn_tile_rows
-    f.restype = ctypes.c_int
-    return int(f())
+    """Rows per tile of the tile kernel with ``qt`` query tiles per wave: four waves of ``qt`` tiles of 16 rows
+    (the compiled module says the same, ``ifx_attn_tile_rows``; asking it would compile a variant that a
+    short step never runs)."""
+    return 64 * qt
 
 
 def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -539,6 +538,8 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     the rows named by ``rows`` (int32: every row of every tiled request) are merged at the end; this
     needs the step's ``row_req`` and ``positions`` [T]."""
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt)
+    if mod.fn("ifx_attn_tile_rows", ())() != attention_tile_rows(d, qt):
+        raise KernelError("attention_tiles: the compiled module's tile rows differ from attention_tile_rows()")
     _check(out, "out", (T, nH * d), torch.bfloat16)
     n_tiles = tile_req.shape[0]
     _check(tile_req, "tile_req", (n_tiles,), torch.int32)
