@@ -33,6 +33,66 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// A normalisation whose factor per row is applied to the product's results instead of to its input:
+// row m of x stands for x[m] * rsqrt(sum_j pieces[j][m] / width + eps).  ``pieces`` is [n][16]
+// (16 rows whatever M is), written by the EPI 2 epilogue below: piece j is the sum of squares of 16
+// consecutive elements of the row before it was weighted.
+struct RowScale {
+  const float* pieces;  // null: no factor
+  int n;
+  float width, eps;
+};
+
+// EPI 2: the product is added to the float stream [M, N] in place, and what the norm that follows needs is
+// written beside it: rows[m, n] = bf16(stream[m, n] * norm_w[n]) and pieces[n / 16][m] (see RowScale).
+struct StreamOut {
+  float* stream;
+  const bf16_t* norm_w;
+  bf16_t* rows;
+  float* pieces;
+};
+
+// Sum over the four lanes col, col + 16, col + 32, col + 48, the same in all four.
+__device__ __forceinline__ float sum_over_groups(float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+// The factor of row lane % 16, computed by one wave.  The pieces are read as float4s (rows 4 (c % 4) ... + 3 of
+// piece c / 4 in float4 number c), lane l taking numbers l, l + 64, ...: sixteen loads are in flight at a time
+// (one after the other they would cost a trip to the L2 each), a lane always meets the same four rows, and the
+// sums are added in a fixed order.
+__device__ __forceinline__ float row_factor(const RowScale& s, int lane) {
+  const int chunks = 4 * s.n;
+  floatx4 t{0.f, 0.f, 0.f, 0.f};
+  for (int base = lane; base < chunks; base += WAVE * 16) {
+    floatx4 v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int c = base + WAVE * u;
+      v[u] = c < chunks ? *(const floatx4*)(s.pieces + (size_t)4 * c) : floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) t[r] += v[u][r];
+  }
+#pragma unroll
+  for (int off = 4; off < WAVE; off <<= 1)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) t[r] += __shfl_xor(t[r], off);
+  // every lane with lane % 4 == q now holds the sums of rows 4 q ... 4 q + 3
+  const int col = lane & 15;
+  float sum = 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float from = __shfl(t[r], col >> 2);
+    if ((col & 3) == r) sum = from;
+  }
+  return rsqrtf(sum / s.width + s.eps);
+}
+
 // The sums of one workgroup: acc[nt][mt] = W tile (first_tile + nt) times x rows 16 mt ..., K split over
 // the workgroup's waves and added through LDS in wave order.  Returns true in the wave that holds the
 // sums (wave 0); the others are done.
@@ -117,16 +177,60 @@ __device__ __forceinline__ bool skinny_accumulate(const bf16_t* __restrict__ x, 
 
 // EPI 0: out[m, n] = acc.  EPI 1: the rows of W alternate gate, up, gate, up ...; a lane holds two
 // such pairs of one output row and writes silu(gate) * up to out[m, n / 2] (out is [M, N / 2]).
+// EPI 2 (up to 16 rows, N a multiple of 4): see StreamOut; ``out`` is not used.
 // ``order`` (tiled copies only): tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
+// ``scale`` (up to 16 rows): the results of row m are multiplied by the row's factor first.
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+
 template <int MT, int NT, int U, typename TO, int EPI, bool TILED>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out,
-                                   int M, int N, int K, int k_tiles, const int* __restrict__ order) {
+                                   int M, int N, int K, int k_tiles, const int* __restrict__ order, RowScale scale,
+                                   StreamOut so) {
   extern __shared__ float red[];  // [(waves - 1)][NT * MT][64 lanes][4]
   const int lane = threadIdx.x % WAVE, col = lane & 15, g = lane >> 4;
   const int first_tile = blockIdx.x * NT, n_tiles = (N + 15) / 16;
+  const bool first_wave = threadIdx.x < WAVE;
+  float rs = 1.f;
+  if (MT == 1 && scale.pieces && first_wave) rs = row_factor(scale, lane);
+  // EPI 2: what the epilogue reads is asked for before the stream of weights, not after it
+  floatx4 was[NT];
+  bf16x4 nw[NT];
+  if (EPI == 2 && first_wave) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int n = 16 * (first_tile + nt) + 4 * g;
+      const bool ok = n < N && col < M;
+      was[nt] = ok ? *(const floatx4*)(so.stream + (size_t)col * N + n) : floatx4{0.f, 0.f, 0.f, 0.f};
+      if (ok) nw[nt] = *(const bf16x4*)(so.norm_w + n);
+    }
+  }
   floatx4 acc[NT][MT];
   if (!skinny_accumulate<MT, NT, U, TILED>(x, W, M, N, K, k_tiles, first_tile, acc, red)) return;
   // acc[nt][mt][r] = out[m = 16 mt + col][n = 16 (row tile of the weight) + 4 g + r]
+  if (EPI == 2) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (first_tile + nt >= n_tiles) continue;   // the same for the whole wave
+      const int n = 16 * (first_tile + nt) + 4 * g;
+      const bool ok = n < N && col < M;
+      float sq = 0.f;
+      if (ok) {
+        floatx4 v;
+        bf16x4 y;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          v[r] = was[nt][r] + acc[nt][0][r] * rs;
+          y[r] = (__bf16)(v[r] * (float)nw[nt][r]);
+          sq += v[r] * v[r];
+        }
+        *(floatx4*)(so.stream + (size_t)col * N + n) = v;
+        *(bf16x4*)(so.rows + (size_t)col * N + n) = y;
+      }
+      sq = sum_over_groups(sq);
+      if (g == 0) so.pieces[(size_t)(first_tile + nt) * 16 + col] = sq;
+    }
+    return;
+  }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     if (first_tile + nt >= n_tiles) continue;
@@ -139,13 +243,13 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int n = n0 + 4 * g + r;
-          if (n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r]);
+          if (n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r] * rs);
         }
       } else {
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
           const int n = n0 + 4 * g + r;  // even: gate at n, up at n + 1
-          const float gt = acc[nt][mt][r], up = acc[nt][mt][r + 1];
+          const float gt = acc[nt][mt][r] * rs, up = acc[nt][mt][r + 1] * rs;
           if (n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
         }
       }
@@ -173,9 +277,11 @@ struct QkvArgs {
 
 template <int U>
 __global__ void qkv_rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, int M, int N, int K, int k_tiles,
-                                QkvArgs a) {
+                                QkvArgs a, RowScale scale) {
   extern __shared__ float red[];
   const int lane = threadIdx.x % WAVE, col = lane & 15, g = lane >> 4;
+  float rs = 1.f;
+  if (scale.pieces && threadIdx.x < WAVE) rs = row_factor(scale, lane);
   floatx4 acc[2][1];
   if (!skinny_accumulate<1, 2, U, true>(x, W, M, N, K, k_tiles, 2 * blockIdx.x, acc, red)) return;
   const int m = col;
@@ -185,8 +291,8 @@ __global__ void qkv_rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __re
   float x0[4], x1[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    x0[r] = acc[0][0][r];
-    x1[r] = acc[1][0][r];
+    x0[r] = acc[0][0][r] * rs;
+    x1[r] = acc[1][0][r] * rs;
     if (a.bias) {
       x0[r] += load_dyn(a.bias, a.bias_dtype, (size_t)head * d + i0 + r);
       x1[r] += load_dyn(a.bias, a.bias_dtype, (size_t)head * d + half + i0 + r);
@@ -202,7 +308,6 @@ __global__ void qkv_rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __re
       x1[r] = y1;
     }
   }
-  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
   bf16x4 lo, hi;
 #pragma unroll
   for (int r = 0; r < 4; ++r) { lo[r] = (__bf16)x0[r]; hi[r] = (__bf16)x1[r]; }
@@ -231,14 +336,17 @@ __global__ void qkv_rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __re
 
 template <int MT, int NT, int U, bool TILED>
 static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int k_tiles, int waves, int epi,
-                  const int* order, hipStream_t s) {
+                  const int* order, const RowScale& scale, const StreamOut& so, hipStream_t s) {
   const int groups = (N + 16 * NT - 1) / (16 * NT);
   const size_t lds = (size_t)(waves - 1) * NT * MT * WAVE * 4 * sizeof(float);
   IFX_REQUIRE(lds <= 64 * 1024, "skinny_gemm: %d waves of %dx%d tiles need %zu bytes of LDS", waves, NT, MT, lds);
 #define GO(TO_, EPI_)                                                                                              \
   hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, TO_, EPI_, TILED>), dim3(groups), dim3(waves * WAVE), lds, s,  \
-                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles, order)
-  if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
+                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles, order, scale, so)
+  if (epi == 2) {
+    if constexpr (MT == 1) GO(float, 2);
+    else IFX_FAIL("skinny_gemm: the stream epilogue takes at most 16 rows");
+  } else if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
   else if (out_dtype == DT_BF16) GO(bf16_t, 1);
   else if (epi == 0) GO(float, 0);
   else GO(float, 1);
@@ -276,9 +384,13 @@ extern "C" int ifx_tile_weights(const void* W, void* Wt, int N, int K, const int
 // The q/k/v projection of M <= 16 tokens from the pair-ordered tiled copy Wt of the concatenated weight
 // [(nH + 2 nKV) d, K], with bias, rotation and the cache write as its epilogue (see qkv_rope_kernel).
 // With slots null only the nH query heads are projected (the copy then holds those rows only).
+// scale_pieces [n_scale_pieces][16] (or null), scale_width, scale_eps: a factor per row of x, see RowScale.
 extern "C" int ifx_qkv_rope(const void* x, const void* Wt, int M, int K, const void* bias, int bias_dtype, const int* slots,
                             const float* cs, const float* sn, int nH, int nKV, int d, int page_size, void* q_out,
-                            void* k_cache, void* v_cache, int waves, int unroll, void* stream) {
+                            void* k_cache, void* v_cache, int waves, int unroll, const float* scale_pieces,
+                            int n_scale_pieces, float scale_width, float scale_eps, void* stream) {
+  IFX_REQUIRE(!scale_pieces || (n_scale_pieces > 0 && scale_width > 0.f), "qkv_rope: bad row factors (%d pieces, width %g)",
+              n_scale_pieces, (double)scale_width);
   IFX_REQUIRE(M >= 0 && M <= 16 && K > 0 && K % 8 == 0, "qkv_rope: M=%d must be at most 16, K=%d a multiple of 8", M, K);
   IFX_REQUIRE(nH > 0 && nKV >= 0 && d > 0 && d % 32 == 0, "qkv_rope: head size %d must be a multiple of 32 (nH=%d nKV=%d)", d, nH, nKV);
   IFX_REQUIRE(cs && sn && q_out, "qkv_rope: needs the rotation table and an output");
@@ -296,20 +408,31 @@ extern "C" int ifx_qkv_rope(const void* x, const void* Wt, int M, int K, const v
   IFX_REQUIRE(waves >= 1 && waves <= 16 && (unroll == 2 || unroll == 4), "qkv_rope: waves=%d unroll=%d", waves, unroll);
   const size_t lds = (size_t)(waves - 1) * 2 * WAVE * 4 * sizeof(float);
   QkvArgs a{bias, bias_dtype, slots, cs, sn, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nH, slots ? nKV : 0, d, page_size};
+  const RowScale scale{scale_pieces, n_scale_pieces, scale_width, scale_eps};
   hipStream_t s = (hipStream_t)stream;
-  if (unroll == 2) hipLaunchKernelGGL(qkv_rope_kernel<2>, dim3(groups), dim3(waves * WAVE), lds, s, (const bf16_t*)x, (const bf16_t*)Wt, M, N, K, k_tiles, a);
-  else hipLaunchKernelGGL(qkv_rope_kernel<4>, dim3(groups), dim3(waves * WAVE), lds, s, (const bf16_t*)x, (const bf16_t*)Wt, M, N, K, k_tiles, a);
+  if (unroll == 2) hipLaunchKernelGGL(qkv_rope_kernel<2>, dim3(groups), dim3(waves * WAVE), lds, s, (const bf16_t*)x, (const bf16_t*)Wt, M, N, K, k_tiles, a, scale);
+  else hipLaunchKernelGGL(qkv_rope_kernel<4>, dim3(groups), dim3(waves * WAVE), lds, s, (const bf16_t*)x, (const bf16_t*)Wt, M, N, K, k_tiles, a, scale);
   IFX_LAUNCH_CHECK();
 }
 
 // nt, waves, unroll = 0: chosen here from the shape.
 // epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2].
+// epi 2: the product is added to ``stream`` [M, N] (float, in place), rows_out [M, N] = bf16(stream * norm_w) and
+//        pieces_out [ceil(N / 16)][16] = sums of squares of the stream in runs of 16, for the norm that follows
+//        (M <= 16, N a multiple of 4, norm_w bfloat16 [N]); ``out`` is not used.
 // tiled 1: W is the tiled form written by ifx_tile_weights, with the row-tile order it was given (or null).
+// scale_pieces [n_scale_pieces][16] (or null), scale_width, scale_eps: a factor per row of x (M <= 16), see RowScale.
 extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int nt,
-                               int waves, int unroll, int epi, int tiled, const int* order, void* stream) {
+                               int waves, int unroll, int epi, int tiled, const int* order, const float* scale_pieces,
+                               int n_scale_pieces, float scale_width, float scale_eps, float* stream_io,
+                               const void* norm_w, void* rows_out, float* pieces_out, void* stream) {
   IFX_REQUIRE(tiled || !order, "skinny_gemm: a tile order goes with a tiled copy");
-  IFX_REQUIRE(epi == 0 || !order, "skinny_gemm: gate/up pairs with a tile order are not supported");
-  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
+  IFX_REQUIRE(epi == 0 || !order, "skinny_gemm: only the plain epilogue takes a tile order");
+  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0) || (epi == 2 && N % 4 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
+  IFX_REQUIRE(epi != 2 || (M <= 16 && stream_io && norm_w && rows_out && pieces_out),
+              "skinny_gemm: the stream epilogue takes at most 16 rows (M=%d) and needs the stream, the norm's weight and two outputs", M);
+  IFX_REQUIRE(!scale_pieces || (M <= 16 && n_scale_pieces > 0 && scale_width > 0.f),
+              "skinny_gemm: row factors take at most 16 rows (M=%d, %d pieces, width %g)", M, n_scale_pieces, (double)scale_width);
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "skinny_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "skinny_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "skinny_gemm: unknown out dtype %d", out_dtype);
@@ -345,12 +468,15 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   }
   while (waves > 1 && (size_t)(waves - 1) * nt * mt * WAVE * 16 > 64 * 1024) waves /= 2;
   IFX_REQUIRE(waves >= 1 && waves <= 16, "skinny_gemm: waves=%d outside 1..16", waves);
+  if (epi == 2 && nt == 2 && unroll == 4) unroll = 2;   // that instantiation spills
   hipStream_t s = (hipStream_t)stream;
   const int k_tiles = ifx_tiled_cols(K) / 32;
-#define CASE(MT_, NT_, U_)                                                                                  \
-  if (mt == MT_ && nt == NT_ && unroll == U_)                                                               \
-    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, s)  \
-                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, s)
+  const RowScale scale{scale_pieces, n_scale_pieces, scale_width, scale_eps};
+  const StreamOut so{stream_io, (const bf16_t*)norm_w, (bf16_t*)rows_out, pieces_out};
+#define CASE(MT_, NT_, U_)                                                                                             \
+  if (mt == MT_ && nt == NT_ && unroll == U_)                                                                          \
+    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, s)  \
+                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, s)
   // (the combinations left out need more than the 128 registers a workgroup of 16 waves leaves a lane)
   CASE(1, 1, 4); CASE(1, 2, 4); CASE(1, 1, 2); CASE(1, 2, 2);
   CASE(2, 1, 4); CASE(2, 2, 2); CASE(2, 1, 2);

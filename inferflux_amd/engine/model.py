@@ -98,8 +98,15 @@ class Model:
         if t is not None:
             t.mark("embed")
         pending = None
-        for i, e in enumerate(self.plan.schedule):
-            residual, pending = self.blocks[e.layer].forward(residual, pending, ctx, storage.binding(i))
+        schedule = self.plan.schedule
+        for i, e in enumerate(schedule):
+            block = self.blocks[e.layer]
+            # a block that can hand on rows prepared for the next block's first norm is told that norm
+            following = self.blocks[schedule[i + 1].layer].entry_norm() if i + 1 < len(schedule) else None
+            if following is not None and block.entry_norm() is not None:
+                residual, pending = block.forward(residual, pending, ctx, storage.binding(i), following=following)
+            else:
+                residual, pending = block.forward(residual, pending, ctx, storage.binding(i))
         if ctx.n_logit_rows == 0:
             logits = torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=residual.device)
         else:

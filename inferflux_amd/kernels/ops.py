@@ -307,6 +307,79 @@ def prepare_linear(weight: torch.Tensor, order: Optional[torch.Tensor] = None) -
     return LinearWeight(weight, tiled, order if tiled is not None else None)
 
 
+class ScaledRows:
+    """Rows of a normalised activation up to one factor per row: row t stands for
+    ``rows[t] * rsqrt(sum(pieces[:, t]) / width + eps)``.  ``rows`` is bfloat16 [T <= 16, width] (the stream times
+    the norm's weight), ``pieces`` float32 [ceil(width / 16), 16] (sums of squares of the stream in runs of 16; rows
+    past T hold zeros).  A weight-streaming product that takes these multiplies its sums by the factor, which
+    saves the norm a kernel of its own; ``linear_into_stream`` makes them."""
+
+    __slots__ = ("rows", "pieces", "width", "eps")
+
+    def __init__(self, rows: torch.Tensor, pieces: torch.Tensor, width: int, eps: float):
+        self.rows, self.pieces, self.width, self.eps = rows, pieces, int(width), float(eps)
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+
+def _scale_args(x):
+    """(rows, the four row-factor arguments of the kernels) of a tensor or a ``ScaledRows``."""
+    if isinstance(x, ScaledRows):
+        _check(x.pieces, "pieces", (-(-x.width // 16), 16), torch.float32)
+        _check(x.rows, "rows", (None, x.width), torch.bfloat16)
+        if x.rows.shape[0] > 16:
+            raise KernelError(f"scaled rows: {x.rows.shape[0]} rows, at most 16")
+        return x.rows, (x.pieces.data_ptr(), x.pieces.shape[0], float(x.width), x.eps)
+    return x, (0, 0, 0.0, 0.0)
+
+
+def takes_scaled_rows(n_rows: int, weight) -> bool:
+    """Whether ``linear`` / ``linear_swiglu`` / ``qkv_rope_append`` take ``ScaledRows`` of ``n_rows`` rows with this weight."""
+    if not isinstance(weight, LinearWeight):
+        return False
+    N, K = weight.rows.shape
+    return (weight.rows.dtype == torch.bfloat16 and n_rows <= 16
+            and _small_m_kernel(n_rows, N, K, weight.tiled is not None) == "skinny")
+
+
+def adds_into_stream(n_rows: int, weight, norm_weight: torch.Tensor) -> bool:
+    """Whether ``linear_into_stream`` takes this shape."""
+    if not isinstance(weight, LinearWeight) or weight.order is not None:
+        return False
+    N, K = weight.rows.shape
+    return (weight.rows.dtype == torch.bfloat16 and norm_weight.dtype == torch.bfloat16 and n_rows <= 16 and N % 4 == 0
+            and _small_m_kernel(n_rows, N, K, weight.tiled is not None) == "skinny")
+
+
+def linear_into_stream(x: torch.Tensor, weight: LinearWeight, stream: torch.Tensor, norm_weight: torch.Tensor,
+                       eps: float) -> ScaledRows:
+    """``stream`` [M <= 16, N] (float32) += x [M, K] W^T in place, as the product's epilogue, which also prepares
+    the RMS norm that follows (weight ``norm_weight`` [N] bfloat16): returns its rows up to the factor per row."""
+    _check(x, "x", (None, None), torch.bfloat16)
+    M, K = x.shape
+    N = weight.rows.shape[0]
+    if not adds_into_stream(M, weight, norm_weight) or weight.rows.shape[1] != K:
+        raise KernelError(f"linear_into_stream: not for {M} rows times a {tuple(weight.rows.shape)} weight")
+    _check(stream, "stream", (M, N), torch.float32)
+    _check(norm_weight, "norm_weight", (N,), torch.bfloat16)
+    rows = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    pieces = torch.empty((-(-N // 16), 16), dtype=torch.float32, device=x.device)
+    w = weight.rows if weight.tiled is None else weight.tiled
+    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
+          x.data_ptr(), w.data_ptr(), 0, DT_F32, M, N, K, 0, 0, 0, 2, 0 if weight.tiled is None else 1, 0,
+          0, 0, 0.0, 0.0, stream.data_ptr(), norm_weight.data_ptr(), rows.data_ptr(), pieces.data_ptr(), _stream())
+    return ScaledRows(rows, pieces, N, eps)
+
+
+_SKINNY_ARGS = (P, P, P, I, I, I, I, I, I, I, I, I, P, P, I, F, F, P, P, P, P, P)
+
+
 def pair_tile_order(n_heads: int, head_dim: int) -> list:
     """Row-tile order of a projection whose rows are ``n_heads`` heads of ``head_dim`` (a multiple of 32) that
     puts the two halves of 16 split-half rotation pairs into consecutive tiles: for head h and j < d / 32,
@@ -322,7 +395,9 @@ def qkv_rope_append(x: torch.Tensor, weight: LinearWeight, bias: Optional[torch.
     """For up to 16 tokens: q, k, v = x W^T + bias from the pair-ordered tiled copy of the concatenated
     weight, q and k rotated (split-half pairs over the whole head, table cos/sin [M, d/2]), k and v written
     into the paged cache at ``slots``, q returned [M, nH, d] -- one kernel, the rotation and the cache
-    write being the product's epilogue.  With ``slots`` None the weight holds the query rows only."""
+    write being the product's epilogue.  With ``slots`` None the weight holds the query rows only.
+    ``x`` may be ``ScaledRows``."""
+    x, scale = _scale_args(x)
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     heads = n_heads + (2 * n_kv_heads if slots is not None else 0)
@@ -339,10 +414,10 @@ def qkv_rope_append(x: torch.Tensor, weight: LinearWeight, bias: Optional[torch.
         _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), torch.bfloat16)
         _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, head_dim, page_size), torch.bfloat16)
     q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=x.device)
-    _call(load_module("gemm_bf16"), "ifx_qkv_rope", (P, P, I, I, P, I, P, P, P, I, I, I, I, P, P, P, I, I, P),
+    _call(load_module("gemm_bf16"), "ifx_qkv_rope", (P, P, I, I, P, I, P, P, P, I, I, I, I, P, P, P, I, I, P, I, F, F, P),
           x.data_ptr(), weight.tiled.data_ptr(), M, K, _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
           cos.data_ptr(), sin.data_ptr(), n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache),
-          _ptr(v_cache), waves, unroll, _stream())
+          _ptr(v_cache), waves, unroll, *scale, _stream())
     return q
 
 
@@ -352,7 +427,9 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
     accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose.
     With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2].
-    With ``tiled`` (``tile_weights(weight, order)``) the kernel streams that copy instead of the rows."""
+    With ``tiled`` (``tile_weights(weight, order)``) the kernel streams that copy instead of the rows.
+    ``x`` may be ``ScaledRows``."""
+    x, scale = _scale_args(x)
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     _check(weight, "weight", (None, K), torch.bfloat16)
@@ -367,9 +444,9 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
     if order is not None and (tiled is None or swiglu_pairs):
         raise KernelError("skinny_gemm: a tile order goes with a tiled copy and a plain product")
-    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", (P, P, P, I, I, I, I, I, I, I, I, I, P, P),
+    _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
           x.data_ptr(), (weight if tiled is None else tiled).data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves,
-          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else 1, _ptr(order), _stream())
+          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else 1, _ptr(order), *scale, 0, 0, 0, 0, _stream())
     return out
 
 
@@ -406,13 +483,15 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> 
     always comes from float accumulators, never through a bfloat16 rounding.
     """
     tiled = order = None
+    if isinstance(x, ScaledRows) and not takes_scaled_rows(x.shape[0], weight):
+        raise KernelError(f"linear: scaled rows are not taken for {x.shape[0]} rows and this weight")
     if isinstance(weight, LinearWeight):
         weight, tiled, order = weight.rows, weight.tiled, weight.order
     if weight.dtype == torch.float32:
         return gemm_f32(x, weight, None, out_dtype or x.dtype)
     if weight.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
         raise KernelError(f"linear: weight {weight.dtype} with activation {x.dtype} is not supported")
-    _check(x, "x", (None, weight.shape[1]))
+    _check(x if not isinstance(x, ScaledRows) else x.rows, "x", (None, weight.shape[1]))
     _check(weight, "weight", (None, None))
     out_dtype = out_dtype or torch.bfloat16
     M, K = x.shape
@@ -445,6 +524,8 @@ def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
     rows of Wg and Wu.  For few rows the activation is the product's epilogue; otherwise a second kernel
     applies it."""
     M, K = x.shape
+    if isinstance(x, ScaledRows) and not takes_scaled_rows(M, weight_pairs):
+        raise KernelError(f"linear_swiglu: scaled rows are not taken for {M} rows and this weight")
     rows, tiled = (weight_pairs.rows, weight_pairs.tiled) if isinstance(weight_pairs, LinearWeight) else (weight_pairs, None)
     if isinstance(weight_pairs, LinearWeight) and weight_pairs.order is not None:
         raise KernelError("linear_swiglu: a tile order is not supported for gate/up pairs")

@@ -76,7 +76,17 @@ class PagedAttention(Mixer):
             order = torch.tensor(ops.pair_tile_order(heads, self.head_dim), dtype=torch.int32, device=weight.device)
         return ops.prepare_linear(weight, order)
 
-    def forward(self, h: torch.Tensor, ctx, binding: MixerBinding) -> torch.Tensor:
+    adds_to_stream = True
+
+    def accepts_scaled_rows(self, n_rows: int) -> bool:
+        return not self.position.needs_apply and ops.takes_scaled_rows(n_rows, self.w_qkv)
+
+    def _project_out(self, out, sink):
+        if sink is not None and ops.adds_into_stream(out.shape[0], self.w_o, sink.norm_weight):
+            return ops.linear_into_stream(out, self.w_o, sink.stream, sink.norm_weight, sink.eps)
+        return ops.linear(out, self.w_o)
+
+    def forward(self, h, ctx, binding: MixerBinding, sink=None):
         cache = binding.cache
         nH, d = self.n_heads, self.head_dim
         nKV = self.n_kv_heads if binding.writes_cache else 0
@@ -93,15 +103,14 @@ class PagedAttention(Mixer):
             # few tokens: the rotation and the cache write are the projection's epilogue
             q = ops.qkv_rope_append(h, w, b, slots, cos, sin, nH, nKV, d, cache.k if slots is not None else None,
                                     cache.v if slots is not None else None, cache.page_size)
-            return ops.linear(paged_attention(q, cache, ctx, self.window, self.scale), self.w_o)
+            return self._project_out(paged_attention(q, cache, ctx, self.window, self.scale), sink)
         qkv = ops.linear(h, w)
         if self.position.needs_apply:
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
         q = ops.rope_append(qkv, b, slots, cos, sin, style, rotary_dim, nH, nKV, d,
                             cache.k if slots is not None else None, cache.v if slots is not None else None,
                             cache.page_size)
-        out = paged_attention(q, cache, ctx, self.window, self.scale)
-        return ops.linear(out, self.w_o)
+        return self._project_out(paged_attention(q, cache, ctx, self.window, self.scale), sink)
 
     def _encode_outside(self, qkv, bias, ctx, nKV):
         """For a position part that transforms q and k itself: add the bias, let the part encode,

@@ -20,6 +20,17 @@ Categories and what each must provide beyond ``param_specs`` / ``load``:
             where ``pending`` is a delta not yet added to the stream (the next norm adds it).
   embedding forward(token_ids) -> float32 stream [T, H].
   head      forward(normalised rows) -> float32 logits [R, V].
+
+A norm's kernel can be saved for steps of few rows, where a launch costs as much as the work.  This is
+optional for every part; one that declares nothing is run as above.
+
+  norm      ``rms_params()`` -> (weight, eps) if the norm is x * rsqrt(mean(x^2) + eps) * weight, else None.
+  mixer,    ``adds_to_stream`` True: forward takes ``sink=StreamSink(stream, weight, eps)`` (or None) and may
+  ffn       then add its result to the stream itself and return ``ScaledRows`` (the rows the norm that follows
+            would give, up to a factor per row; kernels/ops.py) instead of a delta.
+            ``accepts_scaled_rows(n_rows)`` True: forward takes ``ScaledRows`` for h.
+  block     ``entry_norm()`` -> the norm that first reads the stream, if ``pending`` may be ``ScaledRows`` made
+            for it; forward then takes ``following=`` the next block's entry norm (or None).
 """
 from __future__ import annotations
 
@@ -108,7 +119,21 @@ class MixerBinding:
     state: Optional[torch.Tensor] = None
 
 
+@dataclasses.dataclass
+class StreamSink:
+    """Where a mixer or feed-forward may add its result itself: the float32 stream, and the weight and eps
+    of the RMS norm that reads the stream next."""
+    stream: torch.Tensor
+    norm_weight: torch.Tensor
+    eps: float
+
+
 class Mixer(Part):
+    adds_to_stream = False
+
+    def accepts_scaled_rows(self, n_rows: int) -> bool:
+        return False
+
     def cache_spec(self) -> Optional[CacheSpec]:
         return None
 
@@ -120,16 +145,27 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    adds_to_stream = False
+
+    def accepts_scaled_rows(self, n_rows: int) -> bool:
+        return False
+
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         raise NotImplementedError
 
 
 class Norm(Part):
+    def rms_params(self):
+        return None
+
     def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
 
 class Block(Part):
+    def entry_norm(self) -> Optional[Norm]:
+        return None
+
     def forward(self, residual, pending, ctx, binding: MixerBinding):
         raise NotImplementedError

@@ -52,5 +52,13 @@ class SwiGLU(FeedForward):
             torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous())
         self.w_down = ops.prepare_linear(tensors[f"{self.name}.down_proj.weight"])
 
-    def forward(self, h, ctx):
-        return ops.linear(ops.linear_swiglu(h, self.w_gate_up), self.w_down)
+    adds_to_stream = True
+
+    def accepts_scaled_rows(self, n_rows: int) -> bool:
+        return ops.takes_scaled_rows(n_rows, self.w_gate_up)
+
+    def forward(self, h, ctx, sink=None):
+        a = ops.linear_swiglu(h, self.w_gate_up)
+        if sink is not None and ops.adds_into_stream(a.shape[0], self.w_down, sink.norm_weight):
+            return ops.linear_into_stream(a, self.w_down, sink.stream, sink.norm_weight, sink.eps)
+        return ops.linear(a, self.w_down)

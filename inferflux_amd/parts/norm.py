@@ -28,5 +28,8 @@ class RMSNorm(Norm):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[f"{self.name}.weight"]
 
+    def rms_params(self):
+        return self.weight, self.eps
+
     def forward(self, residual, delta, out_dtype, rows=None):
         return ops.add_rmsnorm(residual, delta, self.weight, self.eps, out_dtype, rows)

@@ -244,6 +244,41 @@ def test_a_layer_that_reads_another_entries_cache_in_bfloat16():
     assert rel_err(cb, w32) < REL_TOL["bfloat16"] and rel_err(wb, w32) < REL_TOL["bfloat16"]
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_steps_of_few_rows_need_no_kernel_for_the_norms_between_products(name, sharp_folders, monkeypatch):
+    """In bfloat16 a step of up to 16 rows adds each sub-block's output to the stream in its last product's epilogue
+    and applies the next norm's factor in the next product: only the first layer's first norm and the final norm
+    keep a kernel.  Logits agree with the plain model, and with the same step run with a kernel for every norm."""
+    from inferflux_amd.kernels import ops
+    folder, V, L = sharp_folders[name, "bfloat16"], TINY[name]["vocab_size"], TINY[name]["num_hidden_layers"]
+    ids = seeded_ids(31, 60, V)
+    want = plain_logits(folder, ids)
+    calls = []
+    real = ops.add_rmsnorm
+    monkeypatch.setattr(ops, "add_rmsnorm", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
+
+    def run(runner):
+        runner.decode_graphs = False              # every step eagerly: replays call nothing from Python
+        runner.add_request("n")
+        out, at = [], 0
+        for m in (17, 16, 1, 9, 16, 1):
+            calls.clear()
+            out.append(runner.step([StepEntry("n", ids[at:at + m], list(range(m)))]).cpu()); at += m
+            yield_calls.append((m, len(calls)))
+        runner.free_request("n")
+        return torch.cat(out)
+
+    yield_calls = []
+    fused = run(load_runner(folder, torch.bfloat16, num_pages=16))
+    assert yield_calls == [(17, 2 * L + 1)] + [(m, 2) for m in (16, 1, 9, 16, 1)], yield_calls
+    monkeypatch.setattr(ops, "adds_into_stream", lambda *a: False)
+    yield_calls = []
+    separate = run(load_runner(folder, torch.bfloat16, num_pages=16))
+    assert all(n == 2 * L + 1 for _, n in yield_calls), yield_calls
+    assert rel_err(fused, want[:60]) < REL_TOL["bfloat16"] and rel_err(separate, want[:60]) < REL_TOL["bfloat16"]
+    assert rel_err(fused, separate) < REL_TOL["bfloat16"]
+
+
 # ---- captured decode steps ----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C"])

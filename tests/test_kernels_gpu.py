@@ -575,6 +575,104 @@ def test_linear_swiglu_pairs(M):
     assert torch.allclose(got32, gt / (1 + torch.exp(-gt)) * up, rtol=1e-4, atol=1e-4)
 
 
+def _stream_case(M, N, K, seed, copy):
+    g = gen(seed)
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(BF16)
+    stream = torch.randn(M, N, generator=g) * 2.0
+    nw = (1 + 0.3 * torch.randn(N, generator=g)).to(BF16)
+    lw = ops.LinearWeight(w.to(DEV), ops.tile_weights(w.to(DEV)) if copy else None)
+    return x, w, stream, nw, lw
+
+
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,K", [(100, 72), (3584, 512), (36, 1000), (4100, 64)])
+@pytest.mark.parametrize("copy", [False, True])
+def test_product_added_to_the_stream_with_the_next_norm_prepared(M, N, K, copy):
+    x, w, stream, nw, lw = _stream_case(M, N, K, 30, copy)
+    s = stream.to(DEV)
+    got = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), 1e-5)
+    want = stream.double() + x.double() @ w.double().t()
+    assert torch.allclose(s.cpu().double(), want, rtol=1e-5, atol=1e-5)               # float sums, no rounding of the delta
+    assert got.rows.dtype == BF16 and got.width == N
+    assert torch.allclose(got.rows.cpu().double(), want * nw.double(), **tol(BF16))   # one rounding
+    assert got.pieces.shape == (-(-N // 16), 16)
+    sq = torch.nn.functional.pad(want ** 2, (0, -N % 16)).reshape(M, -1, 16).sum(-1)   # [M, pieces]
+    assert torch.allclose(got.pieces.cpu().double()[:, :M], sq.t(), rtol=1e-5, atol=1e-7)
+    assert float(got.pieces[:, M:].abs().max()) == 0.0 if M < 16 else True
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("copy", [False, True])
+def test_row_factors_are_applied_by_the_product_that_reads_the_rows(M, copy):
+    """The norm's factor per row, applied to sums instead of to the input: the same as norm, then product."""
+    H, I, eps = 200, 300, 1e-3
+    x, w, stream, nw, lw = _stream_case(M, H, 136, 31, copy)
+    s = stream.to(DEV)
+    scaled = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), eps)
+    rows = scaled.rows.cpu().double()
+    normed = pm.rms_norm(s.cpu().double(), nw.double(), eps)              # what the norm's own kernel would give
+    factor = torch.rsqrt((s.cpu().double() ** 2).mean(-1, keepdim=True) + eps)
+    assert torch.allclose(rows * factor, normed, **tol(BF16))
+    g = gen(32)
+    w2 = (torch.randn(I, H, generator=g) * 0.2).to(BF16)
+    lw2 = ops.LinearWeight(w2.to(DEV), ops.tile_weights(w2.to(DEV)) if copy else None)
+    assert ops.takes_scaled_rows(M, lw2) and not ops.takes_scaled_rows(17, lw2)
+    got = ops.linear(scaled, lw2).cpu().double()
+    assert torch.allclose(got, (rows @ w2.double().t()) * factor, **tol(BF16))         # same rounded inputs: one rounding
+    assert torch.allclose(got, normed @ w2.double().t(), rtol=2e-2, atol=2e-2)         # and the function it stands for
+    got32 = ops.linear(scaled, lw2, torch.float32).cpu().double()
+    assert torch.allclose(got32, (rows @ w2.double().t()) * factor, rtol=1e-4, atol=1e-4)
+    gt, up = (rows @ w2[0::2].double().t()) * factor, (rows @ w2[1::2].double().t()) * factor
+    act = ops.linear_swiglu(scaled, lw2).cpu().double()
+    assert torch.allclose(act, gt / (1 + torch.exp(-gt)) * up, **tol(BF16))
+
+
+def test_row_factors_in_the_fused_qkv_product():
+    M, d, nH, nKV, K, P, eps = 6, 32, 3, 1, 96, 16, 1e-6
+    g = gen(33)
+    x, w, stream, nw, lw = _stream_case(M, K, 40, 33, True)
+    s = stream.to(DEV)
+    scaled = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), eps)
+    heads = nH + 2 * nKV
+    wq = (torch.randn(heads * d, K, generator=g) * 0.2).to(BF16)
+    bias = torch.randn(heads * d, generator=g).to(BF16)
+    order = torch.tensor(ops.pair_tile_order(heads, d), dtype=torch.int32, device=DEV)
+    lq = ops.prepare_linear(wq.to(DEV), order)
+    cos, sin = ops.rope_table(torch.arange(M, dtype=torch.int32, device=DEV) + 3, (1.0 / 10000 ** (torch.arange(d // 2) * 2.0 / d)).to(DEV))
+    slots = torch.arange(M, dtype=torch.int32, device=DEV)
+
+    def run(h):
+        kc, vc = torch.zeros(1, nKV, P, d, dtype=BF16, device=DEV), torch.zeros(1, nKV, d, P, dtype=BF16, device=DEV)
+        return ops.qkv_rope_append(h, lq, bias.to(DEV), slots, cos, sin, nH, nKV, d, kc, vc, P), kc, vc
+
+    q1, k1, v1 = run(scaled)
+    # the same with the factor applied to the rows beforehand, in float, by a weight that cannot round: compare with the
+    # plain product on the normalised rows
+    factor = torch.rsqrt((s.cpu().double() ** 2).mean(-1, keepdim=True) + eps)
+    qkv = (scaled.rows.cpu().double() @ wq.double().t()) * factor + bias.double()
+    want_v = qkv[:, (nH + nKV) * d:].reshape(M, nKV, d)
+    assert torch.allclose(v1[0, :, :, :M].permute(2, 0, 1).cpu().double(), want_v, **tol(BF16))
+    c, sn = cos.cpu().double(), sin.cpu().double()
+    qq = qkv[:, : nH * d].reshape(M, nH, d)
+    lo, hi = qq[..., : d // 2], qq[..., d // 2:]
+    want_q = torch.cat([lo * c[:, None] - hi * sn[:, None], lo * sn[:, None] + hi * c[:, None]], -1)
+    assert torch.allclose(q1.cpu().double(), want_q, **tol(BF16))
+
+
+def test_scaled_rows_are_refused_where_no_kernel_applies_them():
+    x, w, stream, nw, lw = _stream_case(4, 64, 32, 34, True)
+    scaled = ops.linear_into_stream(x.to(DEV), lw, stream.to(DEV), nw.to(DEV), 1e-5)
+    with pytest.raises(ops.KernelError, match="scaled rows"):
+        ops.linear(scaled, torch.randn(8, 64, device=DEV))                          # a float32 weight
+    with pytest.raises(ops.KernelError, match="scaled rows"):
+        ops.linear(scaled, torch.randn(8, 64, device=DEV).bfloat16())               # a bare tensor
+    with pytest.raises(ops.KernelError, match="linear_into_stream"):
+        ops.linear_into_stream(torch.zeros(17, 32, dtype=BF16, device=DEV), lw, torch.zeros(17, 64, device=DEV), nw.to(DEV), 1e-5)
+    with pytest.raises(ops.KernelError, match="linear_into_stream"):               # a float32 norm weight
+        ops.linear_into_stream(x.to(DEV), lw, stream.to(DEV), nw.float().to(DEV), 1e-5)
+
+
 @pytest.mark.parametrize("M", [1, 7, 16, 33, 64])
 @pytest.mark.parametrize("N,K,slices", [(50, 64, 0), (3, 8, 0), (130, 200, 2), (577, 1000, 0), (4608, 3584, 0), (200, 2104, 5)])
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
