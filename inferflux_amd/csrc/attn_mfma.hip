@@ -111,21 +111,23 @@ struct RowArgs {
 };
 
 // The operands of one block of 32 keys (two pages' worth of 16): loaded together, K and V at once,
-// so that a block costs one trip to memory, and one block ahead of the arithmetic.
+// so that a block costs one trip to memory, and one block ahead of the arithmetic.  The page numbers come
+// from a register: lane i of ``pages`` holds entry ``page_base + i`` of the request's block table, read once
+// for 64 pages, so that no block waits for a table entry before it can ask for its keys.
 struct RowBlock {
   bf16x8 k[2][KS];
   bf16x4 v[DT][2];
   bool live[2];
 };
 
-__device__ __forceinline__ void load_row_block(RowBlock& b, const RowArgs& a, const int* table, int kvh, int j0,
+__device__ __forceinline__ void load_row_block(RowBlock& b, const RowArgs& a, int pages, int page_base, int kvh, int j0,
                                                int ka, int kb, int col, int g4) {
   const int P = a.P;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int k0 = j0 + 16 * t;  // 16 keys k0..k0+15, all in one page
     bool live = k0 < kb && k0 + 16 > ka;
-    const int page = live ? table[k0 / P] : -1;
+    const int page = live ? __builtin_amdgcn_readlane(pages, k0 / P - page_base) : -1;
     live = live && page >= 0;
     b.live[t] = live;
     const int off = k0 % P;
@@ -213,13 +215,29 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 
     RowBlock b0, b1;
     int j0 = (ka / 32) * 32;
-    load_row_block(b0, a, table, kvh, j0, ka, kb, col, g4);
+    int page_base = 0, pages = -1;
+    bool have_pages = false;
+    // the table entries of the block of 32 keys from j: in ``pages`` already, or read now (64 entries from j's)
+    auto table_for = [&](int j) {
+      if (have_pages && (j + 31) / a.P - page_base < WAVE) return;
+      have_pages = true;
+      page_base = j / a.P;
+      pages = page_base + lane < a.max_blocks ? table[page_base + lane] : -1;
+    };
+    table_for(j0);
+    load_row_block(b0, a, pages, page_base, kvh, j0, ka, kb, col, g4);
     for (; j0 < kb; j0 += 64) {
       const bool more1 = j0 + 32 < kb, more2 = j0 + 64 < kb;
-      if (more1) load_row_block(b1, a, table, kvh, j0 + 32, ka, kb, col, g4);
+      if (more1) {
+        table_for(j0 + 32);
+        load_row_block(b1, a, pages, page_base, kvh, j0 + 32, ka, kb, col, g4);
+      }
       use_row_block(b0, a, qop, o, m, l, j0, ka, kb, g4);
       if (more1) {
-        if (more2) load_row_block(b0, a, table, kvh, j0 + 64, ka, kb, col, g4);
+        if (more2) {
+          table_for(j0 + 64);
+          load_row_block(b0, a, pages, page_base, kvh, j0 + 64, ka, kb, col, g4);
+        }
         use_row_block(b1, a, qop, o, m, l, j0 + 32, ka, kb, g4);
       }
     }

@@ -8,7 +8,7 @@ Sizes default to the Qwen2.5-7B shape (28 query heads, 4 kv heads, head size 128
 intermediate 18944).  Times are averages of back-to-back launches between two events and include what
 the Python wrapper costs per call (10-15 us): for kernels that short, read the kernel's own time from
 ``rocprofv3 --kernel-trace`` around this program instead.  Products rotate through enough copies of the
-weight that no launch finds it in a cache.
+weight, and row attention through enough caches, that no launch finds its operands in a cache.
 """
 from __future__ import annotations
 
@@ -57,8 +57,10 @@ def attention_tiles(args) -> None:
 def attention_rows(args) -> None:
     dev, B, kv, nH, nKV, d, P = "cuda", args.batch, args.context, args.heads, args.kv_heads, args.head_dim, args.page_size
     nb = -(-kv // P)
-    kc = torch.randn(B * nb, nKV, P, d, device=dev, dtype=torch.bfloat16)
-    vc = torch.randn(B * nb, nKV, d, P, device=dev, dtype=torch.bfloat16)
+    # enough caches to rotate through that no launch finds its keys and values in the last-level cache
+    copies = max(2, min(16, int(2e9 // (2 * B * nb * nKV * P * d * 2))))
+    caches = [(torch.randn(B * nb, nKV, P, d, device=dev, dtype=torch.bfloat16),
+               torch.randn(B * nb, nKV, d, P, device=dev, dtype=torch.bfloat16)) for _ in range(copies)]
     table = torch.randperm(B * nb, device=dev).to(torch.int32).view(B, nb).contiguous()
     q = torch.randn(B, nH, d, device=dev, dtype=torch.bfloat16)
     out = torch.empty(B, nH * d, device=dev, dtype=torch.bfloat16)
@@ -66,8 +68,8 @@ def attention_rows(args) -> None:
     pos = torch.full((B,), kv - 1, dtype=torch.int32, device=dev)
     for chunk in ([args.chunk] if args.chunk else [128, 256, 512, 1024]):
         splits = -(-kv // chunk)
-        t = _time_us(lambda i: ops.attention_rows(q, kc, vc, out, None, B, row_req, pos, table, None, 1 / math.sqrt(d), chunk, splits),
-                     args.iters)
+        t = _time_us(lambda i: ops.attention_rows(q, *caches[i % copies], out, None, B, row_req, pos, table, None,
+                                                  1 / math.sqrt(d), chunk, splits), args.iters)
         gb = B * kv * nKV * d * 2 * 2 / 1e9
         print(f"attention-rows batch={B} context={kv} chunk={chunk} splits={splits}: {t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache "
               f"(row kernel + merge)", flush=True)
