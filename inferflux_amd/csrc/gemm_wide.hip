@@ -1,0 +1,227 @@
+// Weight-streaming matrix product for 17-64 rows:  out[M,N] = x[M,K] * W[N,K]^T from the tiled copy of W
+// (layout: gemm_bf16.hip), bf16 in, float accumulate on the matrix cores (16x16x32), out bf16 or float.
+//
+// At these sizes the product is still bound by reading W once, but every tile of W now meets two to four
+// tiles of x, and a wave that fetched those from the L2 itself would move more bytes of x than of W.  A
+// workgroup of 8-16 waves therefore owns one tile of 16 weight rows per wave and one slice of K, and the
+// rows of x for the next 128 k-values are copied to LDS once per workgroup (two buffers, one barrier per
+// round of 128) and read from there by every wave.  Each wave streams its own tile row of W, one
+// contiguous kilobyte per load with streaming loads, DEPTH rounds ahead of the arithmetic; the rows of x are
+// asked for as far ahead and wait in registers (a round's arithmetic is much shorter than a trip to the L2).
+//
+// How many waves and slices: what a compute unit can have on its way from memory is bounded, so the time is
+// set by the unit with the most bytes to fetch, x included.  Measured on the 7B shapes, the best launch has
+// about one workgroup for each of the 256 units, as many waves in it as that takes (8-16), and K cut into
+// slices where the weight has too few rows for that (ifx_wide_gemm_plan).
+//
+// x in LDS: the 16-byte piece (row r, k-piece j of the round's 16) lies at slot j R + (r + j) % R of the
+// buffer (R = 16 MT rows).  A wave reads its B operand of (k-tile kt, x tile mt) as 16-byte pieces
+// j = 4 kt + g of rows 16 mt + col: sixteen consecutive slots per group of 16 lanes, no bank conflict; the
+// shift by j keeps the stores of 16 consecutive pieces of one row apart as well.
+//
+// With more than one slice of K the slices write float partial sums and a second kernel adds them in slice
+// order; the result never depends on timing.
+//
+// The reference sends these products to cuBLAS (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).
+#include "common.h"
+
+IFX_DEFINE_LAST_ERROR()
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+constexpr int DEPTH = 3;                                           // rounds of W and x on their way
+constexpr int MIN_WAVES = 8, MAX_WAVES = 16;
+constexpr int WK = 128, WK_TILES = WK / 32, WK_PIECES = WK / 8;   // k-values, k-tiles and 16-byte pieces of a round
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// EPI 0: out[m, n] = sum.  EPI 1: the rows of W alternate gate, up, ...: out[m, n / 2] = silu(gate) * up.
+// ``order``: tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
+template <int MT, typename TO, int EPI>
+__global__ __launch_bounds__(MAX_WAVES * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
+                                                                     TO* __restrict__ out, float* __restrict__ part, int M,
+                                                                     int N, int K, int k_tiles, int rounds_per_slice,
+                                                                     const int* __restrict__ order) {
+  constexpr int R = MT * 16;                                  // rows of x in LDS
+  constexpr int X_PIECES = R * WK_PIECES;                     // 16-byte pieces of a round's x
+  constexpr int X_PER_THREAD = (X_PIECES + MIN_WAVES * WAVE - 1) / (MIN_WAVES * WAVE);
+  __shared__ __attribute__((aligned(16))) bf16x8 xs[2][X_PIECES];
+  const int tid = threadIdx.x, threads = blockDim.x, waves = threads / WAVE;
+  const int wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x * waves + wid, n_tiles = (N + 15) / 16;
+  const int n_rounds = (K + WK - 1) / WK;
+  const int r_begin = blockIdx.y * rounds_per_slice, n = min(n_rounds, r_begin + rounds_per_slice) - r_begin;
+  // a wave whose tile lies past N reads the last tile again and stores nothing
+  const bf16_t* wtile = Wt + ((size_t)min(tile, n_tiles - 1) * k_tiles * WAVE + lane) * 8;
+  floatx4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 wreg[DEPTH][WK_TILES];
+  bf16x8 xreg[DEPTH][X_PER_THREAD];
+
+  auto load_w = [&](int r, bf16x8 (&w)[WK_TILES]) {
+#pragma unroll
+    for (int kt = 0; kt < WK_TILES; ++kt) {
+      const int t = r * WK_TILES + kt;
+      w[kt] = t < k_tiles ? __builtin_nontemporal_load((const bf16x8*)(wtile + (size_t)t * WAVE * 8)) : zero8();
+    }
+  };
+  auto load_x = [&](int r, bf16x8 (&xp)[X_PER_THREAD]) {
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; ++i) {
+      const int p = tid + threads * i, row = p / WK_PIECES, k = r * WK + 8 * (p % WK_PIECES);
+      xp[i] = (p < X_PIECES && row < M && k < K) ? *(const bf16x8*)(x + (size_t)row * K + k) : zero8();
+    }
+  };
+  auto store_x = [&](int buf, const bf16x8 (&xp)[X_PER_THREAD]) {
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; ++i) {
+      const int p = tid + threads * i, row = p / WK_PIECES, j = p % WK_PIECES;
+      if (p < X_PIECES) xs[buf][j * R + (row + j) % R] = xp[i];
+    }
+  };
+  auto compute = [&](const bf16x8 (&w)[WK_TILES], int buf) {
+#pragma unroll
+    for (int kt = 0; kt < WK_TILES; ++kt) {
+      const int j = 4 * kt + g;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[kt], xs[buf][j * R + (16 * mt + col + j) % R], acc[mt], 0, 0, 0);
+    }
+  };
+  // register set d holds W and x of the rounds c with c % DEPTH == d
+  if (n > 0) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (d < n) {
+        load_x(r_begin + d, xreg[d]);
+        load_w(r_begin + d, wreg[d]);
+      }
+    store_x(0, xreg[0]);
+    if (DEPTH < n) load_x(r_begin + DEPTH, xreg[0]);
+  }
+  __syncthreads();
+  for (int c0 = 0; c0 < n; c0 += 2 * DEPTH) {   // unrolled over the register sets and the two LDS buffers
+#pragma unroll
+    for (int dd = 0; dd < 2 * DEPTH; ++dd) {
+      const int c = c0 + dd;
+      if (c >= n) break;   // the same for every thread
+      compute(wreg[dd % DEPTH], dd & 1);
+      if (c + DEPTH < n) load_w(r_begin + c + DEPTH, wreg[dd % DEPTH]);
+      if (c + 1 < n) {     // the other buffer was last read in round c - 1, which every wave has left
+        store_x((dd + 1) & 1, xreg[(dd + 1) % DEPTH]);
+        if (c + 1 + DEPTH < n) load_x(r_begin + c + 1 + DEPTH, xreg[(dd + 1) % DEPTH]);
+      }
+      __syncthreads();
+    }
+  }
+  if (tile >= n_tiles) return;
+  // acc[mt][r] = out[m = 16 mt + col][n = 16 (row tile of the weight) + 4 g + r]
+  const int n0 = 16 * (order ? order[tile] : tile) + 4 * g;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + col;
+    if (m >= M) continue;
+    if (gridDim.y > 1) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < N) part[((size_t)blockIdx.y * M + m) * N + n0 + r] = acc[mt][r];
+    } else if (EPI == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < N) out[(size_t)m * N + n0 + r] = from_f<TO>(acc[mt][r]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; r += 2) {   // even: gate at n0 + r, up at n0 + r + 1
+        const float gt = acc[mt][r], up = acc[mt][r + 1];
+        if (n0 + r + 1 < N) out[(size_t)m * (N / 2) + (n0 + r) / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+      }
+    }
+  }
+}
+
+template <typename TO>
+__global__ void wide_sum_slices_kernel(const float* __restrict__ part, TO* __restrict__ out, int S, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float a = 0.f;
+  for (int s = 0; s < S; ++s) a += part[(size_t)s * n + i];
+  out[i] = from_f<TO>(a);
+}
+
+// Waves per workgroup and slices of K for a shape.  ``waves`` / ``slices`` 0: chosen here (about one workgroup
+// for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
+// several workgroups to a unit; then slices of at least four rounds, at most eight); the gate/up epilogue takes
+// one slice.  Returns waves * 256 + slices.
+extern "C" int ifx_wide_gemm_plan(int N, int K, int waves, int slices, int epi) {
+  const int n_tiles = (N + 15) / 16, n_rounds = (K + WK - 1) / WK;
+  if (waves <= 0) waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
+  waves = waves < MIN_WAVES ? MIN_WAVES : (waves > MAX_WAVES ? MAX_WAVES : waves);
+  const int groups = (n_tiles + waves - 1) / waves;
+  if (epi != 0) slices = 1;
+  if (slices <= 0) {
+    slices = 256 / groups;
+    if (slices > 8) slices = 8;
+    if (slices > n_rounds / 4) slices = n_rounds / 4;
+  }
+  if (slices < 1) slices = 1;
+  if (slices > n_rounds) slices = n_rounds;
+  const int rps = (n_rounds + slices - 1) / slices;
+  return waves * 256 + (n_rounds + rps - 1) / rps;
+}
+
+template <int MT>
+static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K, int waves,
+                       int slices, int rps, int epi, const int* order, hipStream_t s) {
+  const int n_tiles = (N + 15) / 16;
+  const dim3 grid((n_tiles + waves - 1) / waves, slices);
+  const int k_tiles = (K + 63) / 64 * 2;
+#define GO(TO_, EPI_)                                                                                         \
+  hipLaunchKernelGGL((wide_gemm_kernel<MT, TO_, EPI_>), grid, dim3(waves * WAVE), 0, s, (const bf16_t*)x,     \
+                     (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order)
+  if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
+  else if (out_dtype == DT_BF16) GO(bf16_t, 1);
+  else if (epi == 0) GO(float, 0);
+  else GO(float, 1);
+#undef GO
+  if (slices > 1) {
+    const size_t n = (size_t)M * N;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out_dtype == DT_BF16) hipLaunchKernelGGL(wide_sum_slices_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, part, (bf16_t*)out, slices, n);
+    else hipLaunchKernelGGL(wide_sum_slices_kernel<float>, dim3(blocks), dim3(256), 0, s, part, (float*)out, slices, n);
+  }
+  IFX_LAUNCH_CHECK();
+}
+
+// x [M <= 64, K] times the tiled copy Wt of W [N, K], transposed.  ``waves``, ``slices``: as ifx_wide_gemm_plan
+// returned them; ``part``: slices * M * N floats when there is more than one slice.
+// epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2] (one slice, no tile order).
+// order: the row-tile order the copy was written with (or null).
+extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K,
+                             int waves, int slices, int epi, const int* order, void* stream) {
+  IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "wide_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
+  IFX_REQUIRE(K % 8 == 0, "wide_gemm: K=%d must be a multiple of 8", K);
+  IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "wide_gemm: unknown out dtype %d", out_dtype);
+  IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0 && !order && slices == 1), "wide_gemm: epilogue %d with N=%d, %d slices%s", epi, N,
+              slices, order ? ", a tile order" : "");
+  const int n_rounds = (K + WK - 1) / WK;
+  IFX_REQUIRE(waves >= MIN_WAVES && waves <= MAX_WAVES && slices >= 1 && slices <= n_rounds, "wide_gemm: %d waves (%d-%d), %d slices of %d rounds",
+              waves, MIN_WAVES, MAX_WAVES, slices, n_rounds);
+  IFX_REQUIRE(slices == 1 || part, "wide_gemm: %d slices of K need a scratch buffer", slices);
+  if (M == 0) return 0;
+  const int rps = (n_rounds + slices - 1) / slices;
+  IFX_REQUIRE((n_rounds + rps - 1) / rps == slices, "wide_gemm: %d rounds do not cut into %d slices (ask ifx_wide_gemm_plan)", n_rounds, slices);
+  hipStream_t s = (hipStream_t)stream;
+  switch ((M + 15) / 16) {
+    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
+    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
+    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
+    default: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
+  }
+}

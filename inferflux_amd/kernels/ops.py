@@ -45,6 +45,7 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("attn_plain", ())
     yield ("sampling", ())
     yield ("gemm_bf16", ())
+    yield ("gemm_wide", ())
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
             yield ("attn_mfma", (("HEAD_DIM", d), ("TILE_QT", qt)))
@@ -450,6 +451,31 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
+def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
+              slices: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
+    """bfloat16 x [M <= 64, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
+    of a workgroup: the product for 17-64 rows.  ``waves`` (8-16 per workgroup, one tile of 16 weight rows each)
+    and ``slices`` of K (added in a fixed order): 0 lets the kernel choose."""
+    _check(x, "x", (None, None), torch.bfloat16)
+    M, K = x.shape
+    N = weight.rows.shape[0]
+    if weight.tiled is None or weight.rows.shape[1] != K or weight.rows.dtype != torch.bfloat16:
+        raise KernelError(f"wide_gemm: needs the tiled copy of a bfloat16 [N, {K}] weight")
+    if M > SKINNY_MAX_M or K % 8:
+        raise KernelError(f"wide_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
+    if swiglu_pairs and (N % 2 or weight.order is not None):
+        raise KernelError("wide_gemm: gate/up pairs need an even number of weight rows in their natural order")
+    mod = load_module("gemm_wide")
+    plan = mod.fn("ifx_wide_gemm_plan", (I, I, I, I, I))(N, K, waves, slices, 1 if swiglu_pairs else 0)
+    n_waves, n_slices = plan // 256, plan % 256
+    part = torch.empty((n_slices, M, N), dtype=torch.float32, device=x.device) if n_slices > 1 else None
+    out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
+    _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, P),
+          x.data_ptr(), weight.tiled.data_ptr(), out.data_ptr(), _DT[out_dtype], _ptr(part), M, N, K, n_waves, n_slices,
+          1 if swiglu_pairs else 0, _ptr(weight.order), _stream())
+    return out
+
+
 def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                 slices: int = 0, unroll: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
     """The same product as skinny_gemm with x staged in LDS and shared by the waves of a workgroup
@@ -498,6 +524,8 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> 
     kind = _small_m_kernel(M, weight.shape[0], K, tiled is not None)
     if kind == "skinny":
         return skinny_gemm(x, weight, out_dtype, tiled=tiled, order=order)
+    if kind == "wide":
+        return wide_gemm(x, LinearWeight(weight, tiled, order), out_dtype)
     if kind == "staged":
         return staged_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:
@@ -506,14 +534,17 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> 
 
 
 def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional[str]:
-    """Which of the two streaming kernels takes a bfloat16 product of this shape, or None for the
-    library.  Measured on the 7B shapes: streaming wins up to 16 rows everywhere (with x staged in LDS
-    for very tall weights such as the head's) and up to 32 rows on the narrow products; beyond that
-    the library's tiles reuse the rows better."""
+    """Which of the streaming kernels takes a bfloat16 product of this shape, or None for the library.
+    Measured on the 7B shapes: up to 16 rows the product that splits K over the waves of a workgroup (with x
+    staged in LDS for very tall weights such as the head's when there is no tiled copy); from 17 to 64 rows
+    the product that shares x through LDS, which needs the tiled copy (without it, the first kernel up to 32
+    rows on narrow weights); beyond that the library's tiles reuse the rows better."""
     if K % 8:
         return None
     if M <= 16:
         return "staged" if N >= 65536 and not has_tiled else "skinny"
+    if M <= SKINNY_MAX_M and has_tiled:
+        return "wide"
     if M <= 32 and N <= 4096:
         return "skinny"
     return None
@@ -533,6 +564,8 @@ def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
         kind = _small_m_kernel(M, rows.shape[0], K, tiled is not None)
         if kind == "skinny":
             return skinny_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, tiled=tiled)
+        if kind == "wide":
+            return wide_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
         if kind == "staged":
             return staged_gemm(x, rows, torch.bfloat16, swiglu_pairs=True)
     return swiglu(linear(x, rows), interleaved=True)

@@ -523,6 +523,56 @@ def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, 
     assert torch.allclose(qq.float(), q.float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("M", [17, 32, 33, 50, 64])
+@pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136)])
+@pytest.mark.parametrize("out_dtype", [BF16, F32])
+def test_wide_gemm(M, N, K, out_dtype):
+    g = gen(40)
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = (torch.randn(N, K, generator=g) * 0.3).to(BF16)
+    want = x.double() @ w.double().t()
+    lw = ops.prepare_linear(w.to(DEV))
+    t = dict(rtol=1e-4, atol=3e-3) if out_dtype == F32 else dict(rtol=1e-2, atol=0.1)
+    got = ops.wide_gemm(x.to(DEV), lw, out_dtype).cpu().double()
+    assert got.shape == (M, N) and torch.allclose(got, want, **t), float((got - want).abs().max())
+    assert torch.equal(ops.linear(x.to(DEV), lw, out_dtype).cpu().double(), got)       # what linear picks at these rows
+
+
+@pytest.mark.parametrize("waves,slices", [(8, 1), (8, 3), (11, 2), (16, 1), (16, 8)])
+def test_wide_gemm_every_launch_shape_gives_the_same_product(waves, slices):
+    g = gen(41)
+    M, N, K = 41, 333, 1096                    # 9 rounds of 128 k-values, the last one short; 21 row tiles, the last one short
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = torch.randn(N, K, generator=g).to(BF16)
+    lw = ops.prepare_linear(w.to(DEV))
+    got = ops.wide_gemm(x.to(DEV), lw, F32, waves=waves, slices=slices).cpu().double()
+    assert torch.allclose(got, x.double() @ w.double().t(), rtol=1e-4, atol=3e-3)
+    lw.rows = torch.zeros_like(lw.rows)                                               # it reads the copy, not the rows
+    assert torch.equal(ops.wide_gemm(x.to(DEV), lw, F32, waves=waves, slices=slices).cpu().double(), got)
+
+
+def test_wide_gemm_gate_up_pairs_and_tile_order():
+    g = gen(42)
+    M, I2, K = 37, 2 * 301, 264
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = (torch.randn(I2, K, generator=g) * 0.2).to(BF16)
+    ref = x.double() @ w.double().t()
+    gt, up = ref[:, 0::2], ref[:, 1::2]
+    got = ops.linear_swiglu(x.to(DEV), ops.prepare_linear(w.to(DEV))).cpu().double()
+    assert got.shape == (M, I2 // 2) and torch.allclose(got, gt / (1 + torch.exp(-gt)) * up, rtol=2e-2, atol=2e-2)
+    heads, d = 5, 32                                                                   # 160 rows in pair order, as q/k/v has them
+    wq = (torch.randn(heads * d, K, generator=g) * 0.2).to(BF16)
+    order = torch.tensor(ops.pair_tile_order(heads, d), dtype=torch.int32, device=DEV)
+    lq = ops.prepare_linear(wq.to(DEV), order)
+    out = ops.linear(x.to(DEV), lq, F32).cpu().double()
+    assert torch.allclose(out, x.double() @ wq.double().t(), rtol=1e-4, atol=3e-3)
+    with pytest.raises(ops.KernelError, match="wide_gemm"):
+        ops.wide_gemm(x.to(DEV), lq, BF16, swiglu_pairs=True)                          # pairs in a permuted copy
+    with pytest.raises(ops.KernelError, match="wide_gemm"):
+        ops.wide_gemm(torch.zeros(65, K, dtype=BF16, device=DEV), lq)
+    assert torch.equal(ops.wide_gemm(x.to(DEV), lq, F32, waves=3).cpu().double(), out)    # fewer than 8 waves: taken as 8
+
+
 def test_linear_weight_uses_the_copy_for_few_rows_and_the_rows_beyond():
     g = gen(17)
     w = torch.randn(200, 136, generator=g).to(BF16).to(DEV)
