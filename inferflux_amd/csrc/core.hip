@@ -46,17 +46,23 @@ template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                    const void* __restrict__ weight, int weight_dtype,
                                    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps,
-                                   int write_back) {
+                                   int write_back, int n_slices, size_t slice_stride) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
   float* res = residual + src * H;
   const TD* dl = delta ? delta + src * H : nullptr;
+  // the delta may come as partial sums: slice s lies slice_stride elements after slice s - 1
+  auto delta_at = [&](int i) {
+    float d = to_f(dl[i]);
+    for (int s = 1; s < n_slices; ++s) d += to_f(dl[(size_t)s * slice_stride + i]);
+    return d;
+  };
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float x = res[i];
     if (dl) {
-      x += to_f(dl[i]);
+      x += delta_at(i);
       if (write_back) res[i] = x;
     }
     ss += x * x;
@@ -66,7 +72,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   TO* o = out + (size_t)r * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float x = res[i];
-    if (dl && !write_back) x += to_f(dl[i]);
+    if (dl && !write_back) x += delta_at(i);
     o[i] = from_f<TO>(x * rms * load_dyn(weight, weight_dtype, i));
   }
 }
@@ -100,7 +106,8 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const floa
 template <typename TD, typename TO, typename TW, int NV>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                                               const TW* __restrict__ weight, TO* __restrict__ out,
-                                                              const int* __restrict__ rows, int H, float eps, int write_back) {
+                                                              const int* __restrict__ rows, int H, float eps, int write_back,
+                                                              int n_slices, size_t slice_stride) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -116,6 +123,18 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
       if (dl) {
         float d4[4];
         load4<TD>(dl + i, d4);
+        for (int s0 = 1; s0 < n_slices; s0 += 4) {   // partial sums, added in slice order; four loads go out together
+          float p4[4][4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (s0 + u < n_slices) load4<TD>(dl + (size_t)(s0 + u) * slice_stride + i, p4[u]);
+            else p4[u][0] = p4[u][1] = p4[u][2] = p4[u][3] = 0.f;
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) d4[e] += p4[u][e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) x[v][e] += d4[e];
         if (write_back) store4<float>(res + i, x[v]);
@@ -142,22 +161,25 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 
 template <typename TD, typename TO, typename TW>
 static void launch_rmsnorm_vec(float* residual, const void* delta, const void* weight, void* out, const int* rows,
-                               int n_rows, int H, float eps, int write_back, hipStream_t s) {
+                               int n_rows, int H, float eps, int write_back, int n_slices, size_t slice_stride, hipStream_t s) {
   if (H <= 4 * 256 * 2)
     hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 2>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
-                       (const TW*)weight, (TO*)out, rows, H, eps, write_back);
+                       (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);
   else if (H <= 4 * 256 * 4)
     hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 4>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
-                       (const TW*)weight, (TO*)out, rows, H, eps, write_back);
+                       (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);
   else
     hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 8>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
-                       (const TW*)weight, (TO*)out, rows, H, eps, write_back);
+                       (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);
 }
 
+// n_slices > 1: ``delta`` (float32) holds that many partial sums, slice_stride elements apart, added in order.
 extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* weight,
                                int weight_dtype, void* out, int out_dtype, const int* rows, int n_rows,
-                               int H, float eps, int write_back, void* stream) {
+                               int H, float eps, int write_back, int n_slices, long long slice_stride, void* stream) {
   IFX_REQUIRE(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || (delta && delta_dtype == DT_F32 && slice_stride > 0)),
+              "add_rmsnorm: %d slices need a float32 delta and their distance", n_slices);
   IFX_REQUIRE(!(rows && write_back), "add_rmsnorm: a row gather cannot write the residual back");
   if (n_rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
@@ -168,8 +190,8 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
   if (H % 4 == 0 && H <= 4 * 256 * 8) {
 #define VEC(TD, TO)                                                                                                  \
   do {                                                                                                               \
-    if (weight_dtype == DT_F32) launch_rmsnorm_vec<TD, TO, float>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, s); \
-    else launch_rmsnorm_vec<TD, TO, bf16_t>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, s);      \
+    if (weight_dtype == DT_F32) launch_rmsnorm_vec<TD, TO, float>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, n_slices, (size_t)slice_stride, s); \
+    else launch_rmsnorm_vec<TD, TO, bf16_t>(residual, delta, weight, out, rows, n_rows, H, eps, write_back, n_slices, (size_t)slice_stride, s);      \
   } while (0)
     if (dd == DT_F32 && out_dtype == DT_F32) VEC(float, float);
     else if (dd == DT_BF16 && out_dtype == DT_BF16) VEC(bf16_t, bf16_t);
@@ -181,7 +203,7 @@ extern "C" int ifx_add_rmsnorm(float* residual, const void* delta, int delta_dty
   const int threads = H >= 2048 ? 512 : 256;
 #define LAUNCH(TD, TO)                                                                              \
   hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(threads), 0, s, residual,     \
-                     (const TD*)delta, weight, weight_dtype, (TO*)out, rows, H, eps, write_back)
+                     (const TD*)delta, weight, weight_dtype, (TO*)out, rows, H, eps, write_back, n_slices, (size_t)slice_stride)
   if (dd == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
   else if (dd == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
   else if (dd == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
@@ -220,7 +242,9 @@ extern "C" int ifx_rope_table(const int* positions, const float* inv_freq, float
 // cos/sin come from the step's table [T, rotary_dim / 2]; elements at or beyond rotary_dim are
 // copied.  One block per (token, head): q heads, then k heads, then v heads.
 struct RopeArgs {
-  const void* qkv;
+  const void* qkv;       // [T, row width] of the activation type, or with n_slices > 1 float partial sums
+  int n_slices;          // [n_slices][T, row width], slice_stride elements apart, added in order
+  size_t slice_stride;
   const void* bias;
   int bias_dtype;
   const int* slots;
@@ -240,6 +264,19 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   const int d = a.d, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
   const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
+  const float* part = (const float*)a.qkv + (size_t)t * row_width;
+  auto in = [&](int i) {
+    if (a.n_slices <= 1) return to_f(row[i]);
+    float x = part[i];
+    for (int s0 = 1; s0 < a.n_slices; s0 += 4) {   // four loads go out together
+      float p[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) p[u] = s0 + u < a.n_slices ? part[(size_t)(s0 + u) * a.slice_stride + i] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) x += p[u];
+    }
+    return x;
+  };
   const int slot = a.slots ? a.slots[t] : -1;
   const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
   const int col = head * d;  // q heads, k heads and v heads follow each other in the row
@@ -257,7 +294,7 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
       } else {
         i0 = 2 * p; i1 = 2 * p + 1;  // beyond the rotated part pairs are consecutive in both styles
       }
-      float x0 = to_f(row[col + i0]), x1 = to_f(row[col + i1]);
+      float x0 = in(col + i0), x1 = in(col + i1);
       if (a.bias) {
         x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
         x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
@@ -276,7 +313,7 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
     const int kh = head - a.nH - a.nKV;
     T* vc = (T*)a.v_cache + ((size_t)page * a.nKV + kh) * d * a.page_size + off;
     for (int e = threadIdx.x; e < d; e += blockDim.x) {
-      float x = to_f(row[col + e]);
+      float x = in(col + e);
       if (a.bias) x += load_dyn(a.bias, a.bias_dtype, col + e);
       vc[(size_t)e * a.page_size] = from_f<T>(x);
     }
@@ -367,9 +404,13 @@ __global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T,
   }
 }
 
+// dtype: the type of q_out and the cache, and of qkv unless n_slices > 1 (then qkv holds float partial sums,
+// slice_stride elements apart).
 extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const int* slots,
                                const float* cs, const float* sn, int rope_style, int rotary_dim, int T, int nH,
-                               int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, void* stream) {
+                               int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, int n_slices,
+                               long long slice_stride, void* stream) {
+  IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || slice_stride > 0), "rope_append: %d slices, %lld apart", n_slices, slice_stride);
   IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
   IFX_REQUIRE(rope_style >= 0 && rope_style <= 2, "rope_append: unknown rope style %d", rope_style);
   IFX_REQUIRE(rope_style == 0 || (rotary_dim > 0 && rotary_dim <= d && rotary_dim % 2 == 0 && cs && sn),
@@ -377,10 +418,11 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   IFX_REQUIRE(!slots || (page_size > 0 && k_cache && v_cache), "rope_append: cache write without cache");
   IFX_REQUIRE(nH + 2 * nKV <= 65535, "rope_append: too many heads for one launch");
   if (T == 0) return 0;
-  RopeArgs a{qkv, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size, q_out, k_cache, v_cache};
+  RopeArgs a{qkv, n_slices, (size_t)slice_stride, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size,
+             q_out, k_cache, v_cache};
   hipStream_t s = (hipStream_t)stream;
   // (a few tokens are quicker with one small block per token and head: nothing waits on a loop over tokens)
-  if (T >= 128 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
+  if (T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
       (!slots || page_size % 8 == 0)) {
     const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
     const size_t v_threads = slots ? (size_t)((T + 7) / 8) * nKV * d : 0;

@@ -155,6 +155,16 @@ __global__ void wide_sum_slices_kernel(const float* __restrict__ part, TO* __res
   out[i] = from_f<TO>(a);
 }
 
+// out [n] = part [S][n] added in slice order.
+extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S, long long n, void* stream) {
+  IFX_REQUIRE(S >= 1 && n >= 0 && (out_dtype == DT_BF16 || out_dtype == DT_F32), "sum_slices: %d slices of %lld, out dtype %d", S, n, out_dtype);
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (out_dtype == DT_BF16) hipLaunchKernelGGL(wide_sum_slices_kernel<bf16_t>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, part, (bf16_t*)out, S, (size_t)n);
+  else hipLaunchKernelGGL(wide_sum_slices_kernel<float>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, part, (float*)out, S, (size_t)n);
+  IFX_LAUNCH_CHECK();
+}
+
 // Waves per workgroup and slices of K for a shape.  ``waves`` / ``slices`` 0: chosen here (about one workgroup
 // for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
 // several workgroups to a unit; then slices of at least four rounds, at most eight); the gate/up epilogue takes
@@ -178,7 +188,7 @@ extern "C" int ifx_wide_gemm_plan(int N, int K, int waves, int slices, int epi) 
 
 template <int MT>
 static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K, int waves,
-                       int slices, int rps, int epi, const int* order, hipStream_t s) {
+                       int slices, int rps, int epi, const int* order, bool add_slices, hipStream_t s) {
   const int n_tiles = (N + 15) / 16;
   const dim3 grid((n_tiles + waves - 1) / waves, slices);
   const int k_tiles = (K + 63) / 64 * 2;
@@ -190,7 +200,7 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
   else if (epi == 0) GO(float, 0);
   else GO(float, 1);
 #undef GO
-  if (slices > 1) {
+  if (slices > 1 && add_slices) {
     const size_t n = (size_t)M * N;
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (out_dtype == DT_BF16) hipLaunchKernelGGL(wide_sum_slices_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, part, (bf16_t*)out, slices, n);
@@ -203,8 +213,11 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
 // returned them; ``part``: slices * M * N floats when there is more than one slice.
 // epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2] (one slice, no tile order).
 // order: the row-tile order the copy was written with (or null).
+// ``out`` null with more than one slice: the partial sums are left in ``part`` for a kernel that adds them itself
+// (ifx_add_rmsnorm, ifx_rope_append).
 extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K,
                              int waves, int slices, int epi, const int* order, void* stream) {
+  IFX_REQUIRE(out || slices > 1, "wide_gemm: no output");
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "wide_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "wide_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "wide_gemm: unknown out dtype %d", out_dtype);
@@ -219,9 +232,9 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
   IFX_REQUIRE((n_rounds + rps - 1) / rps == slices, "wide_gemm: %d rounds do not cut into %d slices (ask ifx_wide_gemm_plan)", n_rounds, slices);
   hipStream_t s = (hipStream_t)stream;
   switch ((M + 15) / 16) {
-    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
-    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
-    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
-    default: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, s);
+    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
+    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
+    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
+    default: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
   }
 }

@@ -123,17 +123,21 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     _check(residual, "residual", (None, None), torch.float32)
     T, H = residual.shape
     _check(weight, "weight", (H,))
-    if delta is not None:
+    n_slices = 1
+    if isinstance(delta, SliceSums):               # partial sums: the kernel adds them in slice order
+        _check(delta.parts, "delta", (None, T, H), torch.float32)
+        n_slices, delta = delta.parts.shape[0], delta.parts
+    elif delta is not None:
         _check(delta, "delta", (T, H))
     n = T
     if rows is not None:
         _check(rows, "rows", (None,), torch.int32)
         n = rows.shape[0]
     out = torch.empty((n, H), dtype=out_dtype, device=residual.device)
-    _call(load_module("core"), "ifx_add_rmsnorm", (P, P, I, P, I, P, I, P, I, I, F, I, P),
+    _call(load_module("core"), "ifx_add_rmsnorm", (P, P, I, P, I, P, I, P, I, I, F, I, I, LL, P),
           residual.data_ptr(), _ptr(delta), _dt(delta) if delta is not None else 0, weight.data_ptr(),
           _dt(weight), out.data_ptr(), _DT[out_dtype], _ptr(rows), n, H, float(eps),
-          1 if (delta is not None and rows is None) else 0, _stream())
+          1 if (delta is not None and rows is None) else 0, n_slices, T * H, _stream())
     return out
 
 
@@ -162,7 +166,13 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
     """
     T = qkv.shape[0]
     width = (n_heads + 2 * n_kv_heads) * head_dim
-    _check(qkv, "qkv", (T, width))
+    n_slices = 1
+    if isinstance(qkv, SliceSums):                  # partial sums: the kernel adds them in slice order
+        _check(qkv.parts, "qkv", (None, T, width), torch.float32)
+        n_slices, dtype, qkv = qkv.parts.shape[0], qkv.dtype, qkv.parts
+    else:
+        _check(qkv, "qkv", (T, width))
+        dtype = qkv.dtype
     if bias is not None:
         _check(bias, "bias", (width,))
     if rope_style != ROPE_NONE:
@@ -170,15 +180,16 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
         _check(sin, "sin", (T, rotary_dim // 2), torch.float32)
     if slots is not None:
         _check(slots, "slots", (T,), torch.int32)
-        _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), qkv.dtype)
-        _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, head_dim, page_size), qkv.dtype)
+        _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), dtype)
+        _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, head_dim, page_size), dtype)
     elif n_kv_heads != 0:
         raise KernelError("rope_append: keys and values given but no slots to write them to")
-    q = torch.empty((T, n_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
-    _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, P),
-          qkv.data_ptr(), _dt(qkv), _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
+    q = torch.empty((T, n_heads, head_dim), dtype=dtype, device=qkv.device)
+    _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, P),
+          qkv.data_ptr(), _DT[dtype], _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
           _ptr(cos) if rope_style != ROPE_NONE else 0, _ptr(sin) if rope_style != ROPE_NONE else 0, rope_style,
-          rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache), _ptr(v_cache), _stream())
+          rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache), _ptr(v_cache),
+          n_slices, T * width, _stream())
     return q
 
 
@@ -329,6 +340,28 @@ class ScaledRows:
         return self.rows.dtype
 
 
+class SliceSums:
+    """A product left as partial sums over slices of K: it stands for ``parts.sum(0)`` (float32 [S, M, N], added in
+    slice order).  ``add_rmsnorm`` takes it as its delta and ``rope_append`` as its q/k/v, which saves the kernel
+    that would add the slices; ``sum()`` adds them for everyone else."""
+
+    __slots__ = ("parts", "dtype")
+
+    def __init__(self, parts: torch.Tensor, dtype: torch.dtype):
+        self.parts, self.dtype = parts, dtype      # dtype: what the sum would be rounded to
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+    def sum(self, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        S, M, N = self.parts.shape
+        out = torch.empty((M, N), dtype=dtype or self.dtype, device=self.parts.device)
+        _call(load_module("gemm_wide"), "ifx_sum_slices", (P, P, I, I, LL, P),
+              self.parts.data_ptr(), out.data_ptr(), _DT[out.dtype], S, M * N, _stream())
+        return out
+
+
 def _scale_args(x):
     """(rows, the four row-factor arguments of the kernels) of a tensor or a ``ScaledRows``."""
     if isinstance(x, ScaledRows):
@@ -452,10 +485,11 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
 
 
 def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
-              slices: int = 0, swiglu_pairs: bool = False) -> torch.Tensor:
+              slices: int = 0, swiglu_pairs: bool = False, keep_slices: bool = False):
     """bfloat16 x [M <= 64, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
     of a workgroup: the product for 17-64 rows.  ``waves`` (8-16 per workgroup, one tile of 16 weight rows each)
-    and ``slices`` of K (added in a fixed order): 0 lets the kernel choose."""
+    and ``slices`` of K (added in a fixed order): 0 lets the kernel choose.  With ``keep_slices`` a product of
+    several slices comes back as ``SliceSums``."""
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     N = weight.rows.shape[0]
@@ -469,11 +503,12 @@ def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = to
     plan = mod.fn("ifx_wide_gemm_plan", (I, I, I, I, I))(N, K, waves, slices, 1 if swiglu_pairs else 0)
     n_waves, n_slices = plan // 256, plan % 256
     part = torch.empty((n_slices, M, N), dtype=torch.float32, device=x.device) if n_slices > 1 else None
-    out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
+    keep = keep_slices and n_slices > 1
+    out = None if keep else torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
     _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, P),
-          x.data_ptr(), weight.tiled.data_ptr(), out.data_ptr(), _DT[out_dtype], _ptr(part), M, N, K, n_waves, n_slices,
+          x.data_ptr(), weight.tiled.data_ptr(), _ptr(out), _DT[out_dtype], _ptr(part), M, N, K, n_waves, n_slices,
           1 if swiglu_pairs else 0, _ptr(weight.order), _stream())
-    return out
+    return SliceSums(part, out_dtype) if keep else out
 
 
 def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
@@ -498,9 +533,10 @@ def staged_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
-def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, keep_slices: bool = False):
     """x [M, K] times ``weight`` [N, K] transposed (a tensor or a ``LinearWeight``), chosen by the weight's
-    type and by M.
+    type and by M.  With ``keep_slices`` the result may be ``SliceSums`` (the caller hands it to ``add_rmsnorm`` or
+    ``rope_append``, or calls its ``sum()``).
 
     A float32 weight takes the true 32-bit kernel whatever the activation's type.  A bfloat16
     weight with bfloat16 activations takes the weight-streaming kernel for up to 64 rows and the
@@ -525,7 +561,7 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None) -> 
     if kind == "skinny":
         return skinny_gemm(x, weight, out_dtype, tiled=tiled, order=order)
     if kind == "wide":
-        return wide_gemm(x, LinearWeight(weight, tiled, order), out_dtype)
+        return wide_gemm(x, LinearWeight(weight, tiled, order), out_dtype, keep_slices=keep_slices)
     if kind == "staged":
         return staged_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:

@@ -84,7 +84,7 @@ class PagedAttention(Mixer):
     def _project_out(self, out, sink):
         if sink is not None and ops.adds_into_stream(out.shape[0], self.w_o, sink.norm_weight):
             return ops.linear_into_stream(out, self.w_o, sink.stream, sink.norm_weight, sink.eps)
-        return ops.linear(out, self.w_o)
+        return ops.linear(out, self.w_o, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself
 
     def forward(self, h, ctx, binding: MixerBinding, sink=None):
         cache = binding.cache
@@ -104,7 +104,7 @@ class PagedAttention(Mixer):
             q = ops.qkv_rope_append(h, w, b, slots, cos, sin, nH, nKV, d, cache.k if slots is not None else None,
                                     cache.v if slots is not None else None, cache.page_size)
             return self._project_out(paged_attention(q, cache, ctx, self.window, self.scale), sink)
-        qkv = ops.linear(h, w)
+        qkv = ops.linear(h, w, keep_slices=not self.position.needs_apply)     # the rotary kernel adds partial sums itself
         if self.position.needs_apply:
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
         q = ops.rope_append(qkv, b, slots, cos, sin, style, rotary_dim, nH, nKV, d,

@@ -25,9 +25,12 @@ A norm's kernel can be saved for steps of few rows, where a launch costs as much
 optional for every part; one that declares nothing is run as above.
 
   norm      ``rms_params()`` -> (weight, eps) if the norm is x * rsqrt(mean(x^2) + eps) * weight, else None.
+            Such a norm's forward also takes ``SliceSums`` (a product left as partial sums; kernels/ops.py) for
+            its delta, as ``ops.add_rmsnorm`` does.
   mixer,    ``adds_to_stream`` True: forward takes ``sink=StreamSink(stream, weight, eps)`` (or None) and may
   ffn       then add its result to the stream itself and return ``ScaledRows`` (the rows the norm that follows
-            would give, up to a factor per row; kernels/ops.py) instead of a delta.
+            would give, up to a factor per row; kernels/ops.py) instead of a delta, or return its delta as
+            ``SliceSums``.
             ``accepts_scaled_rows(n_rows)`` True: forward takes ``ScaledRows`` for h.
   block     ``entry_norm()`` -> the norm that first reads the stream, if ``pending`` may be ``ScaledRows`` made
             for it; forward then takes ``following=`` the next block's entry norm (or None).

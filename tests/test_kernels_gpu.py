@@ -573,6 +573,55 @@ def test_wide_gemm_gate_up_pairs_and_tile_order():
     assert torch.equal(ops.wide_gemm(x.to(DEV), lq, F32, waves=3).cpu().double(), out)    # fewer than 8 waves: taken as 8
 
 
+def test_partial_sums_of_a_product_are_added_by_the_kernel_that_reads_them():
+    """A product cut into slices of K may leave its partial sums to the norm or the rotary kernel that follows."""
+    g = gen(43)
+    M, H, K, eps = 23, 200, 1096, 1e-5
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = (torch.randn(H, K, generator=g) * 0.1).to(BF16)
+    lw = ops.prepare_linear(w.to(DEV))
+    sums = ops.wide_gemm(x.to(DEV), lw, BF16, slices=4, keep_slices=True)
+    assert isinstance(sums, ops.SliceSums) and sums.parts.shape == (3, M, H) and sums.shape == (M, H)   # 9 rounds: 3 slices of 3
+    prod = x.double() @ w.double().t()
+    assert torch.allclose(sums.sum(F32).cpu().double(), prod, rtol=1e-4, atol=3e-3)
+    assert torch.equal(sums.sum(), ops.wide_gemm(x.to(DEV), lw, BF16, slices=4))
+    one = ops.wide_gemm(x.to(DEV), lw, BF16, slices=1, keep_slices=True)
+    assert torch.is_tensor(one)                                                       # a single slice is a plain result
+    # as the delta of a norm
+    res = torch.randn(M, H, generator=g)
+    nw = (1 + 0.3 * torch.randn(H, generator=g)).to(BF16)
+    r = res.to(DEV)
+    out = ops.add_rmsnorm(r, sums, nw.to(DEV), eps, BF16)
+    want_res = res.double() + prod
+    assert torch.allclose(r.cpu().double(), want_res, rtol=1e-5, atol=2e-3)
+    assert torch.allclose(out.cpu().double(), pm.rms_norm(want_res, nw.double(), eps), **tol(BF16))
+    rows = torch.tensor([22, 0, 7], dtype=torch.int32)
+    r2 = res.to(DEV)
+    out2 = ops.add_rmsnorm(r2, sums, nw.to(DEV), eps, BF16, rows.to(DEV))               # gathered rows: stream untouched
+    assert torch.equal(r2.cpu(), res)
+    assert torch.allclose(out2.cpu().double(), pm.rms_norm(want_res, nw.double(), eps)[rows.long()], **tol(BF16))
+    # as the q/k/v of the rotary kernel
+    nH, nKV, d, P = 3, 1, 40, 16                                                      # 5 heads of 40 = 200 columns
+    bias = torch.randn(H, generator=g).to(BF16)
+    cos, sin = ops.rope_table(torch.arange(M, dtype=torch.int32, device=DEV) + 5, (1.0 / 10000 ** (torch.arange(d // 2) * 2.0 / d)).to(DEV))
+    slots = torch.arange(M, dtype=torch.int32, device=DEV) + 3
+
+    def run(qkv):
+        kc, vc = torch.zeros(2, nKV, P, d, dtype=BF16, device=DEV), torch.zeros(2, nKV, d, P, dtype=BF16, device=DEV)
+        q = ops.rope_append(qkv, bias.to(DEV), slots, cos, sin, ops.ROPE_SPLIT_HALF, d, nH, nKV, d, kc, vc, P)
+        return q.float().cpu(), kc.float().cpu(), vc.float().cpu()
+
+    got, ref = run(sums), run(sums.sum(F32).to(BF16))                                   # the second rounds the sums first
+    for a, b in zip(got, ref):
+        assert torch.allclose(a, b, rtol=2e-2, atol=3e-2)
+    qkv = prod + bias.double()
+    c, sn = cos.cpu().double(), sin.cpu().double()
+    qq = qkv[:, : nH * d].reshape(M, nH, d)
+    lo, hi = qq[..., : d // 2], qq[..., d // 2:]
+    want_q = torch.cat([lo * c[:, None] - hi * sn[:, None], lo * sn[:, None] + hi * c[:, None]], -1)
+    assert torch.allclose(got[0].double(), want_q, **tol(BF16))
+
+
 def test_linear_weight_uses_the_copy_for_few_rows_and_the_rows_beyond():
     g = gen(17)
     w = torch.randn(200, 136, generator=g).to(BF16).to(DEV)
