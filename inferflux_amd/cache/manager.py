@@ -131,6 +131,10 @@ class CacheManager:
         except KeyError:
             raise KeyError(f"request {rid!r} is not live") from None
 
+    def peek(self, rid: Hashable) -> Optional[RequestPages]:
+        """The live request's record, or None."""
+        return self._requests.get(rid)
+
     def length(self, rid: Hashable) -> int:
         return self.get(rid).length
 

@@ -100,6 +100,14 @@ class StepContext:
         if upload:
             self.bind(slab, pinned)
 
+    def set_tokens(self, entries: Sequence[StepEntry], tokens: Sequence[int]) -> None:
+        """For a context built ahead of its tokens (one placeholder token per request): the step's entries and
+        their tokens, before ``bind``."""
+        if len(tokens) != self.n_tokens or len(entries) != self.n_requests:
+            raise ValueError("set_tokens: not the step this context was built for")
+        self.entries = list(entries)
+        self.h_token_ids[:] = tokens
+
     def bind(self, slab: torch.Tensor = None, pinned: torch.Tensor = None) -> None:
         """Put the step's arrays on the device: into ``slab`` through ``pinned`` when given (an
         asynchronous copy on the current stream), else into a new tensor."""

@@ -131,7 +131,14 @@ class Engine:
         entries = [StepEntry(i.seq.rid, i.tokens, [len(i.tokens) - 1] if i.wants_logits else []) for i in plan.items]
         logits = self.runner.step(entries)
         wanting = [i for i in plan.items if i.wants_logits]
-        tokens = self.sampler.sample(logits, [self._live[i.seq.rid].sampling for i in wanting]) if wanting else []
+        ahead = None
+        if len(wanting) == len(plan.items) and not self.scheduler.waiting and all(len(i.tokens) == 1 for i in plan.items):
+            # A step of decoding with nobody waiting: the next step is most likely the same requests, one token
+            # further, less those that reach their limit now.  While the GPU works on this one, the runner gets
+            # ready what of the next does not depend on its tokens; if the guess is wrong it is dropped.
+            rids = [i.seq.rid for i in plan.items if len(i.seq.generated) + 1 < self._live[i.seq.rid].params.max_tokens]
+            ahead = lambda: self.runner.prepare_decode(rids)
+        tokens = self.sampler.sample(logits, [self._live[i.seq.rid].sampling for i in wanting], ahead) if wanting else []
         dt = (time.perf_counter() - t0) * 1e3
         if any(len(i.tokens) > 1 or i.seq.is_prefilling for i in plan.items):
             self.stats.prefill_ms += dt

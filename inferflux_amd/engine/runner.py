@@ -65,6 +65,7 @@ class ModelRunner:
             self.timer = PhaseTimer()
         self.decode_graphs = decode_graphs and model.graph_safe and self.timer is None
         self._graphs = {}
+        self._prepared = None      # (requests, their lengths, the context) of a step got ready ahead of its tokens
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, rid: Hashable) -> None:
@@ -101,10 +102,53 @@ class ModelRunner:
             if badw:
                 raise StepError(f"request {e.rid!r}: wanted places {badw[:8]} outside its {n} tokens")
 
+    def prepare_decode(self, rids: Sequence[Hashable]) -> bool:
+        """Get ready, while the GPU still works on the last step, everything that does not depend on the tokens of
+        a step in which each of ``rids`` brings one token and wants its logits: checks, pages, the step's arrays.
+        ``step`` uses it if that is the step it is given, and drops it otherwise (pages taken early stay with their
+        request and are used or freed with it).  Returns False, having changed nothing, when it cannot (no graphs,
+        a request at its last position, not enough pages)."""
+        self._prepared = None
+        rids = list(rids)
+        if not self.decode_graphs or not rids or len(set(rids)) != len(rids):
+            return False
+        if not all(self.manager.has(r) and self.manager.length(r) + 1 <= self.max_position for r in rids):
+            return False
+        needs = [(r, 1) for r in rids]
+        if not self.manager.can_reserve(needs):
+            return False
+        for r in rids:
+            self.manager.reserve(r, 1)
+        ctx = StepContext([StepEntry(r, [0], [0]) for r in rids], self.manager, self.dtype, self.device,
+                          width_multiple=self.GRAPH_WIDTH_MULTIPLE, upload=False)
+        self._prepared = ([self.manager.get(r) for r in rids], [self.manager.length(r) for r in rids], ctx)
+        return True
+
+    def _take_prepared(self, entries):
+        """The context ``prepare_decode`` built, if ``entries`` are the step it was built for (the same live
+        requests, none of which has moved since), with their tokens put in; else None."""
+        prep, self._prepared = self._prepared, None
+        if prep is None or len(prep[0]) != len(entries):
+            return None
+        for e, pages, length in zip(entries, *prep[:2]):
+            if len(e.tokens) != 1 or list(e.want) != [0] or self.manager.peek(e.rid) is not pages or pages.length != length:
+                return None
+        tokens = [int(e.tokens[0]) for e in entries]
+        if min(tokens) < 0 or max(tokens) >= self.vocab_size:
+            return None                      # the full check names the culprit
+        prep[2].set_tokens(entries, tokens)
+        return prep[2]
+
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         entries = list(entries)
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        ctx = self._take_prepared(entries) if self._prepared is not None else None
+        if ctx is not None:
+            logits = self._decode_step(entries, ctx)
+            for e in entries:
+                self.manager.commit(e.rid, 1)
+            return logits
         self.validate(entries)
         needs = [(e.rid, len(e.tokens)) for e in entries]
         if not self.manager.can_reserve(needs):
@@ -126,12 +170,13 @@ class ModelRunner:
             self.manager.commit(rid, n)
         return logits
 
-    def _decode_step(self, entries) -> torch.Tensor:
+    def _decode_step(self, entries, ctx=None) -> torch.Tensor:
         """A step of single tokens through a captured graph.  The first step of a layout runs as usual
         and is then captured; later steps copy their arrays into the graph's buffer and replay it.
         The logits returned by a replay live in the graph's memory: they are valid until the next step."""
-        ctx = StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
-                          upload=False)
+        if ctx is None:
+            ctx = StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
+                              upload=False)
         g = self._graphs.get(ctx.layout_key)
         if g is not None:
             g.copied.synchronize()          # the host buffer is free again once the last copy out of it is done

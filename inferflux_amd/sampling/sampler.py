@@ -55,10 +55,11 @@ class Sampler:
     def _dev(self, values, dtype):
         return torch.tensor(values, dtype=dtype, device=self.device)
 
-    def sample(self, logits: torch.Tensor, states: Sequence[SamplingState]) -> List[int]:
+    def sample(self, logits: torch.Tensor, states: Sequence[SamplingState], while_waiting=None) -> List[int]:
         """One token per row of float32 ``logits`` [R, V]; row i belongs to ``states[i]``.  The
         logits are modified in place by penalties and bias.  States are advanced (draw counter,
-        history)."""
+        history).  ``while_waiting`` is called once the kernels are launched, before their results are
+        waited for: host work that needs no token goes there."""
         R = logits.shape[0]
         if R != len(states):
             raise ValueError(f"{R} rows of logits for {len(states)} requests")
@@ -93,7 +94,11 @@ class Sampler:
                                 torch.from_numpy(u).to(self.device))
         top_n = max((s.params.logprobs for s in states if s.params.logprobs is not None), default=None)
         if top_n is not None:
-            lp, top_ids, top_lp = (t.cpu() for t in ops.logprobs(logits, chosen, top_n))
+            lp_dev = ops.logprobs(logits, chosen, top_n)
+        if while_waiting is not None:
+            while_waiting()
+        if top_n is not None:
+            lp, top_ids, top_lp = (t.cpu() for t in lp_dev)
         tokens = chosen.cpu().tolist()
         for r, (st, t) in enumerate(zip(states, tokens)):
             if st.params.logprobs is not None:

@@ -287,6 +287,60 @@ def test_steps_of_few_rows_need_no_kernel_for_the_norms_between_products(name, s
     assert rel_err(fused, separate) < REL_TOL["bfloat16"]
 
 
+def test_a_decode_step_got_ready_ahead_of_its_tokens(sharp_folders):
+    """prepare_decode does, before the tokens are known, what a step of single tokens needs besides them; step uses
+    it for exactly that step and falls back to the ordinary path for any other, with the same logits either way."""
+    folder, V = sharp_folders["C", "float32"], TINY["C"]["vocab_size"]
+    ids = {r: seeded_ids(40 + i, 70, V) for i, r in enumerate("abc")}
+
+    def run(prepare):
+        runner = load_runner(folder, torch.float32, num_pages=24)
+        out, used = [], 0
+        for r in "abc":
+            runner.add_request(r)
+            runner.step([StepEntry(r, ids[r][:30], [])])
+        order = ["abc", "abc", "abc", "acb", "ab", "ab", "abc", "abc"]       # same step, same, same, other order, fewer, ...
+        at = {r: 30 for r in "abc"}
+        for k, who in enumerate(order):
+            if prepare and k > 0:
+                assert runner.prepare_decode(list(order[k - 1])) is True    # the guess: the last step's requests again
+            entries = [StepEntry(r, [ids[r][at[r]]], [0]) for r in who]
+            was = runner._prepared is not None
+            out.append(runner.step(entries).cpu())
+            used += int(was and who == order[k - 1])
+            assert runner._prepared is None
+            for r in who:
+                at[r] += 1
+            runner.manager.check()
+        if prepare:                                                        # got ready for "b" alone, given two tokens of "b"
+            runner.prepare_decode(["b"])
+            out.append(runner.step([StepEntry("b", ids["b"][at["b"]:at["b"] + 2], [0, 1])]).cpu())
+        else:
+            out.append(runner.step([StepEntry("b", ids["b"][at["b"]:at["b"] + 2], [0, 1])]).cpu())
+        for r in "abc":
+            runner.free_request(r)
+        runner.manager.check()
+        assert runner.manager.free_pages() == [24] * len(runner.manager.groups)
+        return out, used
+
+    plain, _ = run(False)
+    ahead, used = run(True)
+    assert used == 4
+    for a, b in zip(plain, ahead):
+        assert torch.equal(a, b)
+    want = plain_logits(folder, ids["a"][:38])
+    assert rel_err(torch.stack([o[0] for o in plain[:8]]), want[30:38]) < REL_TOL["float32"]
+    # what it cannot get ready it leaves alone: a request that is not live, one named twice, no pages left
+    runner = load_runner(folder, torch.float32, num_pages=2)
+    runner.add_request("x")
+    runner.step([StepEntry("x", ids["a"][:32], [])])                       # both pages of both groups are full
+    free = runner.manager.free_pages()
+    assert runner.prepare_decode(["x"]) is False and runner.prepare_decode(["x", "x"]) is False
+    assert runner.prepare_decode(["nobody"]) is False and runner.manager.free_pages() == free
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("x", [5], [0])])
+
+
 # ---- captured decode steps ----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C"])

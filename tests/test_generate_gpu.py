@@ -42,6 +42,39 @@ def test_greedy_generation_equals_the_plain_model(name, model_folders):
     assert st.generated_tokens == n_new * len(prompts) and st.prompt_tokens == sum(lens)
 
 
+def test_steps_got_ready_ahead_change_no_token_and_are_used(model_folders, monkeypatch):
+    """While the GPU decodes, the engine gets the next decode step ready on a guess (the same requests, less those at
+    their limit).  A stop token makes the guess wrong once; tokens are the same with and without the guessing."""
+    from inferflux_amd.engine.runner import ModelRunner
+    folder = model_folders["B"]
+    prompts = [seeded_ids(80 + i, n, TINY["B"]["vocab_size"]) for i, n in enumerate([5, 40, 23])]
+    limits = (6, 30, 17)
+
+    def run(stop):
+        params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True, stop_token_ids=stop if i == 1 else ())
+                  for i, n in enumerate(limits)]
+        return Engine.load(folder, dtype="bfloat16", kv_pages=64, max_batch_size=4).generate(prompts, params)
+
+    taken = []
+    real, real_prepare = ModelRunner._take_prepared, ModelRunner.prepare_decode
+    monkeypatch.setattr(ModelRunner, "_take_prepared", lambda self, e: _count(taken, real(self, e)))
+    with_it = run(())
+    assert [len(o.token_ids) for o in with_it] == list(limits)
+    assert sum(taken) >= 20 and all(taken)                 # requests that reach their limit are foreseen
+    stop = [with_it[1].token_ids[12]]
+    del taken[:]
+    stopped = run(stop)
+    assert stopped[1].finish_reason == "stop" and len(stopped[1].token_ids) <= 13 and not all(taken)
+    monkeypatch.setattr(ModelRunner, "prepare_decode", lambda self, rids: False)
+    assert [o.token_ids for o in run(())] == [o.token_ids for o in with_it]
+    assert [o.token_ids for o in run(stop)] == [o.token_ids for o in stopped]
+
+
+def _count(taken, ctx):
+    taken.append(ctx is not None)
+    return ctx
+
+
 def test_preemption_by_recomputation_changes_no_token(model_folders):
     folder = model_folders["A"]
     prompts = [seeded_ids(70 + i, 40, 512) for i in range(3)]
