@@ -115,9 +115,7 @@ class StepContext:
             host = pinned.numpy()
         else:
             host = np.zeros(self.slab_size, dtype=np.int32)
-        for name, a in self._named:
-            o, n, _ = self._offs[name]
-            host[o:o + n] = a.reshape(-1)
+        self.write_host(host)
         if slab is None:
             slab = torch.from_numpy(host).to(self.device)
         elif pinned is not None:
@@ -125,6 +123,12 @@ class StepContext:
         else:
             slab.copy_(torch.from_numpy(host))
         self.use_slab(slab)
+
+    def write_host(self, host: np.ndarray) -> None:
+        """The step's arrays, end to end, into ``host`` (int32, at least ``slab_size`` long)."""
+        for name, a in self._named:
+            o, n, _ = self._offs[name]
+            host[o:o + n] = a.reshape(-1)
 
     def use_slab(self, slab: torch.Tensor) -> None:
         """Take ``slab`` (which already holds a step of this layout) as the device arrays."""

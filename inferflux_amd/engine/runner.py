@@ -34,6 +34,7 @@ class _DecodeGraph:
 
     def __init__(self, slab, pinned, graph, ctx, logits):
         self.slab, self.pinned, self.graph, self.ctx, self.logits = slab, pinned, graph, ctx, logits
+        self.host = pinned.numpy()      # the pinned buffer as the array the step's arrays are written into
         self.copied = torch.cuda.Event()
 
 
@@ -180,7 +181,8 @@ class ModelRunner:
         g = self._graphs.get(ctx.layout_key)
         if g is not None:
             g.copied.synchronize()          # the host buffer is free again once the last copy out of it is done
-            ctx.bind(g.slab, g.pinned)
+            ctx.write_host(g.host)          # (the replay reads the graph's own views of the slab: none are made here)
+            g.slab.copy_(g.pinned, non_blocking=True)
             g.copied.record()
             g.graph.replay()
             return g.logits

@@ -163,9 +163,10 @@ class Scheduler:
         cfg = self.config
         plan = StepPlan([], [], [])
         budget = cfg.max_batch_tokens
-        # 1. running requests, oldest admission first: decodes cost one token, prompts a portion
-        for seq in sorted(self.running, key=lambda s: s.admitted_at):
-            if seq not in self.running or budget <= 0:      # preempted meanwhile / nothing left to deal
+        # 1. running requests, oldest admission first (the list is kept in that order: admissions are appended,
+        #    preemptions taken out): decodes cost one token, prompts a portion
+        for seq in list(self.running):
+            if budget <= 0 or (plan.preempted and seq not in self.running):   # nothing left to deal / preempted meanwhile
                 continue
             if seq.is_prefilling:
                 n = min(len(seq.prompt) - seq.computed, cfg.chunked_prefill_tokens, budget)
