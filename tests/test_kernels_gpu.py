@@ -523,7 +523,7 @@ def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, 
     assert torch.allclose(qq.float(), q.float(), rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("M", [17, 32, 33, 50, 64])
+@pytest.mark.parametrize("M", [9, 17, 32, 33, 50, 64])
 @pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136)])
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
 def test_wide_gemm(M, N, K, out_dtype):
@@ -535,7 +535,8 @@ def test_wide_gemm(M, N, K, out_dtype):
     t = dict(rtol=1e-4, atol=3e-3) if out_dtype == F32 else dict(rtol=1e-2, atol=0.1)
     got = ops.wide_gemm(x.to(DEV), lw, out_dtype).cpu().double()
     assert got.shape == (M, N) and torch.allclose(got, want, **t), float((got - want).abs().max())
-    assert torch.equal(ops.linear(x.to(DEV), lw, out_dtype).cpu().double(), got)       # what linear picks at these rows
+    if M > 16:
+        assert torch.equal(ops.linear(x.to(DEV), lw, out_dtype).cpu().double(), got)   # what linear picks at these rows
 
 
 @pytest.mark.parametrize("waves,slices", [(8, 1), (8, 3), (11, 2), (16, 1), (16, 8)])
