@@ -58,10 +58,13 @@ def attention_rows(args) -> None:
     dev, B, kv, nH, nKV, d, P = "cuda", args.batch, args.context, args.heads, args.kv_heads, args.head_dim, args.page_size
     nb = -(-kv // P)
     # enough caches to rotate through that no launch finds its keys and values in the last-level cache
-    copies = max(2, min(16, int(2e9 // (2 * B * nb * nKV * P * d * 2))))
-    caches = [(torch.randn(B * nb, nKV, P, d, device=dev, dtype=torch.bfloat16),
-               torch.randn(B * nb, nKV, d, P, device=dev, dtype=torch.bfloat16)) for _ in range(copies)]
-    table = torch.randperm(B * nb, device=dev).to(torch.int32).view(B, nb).contiguous()
+    copies = max(2, int(args.rotate_gb * 1e9 // (2 * B * nb * nKV * P * d * 2)))
+    k0 = torch.randn(B * nb, nKV, P, d, device=dev, dtype=torch.bfloat16)
+    v0 = torch.randn(B * nb, nKV, d, P, device=dev, dtype=torch.bfloat16)
+    caches = [(k0, v0)] + [(k0.clone(), v0.clone()) for _ in range(copies - 1)]
+    # where a request's pages lie: anywhere, or one after the other as a pool hands them to a prompt that comes in whole
+    order = torch.arange(B * nb, device=dev) if args.pages == "in-order" else torch.randperm(B * nb, device=dev)
+    table = order.to(torch.int32).view(B, nb).contiguous()
     q = torch.randn(B, nH, d, device=dev, dtype=torch.bfloat16)
     out = torch.empty(B, nH * d, device=dev, dtype=torch.bfloat16)
     row_req = torch.arange(B, dtype=torch.int32, device=dev)
@@ -109,6 +112,9 @@ def main(argv=None) -> int:
             p.add_argument("--batch", type=int, default=8)
             p.add_argument("--context", type=int, default=3072)
             p.add_argument("--chunk", type=int, default=0, help="keys per split (0: 128, 256, 512 and 1024)")
+            p.add_argument("--rotate-gb", type=float, default=2.0,
+                           help="memory the launches rotate through (a model's step touches tens of GB between two uses of a cache)")
+            p.add_argument("--pages", choices=["shuffled", "in-order"], default="shuffled", help="how a request's pages lie in the pool")
         if name == "gemm":
             p.add_argument("--rows", type=int, default=8, help="rows of x")
             p.add_argument("--shape", choices=list(GEMM_SHAPES), default=None)
