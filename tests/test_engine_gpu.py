@@ -341,6 +341,23 @@ def test_a_decode_step_got_ready_ahead_of_its_tokens(sharp_folders):
         runner.step([StepEntry("x", [5], [0])])
 
 
+@pytest.mark.parametrize("copy", [True, False])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_portions_of_every_product_size_with_and_without_the_decode_copy(name, copy, sharp_folders):
+    """Portions of 1-16, 17-64 and more rows take different matrix-product kernels in bfloat16, and other ones again
+    when the weights have no tiled copy; all of them follow the plain model."""
+    folder, V = sharp_folders[name, "bfloat16"], TINY[name]["vocab_size"]
+    runner = load_runner(folder, torch.bfloat16, num_pages=24, decode_weight_copy=copy)
+    ids = seeded_ids(33, 212, V)
+    want = plain_logits(folder, ids)
+    runner.add_request("p")
+    got, at = [], 0
+    for m in (40, 17, 3, 64, 1, 16, 70, 1):
+        got.append(runner.step([StepEntry("p", ids[at:at + m], list(range(m)))]).cpu()); at += m
+    assert at == 212 and rel_err(torch.cat(got), want) < REL_TOL["bfloat16"]
+    runner.free_request("p")
+
+
 # ---- captured decode steps ----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C"])
