@@ -41,40 +41,23 @@ class StepContext:
         self.timer = None              # a tracing.PhaseTimer while per-phase timing is on
         self.entries = list(entries)
         R = self.n_requests = len(self.entries)
-        P = manager.page_size
-        q_len = np.array([len(e.tokens) for e in self.entries], dtype=np.int32)
-        start = np.array([manager.length(e.rid) for e in self.entries], dtype=np.int32)
-        q_start = np.zeros(R, dtype=np.int32)
-        if R > 1:
-            q_start[1:] = np.cumsum(q_len)[:-1]
-        T = self.n_tokens = int(q_len.sum())
+        # lengths, positions, block tables and write slots come from the cache manager's native side in one call
+        arrays = manager.step_arrays([e.rid for e in self.entries], [len(e.tokens) for e in self.entries], width_multiple)
+        q_len, q_start, start = arrays["q_len"], arrays["q_start"], arrays["start"]
+        T = self.n_tokens = int(arrays["positions"].shape[0])
         self.h_q_len, self.h_q_start, self.h_start_pos = q_len, q_start, start
-        self.h_kv_len = start + q_len
+        self.h_kv_len = arrays["kv_len"]
         self.h_token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in self.entries]) if R else np.zeros(0, np.int32)
-        self.h_row_req = np.repeat(np.arange(R, dtype=np.int32), q_len)
-        self.h_positions = (np.arange(T, dtype=np.int32) - np.repeat(q_start, q_len) + np.repeat(start, q_len)).astype(np.int32)
+        self.h_row_req, self.h_positions = arrays["row_req"], arrays["positions"]
         rows: List[int] = []
         for i, e in enumerate(self.entries):
             rows.extend(int(q_start[i]) + int(w) for w in e.want)
         self.h_logit_rows = np.asarray(rows, dtype=np.int32)
         self.n_logit_rows = len(rows)
-        self.h_state_slots = np.array([manager.state_slot(e.rid) for e in self.entries], dtype=np.int32)
-
+        self.h_state_slots = arrays["state_slots"]
         n_groups = len(manager.groups)
-        self.h_block_tables: List[np.ndarray] = []
-        self.h_write_slots: List[np.ndarray] = []
-        for g in range(n_groups):
-            tables = [manager.block_table(e.rid, g) for e in self.entries]
-            width = max(width_multiple, -(-max((len(t) for t in tables), default=1) // width_multiple) * width_multiple)
-            bt = np.full((R, width), -1, dtype=np.int32)
-            for i, t in enumerate(tables):
-                bt[i, :len(t)] = t
-            self.h_block_tables.append(bt)
-            blk = self.h_positions // P
-            pages = bt[self.h_row_req, blk] if T else np.zeros(0, np.int32)
-            if T and (pages < 0).any():
-                raise RuntimeError(f"cache group {g}: a row of this step has no page (reserve before building the step)")
-            self.h_write_slots.append((pages * P + self.h_positions % P).astype(np.int32))
+        self.h_block_tables: List[np.ndarray] = arrays["block_tables"]
+        self.h_write_slots: List[np.ndarray] = arrays["write_slots"]
 
         # One upload: every array above, end to end, each start aligned to 4 ints.
         named = [("token_ids", self.h_token_ids), ("positions", self.h_positions), ("row_req", self.h_row_req),
@@ -91,7 +74,7 @@ class StepContext:
         # No request of this step holds more positions than its block table has room for.  Kernels size
         # their grids by this bound, not by the lengths themselves, so that a captured step stays valid
         # while lengths grow within the same table width.
-        self.kv_bound = max((bt.shape[1] for bt in self.h_block_tables), default=0) * P
+        self.kv_bound = max((bt.shape[1] for bt in self.h_block_tables), default=0) * manager.page_size
         self.slab_size = max(total, 4)
         self._named, self._offs = named, offs
         self._views: Dict[str, torch.Tensor] = {}

@@ -66,7 +66,7 @@ class ModelRunner:
             self.timer = PhaseTimer()
         self.decode_graphs = decode_graphs and model.graph_safe and self.timer is None
         self._graphs = {}
-        self._prepared = None      # (requests, their lengths, the context) of a step got ready ahead of its tokens
+        self._prepared = None      # (the manager's snapshot of the requests, the context) of a step got ready ahead of its tokens
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, rid: Hashable) -> None:
@@ -122,23 +122,22 @@ class ModelRunner:
             self.manager.reserve(r, 1)
         ctx = StepContext([StepEntry(r, [0], [0]) for r in rids], self.manager, self.dtype, self.device,
                           width_multiple=self.GRAPH_WIDTH_MULTIPLE, upload=False)
-        self._prepared = ([self.manager.get(r) for r in rids], [self.manager.length(r) for r in rids], ctx)
+        self._prepared = (self.manager.snapshot(rids), ctx)
         return True
 
     def _take_prepared(self, entries):
         """The context ``prepare_decode`` built, if ``entries`` are the step it was built for (the same live
         requests, none of which has moved since), with their tokens put in; else None."""
         prep, self._prepared = self._prepared, None
-        if prep is None or len(prep[0]) != len(entries):
+        if prep is None or any(len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0 for e in entries):
             return None
-        for e, pages, length in zip(entries, *prep[:2]):
-            if len(e.tokens) != 1 or list(e.want) != [0] or self.manager.peek(e.rid) is not pages or pages.length != length:
-                return None
+        if not self.manager.unchanged(prep[0], [e.rid for e in entries]):
+            return None
         tokens = [int(e.tokens[0]) for e in entries]
         if min(tokens) < 0 or max(tokens) >= self.vocab_size:
             return None                      # the full check names the culprit
-        prep[2].set_tokens(entries, tokens)
-        return prep[2]
+        prep[1].set_tokens(entries, tokens)
+        return prep[1]
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         entries = list(entries)
@@ -147,8 +146,7 @@ class ModelRunner:
         ctx = self._take_prepared(entries) if self._prepared is not None else None
         if ctx is not None:
             logits = self._decode_step(entries, ctx)
-            for e in entries:
-                self.manager.commit(e.rid, 1)
+            self.manager.commit_each([e.rid for e in entries], 1)
             return logits
         self.validate(entries)
         needs = [(e.rid, len(e.tokens)) for e in entries]

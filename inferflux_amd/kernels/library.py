@@ -1,6 +1,7 @@
-"""Builds and loads the HIP kernel modules.
+"""Builds and loads the native modules: the HIP kernels and the host-side C++ runtime pieces.
 
-Each ``csrc/<name>.hip`` is compiled by hipcc for gfx950 into one shared library
+Each ``csrc/<name>.hip`` is compiled by hipcc for gfx950 (each ``csrc/<name>.cpp``, which is host code
+only, by the C++ compiler) into one shared library
 ``<name>[-variant].<hash>.so`` and loaded through ctypes.  The hash covers the source, the
 shared header, the flags and the variant's defines, so a library on disk always matches the
 source beside it: a stale one is simply not found and the module is compiled again.  A module
@@ -33,6 +34,8 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
 
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
+
 Variant = Tuple[Tuple[str, int], ...]
 
 
@@ -51,12 +54,24 @@ def _variant_tag(variant: Variant) -> str:
     return "".join(f"-{k.lower()}{v}" for k, v in variant)
 
 
+def _is_host_module(name: str) -> bool:
+    return os.path.isfile(os.path.join(CSRC, f"{name}.cpp"))
+
+
+def _cxx() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")):
+        if cand and (os.path.isfile(cand) or shutil.which(cand)):
+            return cand
+    return _hipcc()          # hipcc compiles plain C++ too
+
+
 def _digest(name: str, variant: Variant) -> str:
     h = hashlib.sha256()
-    for fn in (f"{name}.hip", "common.h"):
+    host = _is_host_module(name)
+    for fn in ((f"{name}.cpp",) if host else (f"{name}.hip", "common.h")):
         with open(os.path.join(CSRC, fn), "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(HOST_FLAGS if host else FLAGS).encode())
     h.update(repr(variant).encode())
     return h.hexdigest()[:12]
 
@@ -90,7 +105,8 @@ def compile_module(name: str, variant: Variant = (), force: bool = False) -> str
         hit = find_library(name, variant)
         if hit:
             return hit
-    src = os.path.join(CSRC, f"{name}.hip")
+    host = _is_host_module(name)
+    src = os.path.join(CSRC, f"{name}.cpp" if host else f"{name}.hip")
     if not os.path.isfile(src):
         raise KernelBuildError(f"no kernel source {src}")
     out_dir = CSRC if os.access(CSRC, os.W_OK) else _fallback_dir()
@@ -103,9 +119,10 @@ def compile_module(name: str, variant: Variant = (), force: bool = False) -> str
             if not force and os.path.isfile(out):
                 return out
             tmp = f"{out}.{os.getpid()}.tmp"
-            cmd = [_hipcc(), *FLAGS, *[f"-D{k}={v}" for k, v in variant], src, "-o", tmp]
+            defines = [f"-D{k}={v}" for k, v in variant]
+            cmd = [_cxx(), *HOST_FLAGS, *defines, src, "-o", tmp] if host else [_hipcc(), *FLAGS, *defines, src, "-o", tmp]
             label = f"{name}{_variant_tag(variant)}"
-            _progress(f"compiling {label} for {ARCH} ...")
+            _progress(f"compiling {label} for {'the host' if host else ARCH} ...")
             t0 = time.time()
             proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=out_dir)
             done = threading.Event()
@@ -121,7 +138,7 @@ def compile_module(name: str, variant: Variant = (), force: bool = False) -> str
             if proc.returncode != 0 or not os.path.isfile(tmp):
                 if os.path.exists(tmp):
                     os.unlink(tmp)
-                raise KernelBuildError(f"hipcc failed for {label} (exit {proc.returncode}):\n{' '.join(cmd)}\n{log}")
+                raise KernelBuildError(f"{os.path.basename(cmd[0])} failed for {label} (exit {proc.returncode}):\n{' '.join(cmd)}\n{log}")
             os.replace(tmp, out)
             # Drop libraries of the same module built from older sources.
             prefix = f"{name}{_variant_tag(variant)}."

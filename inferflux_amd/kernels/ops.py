@@ -40,6 +40,7 @@ class KernelError(RuntimeError):
 
 
 def module_variants() -> Iterable[Tuple[str, Variant]]:
+    yield ("cache_manager", ())       # host code: the cache's bookkeeping
     yield ("core", ())
     yield ("gemm_f32", ())
     yield ("attn_plain", ())

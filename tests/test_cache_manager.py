@@ -121,3 +121,120 @@ def test_random_orders_never_lose_or_double_book_a_page(seed):
         m.free(rid)
     m.check()
     assert m.free_pages() == [10, 10]
+
+
+# ---- the native manager against the plain one, operation by operation ------------------------------------
+def _both(pages, window, slots, page_size=16):
+    import plain_cache_manager as plain
+    groups = [GroupSpec(None, (0,)), GroupSpec(window, (1, 2))]
+    pgroups = [plain.GroupSpec(None, (0,)), plain.GroupSpec(window, (1, 2))]
+    return CacheManager(groups, page_size, pages, slots), plain.CacheManager(pgroups, page_size, pages, slots)
+
+
+def _same_state(m, p, live):
+    assert m.free_pages() == p.free_pages() and m.free_slots() == p.free_slots()
+    for g, (a, b) in enumerate(zip(m.pools, p.pools)):
+        assert a._free == b._free, g                               # the same pages, to be handed out in the same order
+    for rid in live:
+        a, b = m.get(rid), p.get(rid)
+        assert (a.length, a.reserved, a.tables, a.state_slot) == (b.length, b.reserved, b.tables, b.state_slot), rid
+    assert sorted(m.live()) == sorted(p.live()) == sorted(live)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_native_manager_follows_the_plain_one(seed):
+    import plain_cache_manager as plain
+    rng = random.Random(100 + seed)
+    m, p = _both(pages=rng.choice([6, 10, 17]), window=rng.choice([24, 40, 7]), slots=4)
+    live, next_id = [], 0
+    for _ in range(500):
+        op = rng.random()
+        if op < 0.2:
+            outcome = []
+            for mgr, exc in ((m, OutOfSlots), (p, plain.OutOfSlots)):
+                try:
+                    outcome.append(mgr.add(next_id))
+                except exc:
+                    outcome.append("full")
+            assert outcome[0] == outcome[1]
+            if outcome[0] != "full":
+                live.append(next_id)
+            next_id += 1
+        elif op < 0.8 and live:
+            rid, n = rng.choice(live), rng.choice([1, 1, 1, 2, 5, 16, 31, 70])
+            assert m.pages_needed(rid, n) == p.pages_needed(rid, n)
+            needs = [(r, rng.choice([1, 3, 20])) for r in rng.sample(live, rng.randint(1, len(live)))]
+            assert m.can_reserve(needs) == p.can_reserve(needs)
+            outcome = []
+            for mgr, exc in ((m, OutOfPages), (p, plain.OutOfPages)):
+                try:
+                    mgr.reserve(rid, n)
+                    outcome.append("ok")
+                except exc as e:
+                    outcome.append((e.group, e.needed, e.free))
+            assert outcome[0] == outcome[1]
+            if outcome[0] == "ok":
+                k = rng.choice([n, n, max(1, n // 2)])              # a step may commit less than was reserved
+                m.commit(rid, k); p.commit(rid, k)
+        elif live:
+            rid = live.pop(rng.randrange(len(live)))
+            m.free(rid); p.free(rid)
+        m.check(); p.check()
+        _same_state(m, p, live)
+    for rid in live:
+        with pytest.raises(ValueError, match="beyond"):
+            m.commit(rid, 10 ** 6)
+        with pytest.raises(ValueError, match="positive"):
+            m.reserve(rid, 0)
+
+
+def test_a_steps_arrays_from_the_native_manager():
+    """Lengths, positions, block tables and write slots of a step, against the plain manager's tables."""
+    import numpy as np
+    m, p = _both(pages=40, window=24, slots=4)
+    for mgr in (m, p):
+        for rid, n in (("a", 37), ("b", 5), ("c", 70)):
+            mgr.add(rid); mgr.reserve(rid, n); mgr.commit(rid, n)
+        for rid, n in (("a", 3), ("b", 1), ("c", 20)):
+            mgr.reserve(rid, n)
+    rids, q_len = ["c", "a", "b"], [20, 3, 1]
+    arr = m.step_arrays(rids, q_len, 8)
+    start = [p.length(r) for r in rids]
+    assert arr["start"].tolist() == start and arr["q_start"].tolist() == [0, 20, 23] and arr["kv_len"].tolist() == [90, 40, 6]
+    assert arr["state_slots"].tolist() == [p.state_slot(r) for r in rids]
+    assert arr["row_req"].tolist() == [0] * 20 + [1] * 3 + [2]
+    assert arr["positions"].tolist() == list(range(70, 90)) + [37, 38, 39] + [5]
+    for g in range(2):
+        tables = [p.block_table(r, g) for r in rids]
+        width = -(-max(len(t) for t in tables) // 8) * 8
+        want = np.full((3, width), -1, dtype=np.int32)
+        for i, t in enumerate(tables):
+            want[i, :len(t)] = t
+        assert np.array_equal(arr["block_tables"][g], want)
+        slots = [tables[i][pos // 16] * 16 + pos % 16 for i, pos in zip(arr["row_req"].tolist(), arr["positions"].tolist())]
+        assert arr["write_slots"][g].tolist() == slots
+    with pytest.raises(RuntimeError, match="no page"):
+        m.step_arrays(["b"], [40], 8)                                # 6 + 40 positions, pages for 6 + 1
+    with pytest.raises(KeyError):
+        m.step_arrays(["nobody"], [1], 8)
+    empty = m.step_arrays([], [], 8)
+    assert empty["positions"].shape == (0,) and [t.shape for t in empty["block_tables"]] == [(0, 8), (0, 8)]
+
+
+def test_many_requests_in_one_call():
+    m = two_groups(pages=12)
+    for rid, n in (("a", 20), ("b", 3)):
+        m.add(rid); m.reserve(rid, n); m.commit(rid, n)
+    snap = m.snapshot(["a", "b"])
+    assert m.unchanged(snap, ["a", "b"]) and not m.unchanged(snap, ["b", "a"]) and not m.unchanged(snap, ["a"])
+    m.reserve("a", 1); m.reserve("b", 1)
+    assert m.unchanged(snap, ["a", "b"])                       # pages taken ahead move nothing
+    m.commit_each(["a", "b"], 1)
+    assert (m.length("a"), m.length("b")) == (21, 4) and not m.unchanged(snap, ["a", "b"])
+    with pytest.raises(ValueError, match="beyond"):
+        m.commit_each(["a", "b"], 1)                           # nothing reserved: neither moves
+    assert (m.length("a"), m.length("b")) == (21, 4)
+    snap = m.snapshot(["a", "b"])
+    m.free("b"); m.add("b"); m.reserve("b", 4); m.commit("b", 4)
+    assert not m.unchanged(snap, ["a", "b"])                   # the same name and length, another request
+    m.check()
