@@ -327,10 +327,12 @@ class ScaledRows:
     past T hold zeros).  A weight-streaming product that takes these multiplies its sums by the factor, which
     saves the norm a kernel of its own; ``linear_into_stream`` makes them."""
 
-    __slots__ = ("rows", "pieces", "width", "eps")
+    __slots__ = ("rows", "pieces", "width", "eps", "norm_weight")
 
-    def __init__(self, rows: torch.Tensor, pieces: torch.Tensor, width: int, eps: float):
+    def __init__(self, rows: torch.Tensor, pieces: torch.Tensor, width: int, eps: float,
+                 norm_weight: Optional[torch.Tensor] = None):
         self.rows, self.pieces, self.width, self.eps = rows, pieces, int(width), float(eps)
+        self.norm_weight = norm_weight      # the weight the rows were multiplied by: whose norm they stand for
 
     @property
     def shape(self):
@@ -409,7 +411,7 @@ def linear_into_stream(x: torch.Tensor, weight: LinearWeight, stream: torch.Tens
     _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
           x.data_ptr(), w.data_ptr(), 0, DT_F32, M, N, K, 0, 0, 0, 2, 0 if weight.tiled is None else 1, 0,
           0, 0, 0.0, 0.0, stream.data_ptr(), norm_weight.data_ptr(), rows.data_ptr(), pieces.data_ptr(), _stream())
-    return ScaledRows(rows, pieces, N, eps)
+    return ScaledRows(rows, pieces, N, eps, norm_weight)
 
 
 _SKINNY_ARGS = (P, P, P, I, I, I, I, I, I, I, I, I, P, P, I, F, F, P, P, P, P, P)

@@ -22,9 +22,11 @@ def _normed(norm, reader, residual, pending, ctx):
     """What ``reader`` is given: the norm of the stream plus ``pending``."""
     if isinstance(pending, ScaledRows):          # the delta is in the stream already
         accepts = getattr(reader, "accepts_scaled_rows", None)
-        if accepts is not None and accepts(pending.shape[0]):
+        params = norm.rms_params()
+        made_for_this_norm = params is not None and pending.norm_weight is params[0] and pending.eps == params[1]
+        if made_for_this_norm and accepts is not None and accepts(pending.shape[0]):
             return pending
-        pending = None
+        pending = None                           # (rows prepared for another norm are of no use: the stream is)
     return norm.forward(residual, pending, ctx.act_dtype)
 
 
