@@ -247,6 +247,7 @@ def run_workload(args, w) -> int:
         "total_s": round(dt, 2), "prompt_tok_per_s_overall": round(sum(lens) / dt, 1),
         "ttft_s": {"min": round(ttft[0], 3), "median": round(ttft[len(ttft) // 2], 3), "max": round(ttft[-1], 3)},
         "preemptions": eng.stats.preemptions,
+        "steps_by_tokens": {f"<={k}": n for k, n in sorted(eng.stats.step_tokens.items())},
     }
     print(json.dumps(out), flush=True)
     return 0

@@ -46,6 +46,8 @@ class EngineStats:
     generated_tokens: int = 0
     steps: int = 0
     preemptions: int = 0
+    # steps by their number of tokens: key 2**k counts the steps of more than 2**(k-1) and at most 2**k tokens
+    step_tokens: Dict[int, int] = dataclasses.field(default_factory=dict)
 
 
 class _Live:
@@ -145,6 +147,8 @@ class Engine:
         else:
             self.stats.decode_ms += dt
         self.stats.steps += 1
+        bucket = 1 << (sum(len(i.tokens) for i in plan.items) - 1).bit_length()
+        self.stats.step_tokens[bucket] = self.stats.step_tokens.get(bucket, 0) + 1
         for i in plan.items:
             self.scheduler.advance(i)
         done: List[RequestOutput] = []

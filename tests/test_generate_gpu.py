@@ -161,6 +161,7 @@ def test_phase_timing_and_cache_planning(model_folders, capfd):
     assert [p.num_pages for p in timed.runner.manager.pools] == [32, 32] and not timed.runner.decode_graphs
     got = timed.generate([prompt], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0].token_ids
     assert got == want
+    assert timed.stats.steps == 5 and timed.stats.step_tokens == {32: 1, 1: 4}    # the prompt's 20 tokens, then one at a time
     err = capfd.readouterr().err
     assert "[phase_timing] #1 L=4 tokens=20" in err and "mixer=" in err and "lm_head=" in err
     t = timed.runner.timer
