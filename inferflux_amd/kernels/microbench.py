@@ -3,6 +3,7 @@
     python -m inferflux_amd.kernels.microbench attention-tiles --rows 8192 [--query-tiles 2]
     python -m inferflux_amd.kernels.microbench attention-rows --batch 64 --context 3072 [--chunk 512]
     python -m inferflux_amd.kernels.microbench gemm --rows 8 [--shape gate_up]
+    python -m inferflux_amd.kernels.microbench ceilings
 
 Sizes default to the Qwen2.5-7B shape (28 query heads, 4 kv heads, head size 128, hidden 3584,
 intermediate 18944).  Times are averages of back-to-back launches between two events and include what
@@ -93,10 +94,49 @@ def gemm(args) -> None:
         del ws
 
 
+def ceilings(args) -> None:
+    """What a kernel that only reads (or copies) gets from this card's memory, and the library's large products."""
+    dev = "cuda"
+    pool = torch.zeros(int(args.pool_gb * 2**30) // 4, dtype=torch.float32, device=dev)
+    pool_bytes = pool.numel() * 4
+    for mb in (32, 128, 512, 2048):
+        n = mb * 2**20 // 4
+        if 2 * n > pool.numel():
+            continue
+        places = pool_bytes // (n * 4)            # each launch reads another piece of the pool: nothing is found in a cache
+        for streaming in (False, True):
+            best = None
+            for waves in (2048, 4096, 8192):
+                t = _time_us(lambda i: ops.stream_read(pool[(i % places) * n:(i % places + 1) * n], waves, streaming), args.iters)
+                if best is None or t < best[0]:
+                    best = (t, waves)
+            print(f"read  {mb:5d} MB {'streaming' if streaming else 'plain    '} loads: {best[0]:8.1f} us  "
+                  f"{mb * 2**20 / best[0] / 1e6:5.2f} TB/s  ({best[1]} waves)", flush=True)
+    for mb in (128, 1024):
+        n = mb * 2**20 // 4
+        places = pool_bytes // (2 * n * 4)
+        if places < 1:
+            continue
+        for streaming in (False, True):
+            def copy(i):
+                at = (i % places) * 2 * n
+                ops.stream_copy(pool[at:at + n], pool[at + n:at + 2 * n], 4096, streaming)
+            t = _time_us(copy, args.iters)
+            print(f"copy  {mb:5d} MB {'streaming' if streaming else 'plain    '}: {t:8.1f} us  "
+                  f"{2 * mb * 2**20 / t / 1e6:5.2f} TB/s read + written", flush=True)
+    del pool
+    for dtype, size in ((torch.bfloat16, 8192), (torch.float32, 4096)):
+        a = torch.randn(size, size, device=dev, dtype=dtype)
+        b = torch.randn(size, size, device=dev, dtype=dtype)
+        t = _time_us(lambda i: torch.matmul(a, b.t()), args.iters)
+        print(f"library product {size}^3 {str(dtype).split('.')[1]}: {t:8.1f} us  {2 * size**3 / t / 1e6:7.1f} TFLOP/s", flush=True)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="python -m inferflux_amd.kernels.microbench")
     sub = ap.add_subparsers(dest="what", required=True)
-    for name, fn in (("attention-tiles", attention_tiles), ("attention-rows", attention_rows), ("gemm", gemm)):
+    for name, fn in (("attention-tiles", attention_tiles), ("attention-rows", attention_rows), ("gemm", gemm),
+                     ("ceilings", ceilings)):
         p = sub.add_parser(name)
         p.set_defaults(fn=fn)
         p.add_argument("--iters", type=int, default=10)
@@ -115,6 +155,8 @@ def main(argv=None) -> int:
             p.add_argument("--rotate-gb", type=float, default=2.0,
                            help="memory the launches rotate through (a model's step touches tens of GB between two uses of a cache)")
             p.add_argument("--pages", choices=["shuffled", "in-order"], default="shuffled", help="how a request's pages lie in the pool")
+        if name == "ceilings":
+            p.add_argument("--pool-gb", type=float, default=16.0, help="memory the reads and copies rotate through")
         if name == "gemm":
             p.add_argument("--rows", type=int, default=8, help="rows of x")
             p.add_argument("--shape", choices=list(GEMM_SHAPES), default=None)

@@ -8,7 +8,7 @@ missing library or a refused size raises.
 from __future__ import annotations
 
 import ctypes
-from typing import Iterable, Optional, Tuple
+from typing import Dict, Iterable, Optional, Tuple
 
 import torch
 
@@ -47,6 +47,7 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("sampling", ())
     yield ("gemm_bf16", ())
     yield ("gemm_wide", ())
+    yield ("ceilings", ())            # measurement only: what the memory gives a kernel that just reads
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
             yield ("attn_mfma", (("HEAD_DIM", d), ("TILE_QT", qt)))
@@ -788,3 +789,27 @@ def logprobs(logits: torch.Tensor, chosen: torch.Tensor, top_n: int):
     _call(load_module("sampling"), "ifx_logprobs", (P, P, I, I, I, P, P, P, P),
           logits.data_ptr(), chosen.data_ptr(), R, V, top_n, lp.data_ptr(), top_ids.data_ptr(), top_lp.data_ptr(), _stream())
     return lp, top_ids, top_lp
+
+
+# ----------------------------------------------------------------------------------------
+_SINKS: Dict[int, torch.Tensor] = {}
+
+
+def stream_read(region: torch.Tensor, waves: int, streaming: bool) -> None:
+    """Measurement only: ``waves`` single-wave workgroups read the whole of ``region`` (a multiple of 8 KB) once."""
+    _check(region, "region")
+    sink = _SINKS.get(region.device.index)
+    if sink is None:
+        sink = _SINKS[region.device.index] = torch.zeros(1, dtype=torch.float32, device=region.device)
+    _call(load_module("ceilings"), "ifx_stream_read", (P, LL, I, I, P, P),
+          region.data_ptr(), region.numel() * region.element_size(), waves, int(streaming), sink.data_ptr(), _stream())
+
+
+def stream_copy(src: torch.Tensor, dst: torch.Tensor, waves: int, streaming: bool) -> None:
+    """Measurement only: copies ``src`` to ``dst`` (same size, a multiple of 8 KB) with ``waves`` single-wave workgroups."""
+    _check(src, "src")
+    _check(dst, "dst")
+    n = src.numel() * src.element_size()
+    if n != dst.numel() * dst.element_size():
+        raise KernelError(f"stream_copy: {n} bytes into {dst.numel() * dst.element_size()}")
+    _call(load_module("ceilings"), "ifx_stream_copy", (P, P, LL, I, I, P), src.data_ptr(), dst.data_ptr(), n, waves, int(streaming), _stream())

@@ -814,3 +814,18 @@ def test_logprobs_against_log_softmax_and_topk():
         assert torch.allclose(tlp[r].double(), want[r, order], atol=1e-4)
     assert ids[1, :2].tolist() == [7, 100]
     assert ops.logprobs(logits.to(DEV), chosen.to(DEV), 0)[1].shape == (R, 0)
+
+
+def test_measurement_kernels_copy_what_they_read():
+    g = gen(23)
+    src = torch.randn(5 * 2048 * 3, generator=g).to(DEV)           # 15 rounds of 8 KB: no multiple of the grid
+    for streaming in (False, True):
+        for waves in (1, 4, 64):
+            dst = torch.zeros_like(src)
+            ops.stream_copy(src, dst, waves, streaming)
+            assert torch.equal(dst, src)
+            ops.stream_read(src, waves, streaming)
+    with pytest.raises(ops.KernelError, match="multiple of"):
+        ops.stream_read(src[:1000], 4, False)
+    with pytest.raises(ops.KernelError, match="overlap"):
+        ops.stream_copy(src[:4096], src[2048:6144], 4, False)
