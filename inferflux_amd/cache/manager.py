@@ -286,6 +286,13 @@ class CacheManager:
         return (list(rids), _ints(slots), (ctypes.c_longlong * len(slots))(*[self._n.cm_epoch(self._h, s) for s in slots]),
                 _ints([self._n.cm_length(self._h, s) for s in slots]))
 
+    @staticmethod
+    def snapshot_rows(snapshot, rows: Sequence[int]):
+        """The snapshot of only the requests at places ``rows`` of ``snapshot``."""
+        was, slots, epochs, lengths = snapshot
+        return ([was[i] for i in rows], _ints([slots[i] for i in rows]),
+                (ctypes.c_longlong * len(rows))(*[epochs[i] for i in rows]), _ints([lengths[i] for i in rows]))
+
     def unchanged(self, snapshot, rids: Sequence[Hashable]) -> bool:
         """Whether ``rids`` are the requests of the snapshot, in its order, all still live and none of them moved."""
         was, slots, epochs, lengths = snapshot

@@ -78,6 +78,11 @@ class CacheStorage:
     def binding(self, entry: int) -> MixerBinding:
         return self._bindings[entry]
 
+    @property
+    def has_state(self) -> bool:
+        """Whether any mixer keeps per-request state besides keys and values (a step over it cannot be run twice)."""
+        return bool(self._states)
+
     def reset_state(self, slot: int) -> None:
         """Zero every mixer's state of one slot: a request that starts sees no history."""
         for t in self._states.values():

@@ -57,8 +57,10 @@ class _Live:
 
 
 class Engine:
-    def __init__(self, runner: ModelRunner, scheduler_config: Optional[SchedulerConfig] = None):
+    def __init__(self, runner: ModelRunner, scheduler_config: Optional[SchedulerConfig] = None,
+                 start_steps_early: bool = True):
         self.runner = runner
+        self.start_steps_early = start_steps_early   # decode steps are started before the host has read the last step's tokens
         self.config = scheduler_config or SchedulerConfig()
         self.config.max_batch_size = min(self.config.max_batch_size, runner.manager.max_requests)
         self.scheduler = Scheduler(runner.manager, self.config, runner.max_position)
@@ -71,7 +73,8 @@ class Engine:
     @classmethod
     def load(cls, model: str, dtype: str = "bfloat16", kv_pages: Optional[int] = None, page_size: int = 16,
              max_batch_size: int = 32, max_batch_tokens: int = 16384, chunked_prefill_tokens: int = 512,
-             ctx_size: int = 4096, phase_timing: bool = False, decode_weight_copy: bool = True) -> "Engine":
+             ctx_size: int = 4096, phase_timing: bool = False, decode_weight_copy: bool = True,
+             start_steps_early: bool = True) -> "Engine":
         """``kv_pages`` None sizes the cache for ``ctx_size`` tokens for each of ``max_batch_size``
         requests, within the device memory that is free once the weights are loaded.
         ``decode_weight_copy`` False saves the second, tiled copy of the weights at the price of slower decoding."""
@@ -81,7 +84,7 @@ class Engine:
                              decode_weight_copy=decode_weight_copy)
         log.info("engine", "model loaded", model=model, dtype=dtype, kv_pages=runner.manager.pools[0].num_pages
                  if runner.manager.pools else 0, page_size=page_size, max_batch_size=max_batch_size)
-        return cls(runner, SchedulerConfig(max_batch_size, max_batch_tokens, chunked_prefill_tokens))
+        return cls(runner, SchedulerConfig(max_batch_size, max_batch_tokens, chunked_prefill_tokens), start_steps_early)
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
@@ -138,8 +141,15 @@ class Engine:
             # A step of decoding with nobody waiting: the next step is most likely the same requests, one token
             # further, less those that reach their limit now.  While the GPU works on this one, the runner gets
             # ready what of the next does not depend on its tokens; if the guess is wrong it is dropped.
+            # If nobody reaches a limit, the next step is also started there, with the tokens taken on the GPU: the
+            # host then reads them and does its bookkeeping while the GPU is already at work on the next step.  A
+            # request that stops on a token nobody could foresee only has its row of that step dropped.
             rids = [i.seq.rid for i in plan.items if len(i.seq.generated) + 1 < self._live[i.seq.rid].params.max_tokens]
-            ahead = lambda: self.runner.prepare_decode(rids)
+            start = len(rids) == len(plan.items) and self.start_steps_early
+
+            def ahead(chosen):
+                if self.runner.prepare_decode(rids) and start:
+                    self.runner.launch_prepared(chosen)
         tokens = self.sampler.sample(logits, [self._live[i.seq.rid].sampling for i in wanting], ahead) if wanting else []
         dt = (time.perf_counter() - t0) * 1e3
         if any(len(i.tokens) > 1 or i.seq.is_prefilling for i in plan.items):

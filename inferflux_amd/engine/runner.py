@@ -20,6 +20,7 @@ import torch
 
 from ..cache.manager import OutOfPages
 from ..cache.storage import CacheStorage
+from ..kernels import ops
 from .context import StepContext, StepEntry
 from .model import Model
 
@@ -67,6 +68,7 @@ class ModelRunner:
         self.decode_graphs = decode_graphs and model.graph_safe and self.timer is None
         self._graphs = {}
         self._prepared = None      # (the manager's snapshot of the requests, the context) of a step got ready ahead of its tokens
+        self._launched = None      # (that snapshot, the graph) of a step already started with tokens the host has not seen
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, rid: Hashable) -> None:
@@ -125,6 +127,55 @@ class ModelRunner:
         self._prepared = (self.manager.snapshot(rids), ctx)
         return True
 
+    def launch_prepared(self, tokens: torch.Tensor) -> bool:
+        """Start the step ``prepare_decode`` got ready, now, with its tokens taken on the GPU from ``tokens`` (int32,
+        one per request of that step, in its order: the sampler's output for the step before), so that the GPU goes
+        on while the host reads those tokens and does its bookkeeping.  ``step`` hands out the logits if it is then
+        given these requests with one token each (it trusts that they are the tokens of ``tokens``), or a part of
+        them in the same order (the others' rows are dropped: a request that has just stopped).  Any other step
+        makes it void and is computed afresh; keys and values written early are written again with the same
+        contents, which is why nothing is started early for a model whose mixers keep state of their own.
+        Returns False, the prepared step kept for ``step``, when it cannot (no captured graph of this layout yet)."""
+        prep = self._prepared
+        if prep is None or self.storage.has_state:
+            return False
+        snapshot, ctx = prep
+        g = self._graphs.get(ctx.layout_key)
+        if g is None or tokens.dtype != torch.int32 or tuple(tokens.shape) != (ctx.n_tokens,) or tokens.device != self.device:
+            return False
+        self._prepared = None
+        self._replay_inputs(g, ctx)
+        g.ctx.token_ids.copy_(tokens)          # (the copy above brought placeholder tokens; both precede the graph on the stream)
+        g.graph.replay()
+        self._launched = (snapshot, g)
+        return True
+
+    def _take_launched(self, entries):
+        """The logits of the step started early, if ``entries`` are its requests or a part of them; else None."""
+        (snapshot, g), self._launched = self._launched, None
+        if any(len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0 for e in entries):
+            return None
+        rids, was = [e.rid for e in entries], snapshot[0]
+        if len(rids) == len(was):
+            if not self.manager.unchanged(snapshot, rids):
+                return None
+            self.manager.commit_each(rids, 1)
+            return g.logits
+        place = {r: i for i, r in enumerate(was)}
+        rows = [place.get(r, -1) for r in rids]
+        if min(rows) < 0 or any(a >= b for a, b in zip(rows, rows[1:])):
+            return None
+        if not self.manager.unchanged(self.manager.snapshot_rows(snapshot, rows), rids):
+            return None
+        self.manager.commit_each(rids, 1)
+        return ops.embedding(torch.tensor(rows, dtype=torch.int32, device=self.device), g.logits)    # those rows of the logits
+
+    def _replay_inputs(self, g, ctx) -> None:
+        g.copied.synchronize()          # the host buffer is free again once the last copy out of it is done
+        ctx.write_host(g.host)          # (the replay reads the graph's own views of the slab: none are made here)
+        g.slab.copy_(g.pinned, non_blocking=True)
+        g.copied.record()
+
     def _take_prepared(self, entries):
         """The context ``prepare_decode`` built, if ``entries`` are the step it was built for (the same live
         requests, none of which has moved since), with their tokens put in; else None."""
@@ -143,6 +194,10 @@ class ModelRunner:
         entries = list(entries)
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        if self._launched is not None:
+            logits = self._take_launched(entries)
+            if logits is not None:
+                return logits
         ctx = self._take_prepared(entries) if self._prepared is not None else None
         if ctx is not None:
             logits = self._decode_step(entries, ctx)
@@ -178,10 +233,7 @@ class ModelRunner:
                               upload=False)
         g = self._graphs.get(ctx.layout_key)
         if g is not None:
-            g.copied.synchronize()          # the host buffer is free again once the last copy out of it is done
-            ctx.write_host(g.host)          # (the replay reads the graph's own views of the slab: none are made here)
-            g.slab.copy_(g.pinned, non_blocking=True)
-            g.copied.record()
+            self._replay_inputs(g, ctx)
             g.graph.replay()
             return g.logits
         slab = torch.empty(ctx.slab_size, dtype=torch.int32, device=self.device)

@@ -51,6 +51,18 @@ class SamplingState:
 class Sampler:
     def __init__(self, device):
         self.device = device
+        self._host_tokens = None      # pinned: the chosen tokens come to the host through it
+        self._copied = torch.cuda.Event()
+
+    def _to_host(self, t: torch.Tensor, keep: bool = False) -> torch.Tensor:
+        """An asynchronous copy of ``t`` into pinned host memory (valid once ``_copied`` has been waited for)."""
+        if keep:
+            if self._host_tokens is None or self._host_tokens.shape[0] < t.shape[0]:
+                self._host_tokens = torch.empty(max(64, t.shape[0]), dtype=t.dtype, pin_memory=True)
+            out = self._host_tokens[:t.shape[0]]
+        else:
+            out = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+        return out.copy_(t, non_blocking=True)
 
     def _dev(self, values, dtype):
         return torch.tensor(values, dtype=dtype, device=self.device)
@@ -58,8 +70,10 @@ class Sampler:
     def sample(self, logits: torch.Tensor, states: Sequence[SamplingState], while_waiting=None) -> List[int]:
         """One token per row of float32 ``logits`` [R, V]; row i belongs to ``states[i]``.  The
         logits are modified in place by penalties and bias.  States are advanced (draw counter,
-        history).  ``while_waiting`` is called once the kernels are launched, before their results are
-        waited for: host work that needs no token goes there."""
+        history).  ``while_waiting`` is called with the chosen tokens (int32 [R], on the GPU) once the kernels and
+        the copies of their results to the host are launched, before these are waited for: host work that needs no
+        token goes there, and so may GPU work that takes the tokens where they are; the wait is for the copies
+        only, not for what ``while_waiting`` launched."""
         R = logits.shape[0]
         if R != len(states):
             raise ValueError(f"{R} rows of logits for {len(states)} requests")
@@ -95,11 +109,13 @@ class Sampler:
         top_n = max((s.params.logprobs for s in states if s.params.logprobs is not None), default=None)
         if top_n is not None:
             lp_dev = ops.logprobs(logits, chosen, top_n)
+            lp, top_ids, top_lp = (self._to_host(t) for t in lp_dev)
+        host_tokens = self._to_host(chosen, keep=True)
+        self._copied.record()
         if while_waiting is not None:
-            while_waiting()
-        if top_n is not None:
-            lp, top_ids, top_lp = (t.cpu() for t in lp_dev)
-        tokens = chosen.cpu().tolist()
+            while_waiting(chosen)
+        self._copied.synchronize()
+        tokens = host_tokens.tolist()
         for r, (st, t) in enumerate(zip(states, tokens)):
             if st.params.logprobs is not None:
                 n = st.params.logprobs

@@ -287,6 +287,65 @@ def test_steps_of_few_rows_need_no_kernel_for_the_norms_between_products(name, s
     assert rel_err(fused, separate) < REL_TOL["bfloat16"]
 
 
+def test_a_decode_step_started_before_the_host_has_its_tokens(sharp_folders):
+    """launch_prepared starts the prepared step with tokens that are on the GPU only; step hands out its logits for
+    the same requests, or the rows of those that are left of them, and computes anything else afresh: bit for bit
+    the logits of steps that were not started early."""
+    folder, V = sharp_folders["C", "float32"], TINY["C"]["vocab_size"]
+    ids = {r: seeded_ids(40 + i, 70, V) for i, r in enumerate("abc")}
+    order = ["abc", "abc", "abc", "acb", "ab", "ab", "ab", "abc", "abc", "c"]
+
+    def run(early):
+        runner = load_runner(folder, torch.float32, num_pages=24)
+        out, outcome = [], []
+        for r in "abc":
+            runner.add_request(r)
+            runner.step([StepEntry(r, ids[r][:30], [])])
+        at = {r: 30 for r in "abc"}
+        for k, who in enumerate(order):
+            started = False
+            if early and k > 0:
+                guess = order[k - 1]
+                assert runner.prepare_decode(list(guess)) is True
+                tokens = torch.tensor([ids[r][at[r]] for r in guess], dtype=torch.int32, device="cuda")
+                started = runner.launch_prepared(tokens)
+                assert (runner._launched is not None) == started and (runner._prepared is None) == started
+            got = []
+            real = runner._take_launched
+            runner._take_launched = lambda e: (got.append(real(e)), got[0])[1]
+            out.append(runner.step([StepEntry(r, [ids[r][at[r]]], [0]) for r in who]).cpu())
+            del runner._take_launched
+            assert len(got) == int(started)
+            outcome.append("-" if not started else "void" if got[0] is None else "taken")
+            assert runner._launched is None and runner._prepared is None
+            for r in who:
+                at[r] += 1
+            runner.manager.check()
+        for r in "abc":
+            runner.free_request(r)
+        runner.manager.check()
+        assert runner.manager.free_pages() == [24] * len(runner.manager.groups)
+        return out, outcome
+
+    plain, _ = run(False)
+    early, outcome = run(True)
+    #          abc  abc      abc      acb (order)  ab of acb  ab (no graph yet)  ab   abc of ab  abc      c of abc
+    assert outcome == ["-", "taken", "taken", "void", "taken", "-", "taken", "void", "taken", "taken"]
+    for a, b in zip(plain, early):
+        assert torch.equal(a, b)
+    # tokens of another kind or number are refused, and so is a model whose mixers keep state of their own
+    runner = load_runner(folder, torch.float32, num_pages=24)
+    runner.add_request("x")
+    runner.step([StepEntry("x", ids["a"][:30], [])])
+    runner.step([StepEntry("x", [ids["a"][30]], [0])])                     # captures the graph of this layout
+    assert runner.prepare_decode(["x"])
+    assert not runner.launch_prepared(torch.zeros(2, dtype=torch.int32, device="cuda"))
+    assert not runner.launch_prepared(torch.zeros(1, dtype=torch.int64, device="cuda"))
+    assert not runner.launch_prepared(torch.zeros(1, dtype=torch.int32))
+    runner.storage._states[0] = torch.zeros(1, device="cuda")
+    assert not runner.launch_prepared(torch.zeros(1, dtype=torch.int32, device="cuda")) and runner._prepared is not None
+
+
 def test_a_decode_step_got_ready_ahead_of_its_tokens(sharp_folders):
     """prepare_decode does, before the tokens are known, what a step of single tokens needs besides them; step uses
     it for exactly that step and falls back to the ordinary path for any other, with the same logits either way."""

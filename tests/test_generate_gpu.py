@@ -42,29 +42,44 @@ def test_greedy_generation_equals_the_plain_model(name, model_folders):
     assert st.generated_tokens == n_new * len(prompts) and st.prompt_tokens == sum(lens)
 
 
-def test_steps_got_ready_ahead_change_no_token_and_are_used(model_folders, monkeypatch):
+def test_steps_got_ready_and_started_ahead_change_no_token_and_are_used(model_folders, monkeypatch):
     """While the GPU decodes, the engine gets the next decode step ready on a guess (the same requests, less those at
-    their limit).  A stop token makes the guess wrong once; tokens are the same with and without the guessing."""
+    their limit) and, where nobody is at a limit, starts it with the tokens taken on the GPU.  A stop token makes the
+    guess wrong once: only that request's row is dropped.  Tokens are the same with and without all this."""
     from inferflux_amd.engine.runner import ModelRunner
     folder = model_folders["B"]
     prompts = [seeded_ids(80 + i, n, TINY["B"]["vocab_size"]) for i, n in enumerate([5, 40, 23])]
     limits = (6, 30, 17)
 
-    def run(stop):
+    def run(stop, **kw):
         params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True, stop_token_ids=stop if i == 1 else ())
                   for i, n in enumerate(limits)]
-        return Engine.load(folder, dtype="bfloat16", kv_pages=64, max_batch_size=4).generate(prompts, params)
+        eng = Engine.load(folder, dtype="bfloat16", kv_pages=64, max_batch_size=4, **kw)
+        outs = eng.generate(prompts, params)
+        eng.runner.manager.check()
+        assert eng.runner.manager.free_pages() == [64]
+        return outs
 
-    taken = []
-    real, real_prepare = ModelRunner._take_prepared, ModelRunner.prepare_decode
+    taken, started = [], []
+    real, real_launched = ModelRunner._take_prepared, ModelRunner._take_launched
     monkeypatch.setattr(ModelRunner, "_take_prepared", lambda self, e: _count(taken, real(self, e)))
+    monkeypatch.setattr(ModelRunner, "_take_launched", lambda self, e: _count(started, real_launched(self, e)))
     with_it = run(())
     assert [len(o.token_ids) for o in with_it] == list(limits)
-    assert sum(taken) >= 20 and all(taken)                 # requests that reach their limit are foreseen
-    stop = [with_it[1].token_ids[12]]
-    del taken[:]
+    assert sum(started) >= 15 and all(started) and all(taken)     # requests that reach their limit are foreseen
+    n_taken = len(taken)
+    ids1 = with_it[1].token_ids
+    at = next(j for j in range(8, 16) if ids1[j] not in ids1[:j])   # a token's first appearance, while nobody is at a limit
+    stop = [ids1[at]]
+    del taken[:], started[:]
     stopped = run(stop)
-    assert stopped[1].finish_reason == "stop" and len(stopped[1].token_ids) <= 13 and not all(taken)
+    assert stopped[1].finish_reason == "stop" and stopped[1].token_ids == ids1[:at + 1]
+    assert all(started) and all(taken)                             # the stopped request's row was dropped, no step lost
+    del taken[:], started[:]
+    only_ready = run((), start_steps_early=False)
+    assert not started and len(taken) > n_taken and all(taken)
+    assert [o.token_ids for o in only_ready] == [o.token_ids for o in with_it]
+    assert [o.token_ids for o in run(stop, start_steps_early=False)] == [o.token_ids for o in stopped]
     monkeypatch.setattr(ModelRunner, "prepare_decode", lambda self, rids: False)
     assert [o.token_ids for o in run(())] == [o.token_ids for o in with_it]
     assert [o.token_ids for o in run(stop)] == [o.token_ids for o in stopped]
