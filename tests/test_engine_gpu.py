@@ -592,3 +592,39 @@ def test_prompt_portions_with_a_long_past_split_their_keys(sharp_folders, monkey
             pos += n
         runner.free_request("p")
     assert max(calls) > 1      # some portion did run in splits
+
+
+ODD_SIZES = {
+    # hidden width that no head count divides into, feed-forward and vocabulary that are multiples of nothing much
+    "width100": dict(vocab_size=333, hidden_size=100, num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=5,
+                     head_dim=16, intermediate_size=90),
+    # thirty-two query heads on one key head (two tiles of sixteen in the grouped kernels)
+    "ratio32": dict(vocab_size=5001, hidden_size=200, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=1,
+                    head_dim=48, intermediate_size=1000),
+    # a head size beyond what the matrix-core attention takes: the plain kernel in both precisions
+    "head256": dict(vocab_size=1111, hidden_size=136, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1,
+                    head_dim=256, intermediate_size=264),
+    # seventeen heads of 80
+    "heads17": dict(vocab_size=4099, hidden_size=272, num_hidden_layers=1, num_attention_heads=17, num_key_value_heads=17,
+                    head_dim=80, intermediate_size=530, tie_word_embeddings=True),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(ODD_SIZES))
+def test_sizes_that_are_multiples_of_little(name, dtype, tmp_path):
+    from conftest import QK_GAIN, sharpen
+    from inferflux_amd.config import config_from_dict
+    from inferflux_amd.weights import write_random_model
+    cfg = {**TINY["A"], "tie_word_embeddings": False, **ODD_SIZES[name]}
+    raw, folder = str(tmp_path / "raw"), str(tmp_path / "sharp")
+    write_random_model(raw, config_from_dict(cfg), seed=5, dtype=torch.bfloat16)
+    sharpen(raw, folder, 6, QK_GAIN[dtype] / 2 if name == "heads17" else QK_GAIN[dtype])   # (272 wide: scores grow with the width)
+    ids = seeded_ids(3, 120, cfg["vocab_size"])
+    want = plain_logits(folder, ids)
+    runner = load_runner(folder, DT[dtype], num_pages=16)
+    runner.add_request("a")
+    got = [runner.step([StepEntry("a", ids[:70], list(range(70)))]).cpu(),
+           runner.step([StepEntry("a", ids[70:87], list(range(17)))]).cpu()]        # 17 rows: one more than a tile
+    got += [runner.step([StepEntry("a", [ids[p]], [0])]).cpu() for p in range(87, 120)]
+    assert rel_err(torch.cat(got), want) < REL_TOL[dtype]
