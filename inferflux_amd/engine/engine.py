@@ -141,15 +141,21 @@ class Engine:
             # A step of decoding with nobody waiting: the next step is most likely the same requests, one token
             # further, less those that reach their limit now.  While the GPU works on this one, the runner gets
             # ready what of the next does not depend on its tokens; if the guess is wrong it is dropped.
-            # If nobody reaches a limit, the next step is also started there, with the tokens taken on the GPU: the
-            # host then reads them and does its bookkeeping while the GPU is already at work on the next step.  A
-            # request that stops on a token nobody could foresee only has its row of that step dropped.
-            rids = [i.seq.rid for i in plan.items if len(i.seq.generated) + 1 < self._live[i.seq.rid].params.max_tokens]
-            start = len(rids) == len(plan.items) and self.start_steps_early
+            # Where it can, the runner also starts that step, for everyone of this one and with the tokens taken on
+            # the GPU: the host then reads them and does its bookkeeping while the GPU is already at work on the
+            # next step.  A request that is at its limit, or stops on a token nobody could foresee, only has its
+            # row of that step dropped.
+            everyone = [i.seq.rid for i in plan.items]
+            staying = [i.seq.rid for i in plan.items if len(i.seq.generated) + 1 < self._live[i.seq.rid].params.max_tokens]
+            early = self.start_steps_early and self.runner.starts_steps_early and bool(staying)
 
             def ahead(chosen):
-                if self.runner.prepare_decode(rids) and start:
-                    self.runner.launch_prepared(chosen)
+                if early:
+                    if self.runner.prepare_decode(everyone) and self.runner.launch_prepared(chosen):
+                        return
+                    if len(staying) == len(everyone):
+                        return                      # what was got ready stands
+                self.runner.prepare_decode(staying)
         tokens = self.sampler.sample(logits, [self._live[i.seq.rid].sampling for i in wanting], ahead) if wanting else []
         dt = (time.perf_counter() - t0) * 1e3
         if any(len(i.tokens) > 1 or i.seq.is_prefilling for i in plan.items):

@@ -127,6 +127,11 @@ class ModelRunner:
         self._prepared = (self.manager.snapshot(rids), ctx)
         return True
 
+    @property
+    def starts_steps_early(self) -> bool:
+        """Whether ``launch_prepared`` can ever start a step (graphs are on and no mixer keeps state of its own)."""
+        return self.decode_graphs and not self.storage.has_state
+
     def launch_prepared(self, tokens: torch.Tensor) -> bool:
         """Start the step ``prepare_decode`` got ready, now, with its tokens taken on the GPU from ``tokens`` (int32,
         one per request of that step, in its order: the sampler's output for the step before), so that the GPU goes
