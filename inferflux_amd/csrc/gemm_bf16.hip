@@ -98,7 +98,8 @@ __device__ __forceinline__ float row_factor(const RowScale& s, int lane) {
 // sums (wave 0); the others are done.
 template <int MT, int NT, int U, bool TILED>
 __device__ __forceinline__ bool skinny_accumulate(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, int M, int N,
-                                                  int K, int k_tiles, int first_tile, floatx4 (&acc)[NT][MT], float* red) {
+                                                  int K, int k_tiles, int first_tile, floatx4 (&acc)[NT][MT], float* red,
+                                                  int tile_rows = 16) {
   const int wid = threadIdx.x / WAVE, nw = blockDim.x / WAVE, lane = threadIdx.x % WAVE;
   const int col = lane & 15, g = lane >> 4;
 #pragma unroll
@@ -109,8 +110,9 @@ __device__ __forceinline__ bool skinny_accumulate(const bf16_t* __restrict__ x, 
   const bf16_t* wrow[NT];  // rows (tiles) past N are read again, never stored
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
-    wrow[nt] = TILED ? W + ((size_t)min(first_tile + nt, (N - 1) / 16) * k_tiles * WAVE + lane) * 8
+    wrow[nt] = TILED ? W + ((size_t)min(first_tile + nt, (N - 1) / tile_rows) * k_tiles * 4 * tile_rows + tile_rows * g + col) * 8
                      : W + (size_t)min(16 * (first_tile + nt) + col, N - 1) * K;
+  const bool row_held = !TILED || col < tile_rows;   // a tile of the copy holds tile_rows rows: the other lanes' rows are zeros
   const bf16_t* xrow[MT];
   bool xok[MT];
 #pragma unroll
@@ -128,8 +130,8 @@ __device__ __forceinline__ bool skinny_accumulate(const bf16_t* __restrict__ x, 
       for (int h = 0; h < 2; ++h) {
         // the lane's 8 k-values of step h of block kb0 + u, and where its piece of W lies
         const int k = TILED ? (kb0 + u) * 64 + 32 * h + 8 * g : (kb0 + u) * 64 + 16 * g + 8 * h;
-        const size_t w_off = TILED ? (size_t)(2 * (kb0 + u) + h) * WAVE * 8 : (size_t)k;
-        const bool blk = kb0 + u < nkb, kok = blk && k < K;
+        const size_t w_off = TILED ? (size_t)(2 * (kb0 + u) + h) * 4 * tile_rows * 8 : (size_t)k;
+        const bool blk = kb0 + u < nkb && row_held, kok = kb0 + u < nkb && k < K;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           // Tiles are read once, in whole lines: a streaming load keeps them from pushing x out of the L2.
@@ -181,50 +183,58 @@ __device__ __forceinline__ bool skinny_accumulate(const bf16_t* __restrict__ x, 
 // ``order`` (tiled copies only): tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
 // ``scale`` (up to 16 rows): the results of row m are multiplied by the row's factor first.
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
 
 template <int MT, int NT, int U, typename TO, int EPI, bool TILED>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out,
                                    int M, int N, int K, int k_tiles, const int* __restrict__ order, RowScale scale,
-                                   StreamOut so) {
+                                   StreamOut so, int tile_rows) {
   extern __shared__ float red[];  // [(waves - 1)][NT * MT][64 lanes][4]
   const int lane = threadIdx.x % WAVE, col = lane & 15, g = lane >> 4;
-  const int first_tile = blockIdx.x * NT, n_tiles = (N + 15) / 16;
+  const int first_tile = blockIdx.x * NT, n_tiles = (N + tile_rows - 1) / tile_rows;
   const bool first_wave = threadIdx.x < WAVE;
   float rs = 1.f;
   if (MT == 1 && scale.pieces && first_wave) rs = row_factor(scale, lane);
+  // The lane's four sums of a tile are rows 4 g ... 4 g + 3 of it, handled as two pairs: tile_rows is even, so a
+  // pair is held or not as a whole, and a pair's first column is even.
   // EPI 2: what the epilogue reads is asked for before the stream of weights, not after it
-  floatx4 was[NT];
-  bf16x4 nw[NT];
+  floatx2 was[NT][2];
+  bf16x2 nw[NT][2];
   if (EPI == 2 && first_wave) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int n = 16 * (first_tile + nt) + 4 * g;
-      const bool ok = n < N && col < M;
-      was[nt] = ok ? *(const floatx4*)(so.stream + (size_t)col * N + n) : floatx4{0.f, 0.f, 0.f, 0.f};
-      if (ok) nw[nt] = *(const bf16x4*)(so.norm_w + n);
-    }
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int n = tile_rows * (first_tile + nt) + 4 * g + 2 * q;
+        const bool ok = 4 * g + 2 * q < tile_rows && n < N && col < M;
+        was[nt][q] = ok ? *(const floatx2*)(so.stream + (size_t)col * N + n) : floatx2{0.f, 0.f};
+        if (ok) nw[nt][q] = *(const bf16x2*)(so.norm_w + n);
+      }
   }
   floatx4 acc[NT][MT];
-  if (!skinny_accumulate<MT, NT, U, TILED>(x, W, M, N, K, k_tiles, first_tile, acc, red)) return;
-  // acc[nt][mt][r] = out[m = 16 mt + col][n = 16 (row tile of the weight) + 4 g + r]
+  if (!skinny_accumulate<MT, NT, U, TILED>(x, W, M, N, K, k_tiles, first_tile, acc, red, tile_rows)) return;
+  // acc[nt][mt][r] = out[m = 16 mt + col][n = tile_rows (row tile of the weight) + 4 g + r], for 4 g + r < tile_rows
   if (EPI == 2) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       if (first_tile + nt >= n_tiles) continue;   // the same for the whole wave
-      const int n = 16 * (first_tile + nt) + 4 * g;
-      const bool ok = n < N && col < M;
       float sq = 0.f;
-      if (ok) {
-        floatx4 v;
-        bf16x4 y;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          v[r] = was[nt][r] + acc[nt][0][r] * rs;
-          y[r] = (__bf16)(v[r] * (float)nw[nt][r]);
-          sq += v[r] * v[r];
+      for (int q = 0; q < 2; ++q) {
+        const int n = tile_rows * (first_tile + nt) + 4 * g + 2 * q;
+        if (4 * g + 2 * q < tile_rows && n < N && col < M) {
+          floatx2 v;
+          bf16x2 y;
+#pragma unroll
+          for (int r = 0; r < 2; ++r) {
+            v[r] = was[nt][q][r] + acc[nt][0][2 * q + r] * rs;
+            y[r] = (__bf16)(v[r] * (float)nw[nt][q][r]);
+            sq += v[r] * v[r];
+          }
+          *(floatx2*)(so.stream + (size_t)col * N + n) = v;
+          *(bf16x2*)(so.rows + (size_t)col * N + n) = y;
         }
-        *(floatx4*)(so.stream + (size_t)col * N + n) = v;
-        *(bf16x4*)(so.rows + (size_t)col * N + n) = y;
       }
       sq = sum_over_groups(sq);
       if (g == 0) so.pieces[(size_t)(first_tile + nt) * 16 + col] = sq;
@@ -234,7 +244,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     if (first_tile + nt >= n_tiles) continue;
-    const int n0 = 16 * ((TILED && order) ? order[first_tile + nt] : first_tile + nt);
+    const int n0 = tile_rows * ((TILED && order) ? order[first_tile + nt] : first_tile + nt);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = 16 * mt + col;
@@ -243,14 +253,14 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* _
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int n = n0 + 4 * g + r;
-          if (n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r] * rs);
+          if (4 * g + r < tile_rows && n < N) out[(size_t)m * N + n] = from_f<TO>(acc[nt][mt][r] * rs);
         }
       } else {
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
           const int n = n0 + 4 * g + r;  // even: gate at n, up at n + 1
           const float gt = acc[nt][mt][r] * rs, up = acc[nt][mt][r + 1] * rs;
-          if (n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+          if (4 * g + r < tile_rows && n + 1 < N) out[(size_t)m * (N / 2) + n / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
         }
       }
     }
@@ -336,13 +346,13 @@ __global__ void qkv_rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __re
 
 template <int MT, int NT, int U, bool TILED>
 static int launch(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int k_tiles, int waves, int epi,
-                  const int* order, const RowScale& scale, const StreamOut& so, hipStream_t s) {
-  const int groups = (N + 16 * NT - 1) / (16 * NT);
+                  const int* order, const RowScale& scale, const StreamOut& so, int tile_rows, hipStream_t s) {
+  const int groups = ((N + tile_rows - 1) / tile_rows + NT - 1) / NT;
   const size_t lds = (size_t)(waves - 1) * NT * MT * WAVE * 4 * sizeof(float);
   IFX_REQUIRE(lds <= 64 * 1024, "skinny_gemm: %d waves of %dx%d tiles need %zu bytes of LDS", waves, NT, MT, lds);
 #define GO(TO_, EPI_)                                                                                              \
   hipLaunchKernelGGL((skinny_gemm_kernel<MT, NT, U, TO_, EPI_, TILED>), dim3(groups), dim3(waves * WAVE), lds, s,  \
-                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles, order, scale, so)
+                     (const bf16_t*)x, (const bf16_t*)W, (TO_*)out, M, N, K, k_tiles, order, scale, so, tile_rows)
   if (epi == 2) {
     if constexpr (MT == 1) GO(float, 2);
     else IFX_FAIL("skinny_gemm: the stream epilogue takes at most 16 rows");
@@ -354,30 +364,39 @@ static int launch(const void* x, const void* W, void* out, int out_dtype, int M,
   IFX_LAUNCH_CHECK();
 }
 
-// Rows and k-values of the tiled form of an [N, K] weight: whole tiles, an even number along k.
+// The tiled form of an [N, K] weight: row tiles of ``tile_rows`` rows (even, 8 to 16; the last one padded with
+// zeros), k in whole tiles of 32, an even number of them.  Piece ((t k_tiles + kt) 4 + g) tile_rows + col
+// (16 bytes) holds the 8 k-values from 32 kt + 8 g of row tile t's row col: a wave reads a (t, kt) as 64 tile_rows
+// contiguous bytes, lane 16 g + col taking that piece (lanes with col >= tile_rows none), which is its share of
+// the 16x32 operand of the matrix core, rows past tile_rows being zeros.  Fewer than 16 rows to a tile are for
+// weights with so few rows that 16-row tiles would leave compute units without a tile (see ops.choose_tile_rows).
 extern "C" int ifx_tiled_rows(int N) { return (N + 15) / 16 * 16; }
 extern "C" int ifx_tiled_cols(int K) { return (K + 63) / 64 * 64; }
+extern "C" long long ifx_tiled_size(int N, int K, int tile_rows) {   // elements of the copy
+  return (long long)((N + tile_rows - 1) / tile_rows) * tile_rows * ifx_tiled_cols(K);
+}
 
 __global__ void tile_weights_kernel(const bf16_t* __restrict__ W, bf16_t* __restrict__ Wt, int N, int K, int k_tiles, size_t pieces,
-                                    const int* __restrict__ order) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // piece number: ((t * k_tiles + kt) * 64 + 16 g + col)
+                                    const int* __restrict__ order, int tile_rows) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // piece number: ((t * k_tiles + kt) * 4 + g) * tile_rows + col
   if (i >= pieces) return;
-  const int lane = (int)(i % WAVE), col = lane & 15, g = lane >> 4;
-  const size_t tile = i / WAVE;
+  const int col = (int)(i % tile_rows), g = (int)(i / tile_rows % 4);
+  const size_t tile = i / (4 * tile_rows);
   const int t = (int)(tile / k_tiles), kt = (int)(tile % k_tiles);
-  const int n = (order ? order[t] : t) * 16 + col, k = 32 * kt + 8 * g;
+  const int n = (order ? order[t] : t) * tile_rows + col, k = 32 * kt + 8 * g;
   *(bf16x8*)(Wt + i * 8) = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero8();
 }
 
-// Wt [ifx_tiled_rows(N) * ifx_tiled_cols(K)] = the tiled form of W [N, K] (K a multiple of 8).  ``order``
-// [ifx_tiled_rows(N) / 16] (or null): row tile t of the copy is row tile order[t] of W (a permutation,
+// Wt [ifx_tiled_size(N, K, tile_rows)] = the tiled form of W [N, K] (K a multiple of 8).  ``order``
+// [ceil(N / tile_rows)] (or null): row tile t of the copy is row tile order[t] of W (a permutation,
 // checked by the caller).
-extern "C" int ifx_tile_weights(const void* W, void* Wt, int N, int K, const int* order, void* stream) {
+extern "C" int ifx_tile_weights(const void* W, void* Wt, int N, int K, const int* order, int tile_rows, void* stream) {
   IFX_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "tile_weights: N=%d K=%d (K must be a multiple of 8)", N, K);
+  IFX_REQUIRE(tile_rows >= 8 && tile_rows <= 16 && tile_rows % 2 == 0, "tile_weights: %d rows to a tile (8 to 16, even)", tile_rows);
   const int k_tiles = ifx_tiled_cols(K) / 32;
-  const size_t pieces = (size_t)(ifx_tiled_rows(N) / 16) * k_tiles * WAVE;
+  const size_t pieces = (size_t)((N + tile_rows - 1) / tile_rows) * k_tiles * 4 * tile_rows;
   hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)W, (bf16_t*)Wt, N, K, k_tiles, pieces, order);
+                     (const bf16_t*)W, (bf16_t*)Wt, N, K, k_tiles, pieces, order, tile_rows);
   IFX_LAUNCH_CHECK();
 }
 
@@ -420,13 +439,16 @@ extern "C" int ifx_qkv_rope(const void* x, const void* Wt, int M, int K, const v
 // epi 2: the product is added to ``stream`` [M, N] (float, in place), rows_out [M, N] = bf16(stream * norm_w) and
 //        pieces_out [ceil(N / 16)][16] = sums of squares of the stream in runs of 16, for the norm that follows
 //        (M <= 16, N a multiple of 4, norm_w bfloat16 [N]); ``out`` is not used.
-// tiled 1: W is the tiled form written by ifx_tile_weights, with the row-tile order it was given (or null).
+// tiled 1 or 16: W is the tiled form written by ifx_tile_weights, with the row-tile order it was given (or null);
+//        8 to 14 (even): that form with so many rows to a tile (no order).
 // scale_pieces [n_scale_pieces][16] (or null), scale_width, scale_eps: a factor per row of x (M <= 16), see RowScale.
 extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K, int nt,
                                int waves, int unroll, int epi, int tiled, const int* order, const float* scale_pieces,
                                int n_scale_pieces, float scale_width, float scale_eps, float* stream_io,
                                const void* norm_w, void* rows_out, float* pieces_out, void* stream) {
-  IFX_REQUIRE(tiled || !order, "skinny_gemm: a tile order goes with a tiled copy");
+  IFX_REQUIRE(tiled == 0 || tiled == 1 || (tiled >= 8 && tiled <= 16 && tiled % 2 == 0), "skinny_gemm: tiled=%d (0, 1, or 8 to 16 rows to a tile)", tiled);
+  const int tile_rows = tiled >= 8 ? tiled : 16;
+  IFX_REQUIRE((tiled && tile_rows == 16) || !order, "skinny_gemm: a tile order goes with a tiled copy of 16-row tiles");
   IFX_REQUIRE(epi == 0 || !order, "skinny_gemm: only the plain epilogue takes a tile order");
   IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0) || (epi == 2 && N % 4 == 0), "skinny_gemm: epilogue %d with N=%d", epi, N);
   IFX_REQUIRE(epi != 2 || (M <= 16 && stream_io && norm_w && rows_out && pieces_out),
@@ -445,23 +467,24 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
     // Measured on the tiled copy (7B shapes, 1-16 rows): two row tiles per wave halve the reads of x and
     // win wherever they leave 128 workgroups or more, except for the tallest weights at 1-4 rows; tall
     // weights want 8 waves per workgroup up to 8 rows of x and one beyond; the others enough waves to
-    // reach about a thousand.
+    // reach fifteen hundred (eight to a workgroup where every compute unit has one).
     const bool tall = N >= 32768;
-    if (nt == 0) nt = tall ? (M <= 4 ? 1 : 2) : ((N + 31) / 32 >= 128 ? 2 : 1);
+    const int n_tiles = (N + tile_rows - 1) / tile_rows;
+    if (nt == 0) nt = tall ? (M <= 4 ? 1 : 2) : ((n_tiles + 1) / 2 >= 128 && tile_rows == 16 ? 2 : 1);
     if (unroll == 0) unroll = (nt == 1 && M <= 4) ? 4 : 2;
     if (waves == 0) {
-      const int groups = (N + 16 * nt - 1) / (16 * nt);
+      const int groups = (n_tiles + nt - 1) / nt;
       waves = 1;
       if (tall) waves = M <= 8 ? 8 : 1;
       else
-        while (waves < 16 && groups * waves < 1024) waves *= 2;
+        while (waves < 16 && groups * waves < 1536) waves *= 2;
       while (waves > 1 && nkb < waves * 2) waves /= 2;
     }
   }
   if (nt == 0) nt = (N >= 32768 && mt <= 2) ? 2 : 1;
   if (unroll == 0) unroll = (mt * nt >= 2) ? 2 : 4;
   if (waves == 0) {
-    const int groups = (N + 16 * nt - 1) / (16 * nt);
+    const int groups = (N + tile_rows * nt - 1) / (tile_rows * nt);
     waves = 1;
     if (groups < 1024)
       while (waves < 16 && groups * waves < 1536 && nkb >= waves * 2) waves *= 2;
@@ -475,8 +498,8 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   const StreamOut so{stream_io, (const bf16_t*)norm_w, (bf16_t*)rows_out, pieces_out};
 #define CASE(MT_, NT_, U_)                                                                                             \
   if (mt == MT_ && nt == NT_ && unroll == U_)                                                                          \
-    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, s)  \
-                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, s)
+    return tiled ? launch<MT_, NT_, U_, true>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, tile_rows, s)  \
+                 : launch<MT_, NT_, U_, false>(x, W, out, out_dtype, M, N, K, k_tiles, waves, epi, order, scale, so, 16, s)
   // (the combinations left out need more than the 128 registers a workgroup of 16 waves leaves a lane)
   CASE(1, 1, 4); CASE(1, 2, 4); CASE(1, 1, 2); CASE(1, 2, 2);
   CASE(2, 1, 4); CASE(2, 2, 2); CASE(2, 1, 2);

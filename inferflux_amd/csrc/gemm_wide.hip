@@ -47,18 +47,20 @@ template <int MT, typename TO, int EPI>
 __global__ __launch_bounds__(MAX_WAVES * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
                                                                      TO* __restrict__ out, float* __restrict__ part, int M,
                                                                      int N, int K, int k_tiles, int rounds_per_slice,
-                                                                     const int* __restrict__ order) {
+                                                                     const int* __restrict__ order, int tile_rows) {
   constexpr int R = MT * 16;                                  // rows of x in LDS
   constexpr int X_PIECES = R * WK_PIECES;                     // 16-byte pieces of a round's x
   constexpr int X_PER_THREAD = (X_PIECES + MIN_WAVES * WAVE - 1) / (MIN_WAVES * WAVE);
   __shared__ __attribute__((aligned(16))) bf16x8 xs[2][X_PIECES];
   const int tid = threadIdx.x, threads = blockDim.x, waves = threads / WAVE;
   const int wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g = lane >> 4;
-  const int tile = blockIdx.x * waves + wid, n_tiles = (N + 15) / 16;
+  const int tile = blockIdx.x * waves + wid, n_tiles = (N + tile_rows - 1) / tile_rows;
   const int n_rounds = (K + WK - 1) / WK;
   const int r_begin = blockIdx.y * rounds_per_slice, n = min(n_rounds, r_begin + rounds_per_slice) - r_begin;
   // a wave whose tile lies past N reads the last tile again and stores nothing
-  const bf16_t* wtile = Wt + ((size_t)min(tile, n_tiles - 1) * k_tiles * WAVE + lane) * 8;
+  // (a tile of the copy holds tile_rows rows, 64 tile_rows bytes per k-tile: see gemm_bf16.hip; the lanes of the other rows hold zeros)
+  const bf16_t* wtile = Wt + ((size_t)min(tile, n_tiles - 1) * k_tiles * 4 * tile_rows + tile_rows * g + col) * 8;
+  const bool row_held = col < tile_rows;
   floatx4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(MAX_WAVES * WAVE) void wide_gemm_kernel(const bf16_
 #pragma unroll
     for (int kt = 0; kt < WK_TILES; ++kt) {
       const int t = r * WK_TILES + kt;
-      w[kt] = t < k_tiles ? __builtin_nontemporal_load((const bf16x8*)(wtile + (size_t)t * WAVE * 8)) : zero8();
+      w[kt] = (t < k_tiles && row_held) ? __builtin_nontemporal_load((const bf16x8*)(wtile + (size_t)t * 4 * tile_rows * 8)) : zero8();
     }
   };
   auto load_x = [&](int r, bf16x8 (&xp)[X_PER_THREAD]) {
@@ -122,8 +124,9 @@ __global__ __launch_bounds__(MAX_WAVES * WAVE) void wide_gemm_kernel(const bf16_
     }
   }
   if (tile >= n_tiles) return;
-  // acc[mt][r] = out[m = 16 mt + col][n = 16 (row tile of the weight) + 4 g + r]
-  const int n0 = 16 * (order ? order[tile] : tile) + 4 * g;
+  // acc[mt][r] = out[m = 16 mt + col][n = tile_rows (row tile of the weight) + 4 g + r], for 4 g + r < tile_rows
+  const int n0 = tile_rows * (order ? order[tile] : tile) + 4 * g;
+  const int held = min(4, tile_rows - 4 * g);      // how many of the lane's four rows the tile holds (even, may be <= 0)
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + col;
@@ -131,16 +134,16 @@ __global__ __launch_bounds__(MAX_WAVES * WAVE) void wide_gemm_kernel(const bf16_
     if (gridDim.y > 1) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (n0 + r < N) part[((size_t)blockIdx.y * M + m) * N + n0 + r] = acc[mt][r];
+        if (r < held && n0 + r < N) part[((size_t)blockIdx.y * M + m) * N + n0 + r] = acc[mt][r];
     } else if (EPI == 0) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (n0 + r < N) out[(size_t)m * N + n0 + r] = from_f<TO>(acc[mt][r]);
+        if (r < held && n0 + r < N) out[(size_t)m * N + n0 + r] = from_f<TO>(acc[mt][r]);
     } else {
 #pragma unroll
       for (int r = 0; r < 4; r += 2) {   // even: gate at n0 + r, up at n0 + r + 1
         const float gt = acc[mt][r], up = acc[mt][r + 1];
-        if (n0 + r + 1 < N) out[(size_t)m * (N / 2) + (n0 + r) / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+        if (r < held && n0 + r + 1 < N) out[(size_t)m * (N / 2) + (n0 + r) / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
       }
     }
   }
@@ -169,8 +172,9 @@ extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S
 // for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
 // several workgroups to a unit; then slices of at least four rounds, at most eight); the gate/up epilogue takes
 // one slice.  Returns waves * 256 + slices.
-extern "C" int ifx_wide_gemm_plan(int N, int K, int waves, int slices, int epi) {
-  const int n_tiles = (N + 15) / 16, n_rounds = (K + WK - 1) / WK;
+extern "C" int ifx_wide_gemm_plan(int N, int K, int waves, int slices, int epi, int tile_rows) {
+  if (tile_rows < 8 || tile_rows > 16) tile_rows = 16;
+  const int n_tiles = (N + tile_rows - 1) / tile_rows, n_rounds = (K + WK - 1) / WK;
   if (waves <= 0) waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
   waves = waves < MIN_WAVES ? MIN_WAVES : (waves > MAX_WAVES ? MAX_WAVES : waves);
   const int groups = (n_tiles + waves - 1) / waves;
@@ -188,13 +192,13 @@ extern "C" int ifx_wide_gemm_plan(int N, int K, int waves, int slices, int epi) 
 
 template <int MT>
 static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K, int waves,
-                       int slices, int rps, int epi, const int* order, bool add_slices, hipStream_t s) {
-  const int n_tiles = (N + 15) / 16;
+                       int slices, int rps, int epi, const int* order, bool add_slices, int tile_rows, hipStream_t s) {
+  const int n_tiles = (N + tile_rows - 1) / tile_rows;
   const dim3 grid((n_tiles + waves - 1) / waves, slices);
   const int k_tiles = (K + 63) / 64 * 2;
 #define GO(TO_, EPI_)                                                                                         \
   hipLaunchKernelGGL((wide_gemm_kernel<MT, TO_, EPI_>), grid, dim3(waves * WAVE), 0, s, (const bf16_t*)x,     \
-                     (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order)
+                     (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order, tile_rows)
   if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
   else if (out_dtype == DT_BF16) GO(bf16_t, 1);
   else if (epi == 0) GO(float, 0);
@@ -212,12 +216,14 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
 // x [M <= 64, K] times the tiled copy Wt of W [N, K], transposed.  ``waves``, ``slices``: as ifx_wide_gemm_plan
 // returned them; ``part``: slices * M * N floats when there is more than one slice.
 // epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2] (one slice, no tile order).
-// order: the row-tile order the copy was written with (or null).
+// order: the row-tile order the copy was written with (or null); tile_rows: the rows to a tile it was written with.
 // ``out`` null with more than one slice: the partial sums are left in ``part`` for a kernel that adds them itself
 // (ifx_add_rmsnorm, ifx_rope_append).
 extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K,
-                             int waves, int slices, int epi, const int* order, void* stream) {
+                             int waves, int slices, int epi, const int* order, int tile_rows, void* stream) {
   IFX_REQUIRE(out || slices > 1, "wide_gemm: no output");
+  IFX_REQUIRE(tile_rows >= 8 && tile_rows <= 16 && tile_rows % 2 == 0 && (tile_rows == 16 || !order),
+              "wide_gemm: %d rows to a tile (8 to 16, even; a tile order goes with 16)", tile_rows);
   IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "wide_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
   IFX_REQUIRE(K % 8 == 0, "wide_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "wide_gemm: unknown out dtype %d", out_dtype);
@@ -232,9 +238,9 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
   IFX_REQUIRE((n_rounds + rps - 1) / rps == slices, "wide_gemm: %d rounds do not cut into %d slices (ask ifx_wide_gemm_plan)", n_rounds, slices);
   hipStream_t s = (hipStream_t)stream;
   switch ((M + 15) / 16) {
-    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
-    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
-    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
-    default: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, s);
+    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    default: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
   }
 }

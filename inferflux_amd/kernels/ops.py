@@ -260,25 +260,47 @@ def pause_library_gemm_tuning(paused: bool) -> None:
         tunable.tuning_enable(not paused)
 
 
-def tile_weights(weight: torch.Tensor, order: Optional[torch.Tensor] = None) -> torch.Tensor:
+def tile_weights(weight: torch.Tensor, order: Optional[torch.Tensor] = None, tile_rows: int = 16) -> torch.Tensor:
     """The tiled form of a bfloat16 ``weight`` [N, K] that the weight-streaming product reads in
-    contiguous kilobytes: a flat tensor of rows16(N) * cols64(K) elements (zeros in the padding).
-    ``order`` (int32, a permutation of the ceil(N / 16) row tiles): tile t of the copy is row tile
-    order[t] of the weight."""
+    contiguous runs: a flat tensor of ceil(N / tile_rows) row tiles of ``tile_rows`` rows (even, 8 to 16) by
+    cols64(K) k-values (zeros in the padding).  ``order`` (int32, a permutation of the row tiles, tiles of 16
+    only): tile t of the copy is row tile order[t] of the weight."""
     _check(weight, "weight", (None, None), torch.bfloat16)
     N, K = weight.shape
     if K % 8:
         raise KernelError(f"tile_weights: K={K} must be a multiple of 8")
+    if tile_rows not in TILE_ROWS or (order is not None and tile_rows != 16):
+        raise KernelError(f"tile_weights: {tile_rows} rows to a tile (one of {TILE_ROWS}; 16 with a tile order)")
     mod = load_module("gemm_bf16")
-    rows16 = mod.fn("ifx_tiled_rows", (I,))(N)
+    n_tiles = -(-N // tile_rows)
     if order is not None:
-        _check(order, "order", (rows16 // 16,), torch.int32)
-        if sorted(order.tolist()) != list(range(rows16 // 16)):
+        _check(order, "order", (n_tiles,), torch.int32)
+        if sorted(order.tolist()) != list(range(n_tiles)):
             raise KernelError("tile_weights: order is not a permutation of the weight's row tiles")
-    size = rows16 * mod.fn("ifx_tiled_cols", (I,))(K)
-    out = torch.empty((size,), dtype=torch.bfloat16, device=weight.device)
-    _call(mod, "ifx_tile_weights", (P, P, I, I, P, P), weight.data_ptr(), out.data_ptr(), N, K, _ptr(order), _stream())
+    out = torch.empty((_tiled_size(N, K, tile_rows),), dtype=torch.bfloat16, device=weight.device)
+    _call(mod, "ifx_tile_weights", (P, P, I, I, P, I, P), weight.data_ptr(), out.data_ptr(), N, K, _ptr(order), tile_rows, _stream())
     return out
+
+
+TILE_ROWS = (8, 10, 12, 14, 16)      # rows a tile of the copy may hold
+COMPUTE_UNITS = 256
+
+
+def _tiled_size(N: int, K: int, tile_rows: int) -> int:
+    return -(-N // tile_rows) * tile_rows * (-(-K // 64) * 64)
+
+
+def choose_tile_rows(N: int) -> int:
+    """Rows to a tile of a weight's streamed copy.  A workgroup of the products for few rows of x owns whole row
+    tiles, and a compute unit can have only so many bytes on their way: a weight of 3,584 rows in tiles of 16
+    gives 224 of the 256 units a tile and takes as long as one of 4,096 rows.  Where 16-row tiles leave units
+    without one, the tiles are made as low as still gives every unit at most one (3,584 rows: 14; 2,048: 8).
+    Measured at 1-64 rows of x: 3,584 x 18,944 takes 24.8 us instead of 25.9 at 8 rows, 2,048 x 11,008 16.3
+    instead of 20.1 at 16 rows; weights with more tiles than units gain nothing from lower tiles or lose."""
+    if N > 16 * COMPUTE_UNITS:
+        return 16
+    rows = -(-N // COMPUTE_UNITS)
+    return min(16, max(8, rows + rows % 2))
 
 
 class LinearWeight:
@@ -287,10 +309,12 @@ class LinearWeight:
     copy doubles the weight's memory; it is left out when ``decode_weight_copy`` is off or when the
     card has no room for it, and products with few rows then read ``rows``."""
 
-    __slots__ = ("rows", "tiled", "order")
+    __slots__ = ("rows", "tiled", "order", "tile_rows")
 
-    def __init__(self, rows: torch.Tensor, tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None):
-        self.rows, self.tiled, self.order = rows, tiled, order   # order: the copy's row-tile order (see tile_weights)
+    def __init__(self, rows: torch.Tensor, tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None,
+                 tile_rows: int = 16):
+        # order: the copy's row-tile order, tile_rows: the rows to a tile of the copy (see tile_weights)
+        self.rows, self.tiled, self.order, self.tile_rows = rows, tiled, order, tile_rows
 
     @property
     def shape(self):
@@ -306,26 +330,30 @@ decode_weight_copy = True
 DECODE_COPY_RESERVE_BYTES = 8 << 30
 
 
-def prepare_linear(weight: torch.Tensor, order: Optional[torch.Tensor] = None) -> LinearWeight:
+def prepare_linear(weight: torch.Tensor, order: Optional[torch.Tensor] = None, tile_rows: int = 0) -> LinearWeight:
     """Wrap a projection's weight for ``linear`` / ``linear_swiglu``, with the tiled copy if wanted and possible
-    (its row tiles in ``order``, if given)."""
+    (its row tiles in ``order``, if given, and then of 16 rows; else of ``tile_rows`` rows, 0: ``choose_tile_rows``)."""
     tiled = None
+    if order is not None:
+        tile_rows = 16
+    elif tile_rows == 0:
+        tile_rows = choose_tile_rows(weight.shape[0]) if weight.dim() == 2 else 16
     if (decode_weight_copy and weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2
             and weight.shape[1] % 8 == 0):
         free, _ = torch.cuda.mem_get_info(weight.device)
         if free >= weight.numel() * 2 + DECODE_COPY_RESERVE_BYTES:
-            tiled = tile_weights(weight.contiguous(), order)
+            tiled = tile_weights(weight.contiguous(), order, tile_rows)
         else:
             log.warn("kernels", f"no room for the decode copy of a {tuple(weight.shape)} weight "
                                 f"({free / 2**30:.1f} GiB free): decoding reads the plain rows")
-    return LinearWeight(weight, tiled, order if tiled is not None else None)
+    return LinearWeight(weight, tiled, order if tiled is not None else None, tile_rows if tiled is not None else 16)
 
 
 class ScaledRows:
     """Rows of a normalised activation up to one factor per row: row t stands for
     ``rows[t] * rsqrt(sum(pieces[:, t]) / width + eps)``.  ``rows`` is bfloat16 [T <= 16, width] (the stream times
-    the norm's weight), ``pieces`` float32 [ceil(width / 16), 16] (sums of squares of the stream in runs of 16; rows
-    past T hold zeros).  A weight-streaming product that takes these multiplies its sums by the factor, which
+    the norm's weight), ``pieces`` float32 [n, 16] (sums of squares of the stream over runs of columns, one run
+    per row tile of the product that made them; rows past T hold zeros).  A weight-streaming product that takes these multiplies its sums by the factor, which
     saves the norm a kernel of its own; ``linear_into_stream`` makes them."""
 
     __slots__ = ("rows", "pieces", "width", "eps", "norm_weight")
@@ -369,7 +397,9 @@ class SliceSums:
 def _scale_args(x):
     """(rows, the four row-factor arguments of the kernels) of a tensor or a ``ScaledRows``."""
     if isinstance(x, ScaledRows):
-        _check(x.pieces, "pieces", (-(-x.width // 16), 16), torch.float32)
+        _check(x.pieces, "pieces", (None, 16), torch.float32)
+        if not 1 <= x.pieces.shape[0] <= x.width:
+            raise KernelError(f"scaled rows: {x.pieces.shape[0]} pieces for a width of {x.width}")
         _check(x.rows, "rows", (None, x.width), torch.bfloat16)
         if x.rows.shape[0] > 16:
             raise KernelError(f"scaled rows: {x.rows.shape[0]} rows, at most 16")
@@ -407,10 +437,11 @@ def linear_into_stream(x: torch.Tensor, weight: LinearWeight, stream: torch.Tens
     _check(stream, "stream", (M, N), torch.float32)
     _check(norm_weight, "norm_weight", (N,), torch.bfloat16)
     rows = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    pieces = torch.empty((-(-N // 16), 16), dtype=torch.float32, device=x.device)
+    tile_rows = 16 if weight.tiled is None else weight.tile_rows
+    pieces = torch.empty((-(-N // tile_rows), 16), dtype=torch.float32, device=x.device)    # one piece per row tile
     w = weight.rows if weight.tiled is None else weight.tiled
     _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
-          x.data_ptr(), w.data_ptr(), 0, DT_F32, M, N, K, 0, 0, 0, 2, 0 if weight.tiled is None else 1, 0,
+          x.data_ptr(), w.data_ptr(), 0, DT_F32, M, N, K, 0, 0, 0, 2, 0 if weight.tiled is None else tile_rows, 0,
           0, 0, 0.0, 0.0, stream.data_ptr(), norm_weight.data_ptr(), rows.data_ptr(), pieces.data_ptr(), _stream())
     return ScaledRows(rows, pieces, N, eps, norm_weight)
 
@@ -461,11 +492,11 @@ def qkv_rope_append(x: torch.Tensor, weight: LinearWeight, bias: Optional[torch.
 
 def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                 nt: int = 0, waves: int = 0, unroll: int = 0, swiglu_pairs: bool = False,
-                tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None) -> torch.Tensor:
+                tiled: Optional[torch.Tensor] = None, order: Optional[torch.Tensor] = None, tile_rows: int = 16) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] times bfloat16 ``weight`` [N, K] transposed on the matrix cores, float
     accumulation, output bfloat16 or float32.  ``nt``, ``waves``, ``unroll`` = 0 lets the kernel choose.
     With ``swiglu_pairs`` the weight's rows alternate gate and up and the output is silu(gate) * up [M, N/2].
-    With ``tiled`` (``tile_weights(weight, order)``) the kernel streams that copy instead of the rows.
+    With ``tiled`` (``tile_weights(weight, order, tile_rows)``) the kernel streams that copy instead of the rows.
     ``x`` may be ``ScaledRows``."""
     x, scale = _scale_args(x)
     _check(x, "x", (None, None), torch.bfloat16)
@@ -473,8 +504,9 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _check(weight, "weight", (None, K), torch.bfloat16)
     N = weight.shape[0]
     if tiled is not None:
-        mod = load_module("gemm_bf16")
-        _check(tiled, "tiled", (mod.fn("ifx_tiled_rows", (I,))(N) * mod.fn("ifx_tiled_cols", (I,))(K),), torch.bfloat16)
+        if tile_rows not in TILE_ROWS or (order is not None and tile_rows != 16):
+            raise KernelError(f"skinny_gemm: {tile_rows} rows to a tile (one of {TILE_ROWS}; 16 with a tile order)")
+        _check(tiled, "tiled", (_tiled_size(N, K, tile_rows),), torch.bfloat16)
     if M > SKINNY_MAX_M or K % 8:
         raise KernelError(f"skinny_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
     if swiglu_pairs and N % 2:
@@ -484,7 +516,7 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         raise KernelError("skinny_gemm: a tile order goes with a tiled copy and a plain product")
     _call(load_module("gemm_bf16"), "ifx_skinny_gemm", _SKINNY_ARGS,
           x.data_ptr(), (weight if tiled is None else tiled).data_ptr(), out.data_ptr(), _DT[out_dtype], M, N, K, nt, waves,
-          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else 1, _ptr(order), *scale, 0, 0, 0, 0, _stream())
+          unroll, 1 if swiglu_pairs else 0, 0 if tiled is None else tile_rows, _ptr(order), *scale, 0, 0, 0, 0, _stream())
     return out
 
 
@@ -504,14 +536,16 @@ def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = to
     if swiglu_pairs and (N % 2 or weight.order is not None):
         raise KernelError("wide_gemm: gate/up pairs need an even number of weight rows in their natural order")
     mod = load_module("gemm_wide")
-    plan = mod.fn("ifx_wide_gemm_plan", (I, I, I, I, I))(N, K, waves, slices, 1 if swiglu_pairs else 0)
+    if _tiled_size(N, K, weight.tile_rows) != weight.tiled.numel():
+        raise KernelError(f"wide_gemm: the copy is not that of a [{N}, {K}] weight in tiles of {weight.tile_rows} rows")
+    plan = mod.fn("ifx_wide_gemm_plan", (I, I, I, I, I, I))(N, K, waves, slices, 1 if swiglu_pairs else 0, weight.tile_rows)
     n_waves, n_slices = plan // 256, plan % 256
     part = torch.empty((n_slices, M, N), dtype=torch.float32, device=x.device) if n_slices > 1 else None
     keep = keep_slices and n_slices > 1
     out = None if keep else torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
-    _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, P),
+    _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, I, P),
           x.data_ptr(), weight.tiled.data_ptr(), _ptr(out), _DT[out_dtype], _ptr(part), M, N, K, n_waves, n_slices,
-          1 if swiglu_pairs else 0, _ptr(weight.order), _stream())
+          1 if swiglu_pairs else 0, _ptr(weight.order), weight.tile_rows, _stream())
     return SliceSums(part, out_dtype) if keep else out
 
 
@@ -549,10 +583,11 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, kee
     always comes from float accumulators, never through a bfloat16 rounding.
     """
     tiled = order = None
+    tile_rows = 16
     if isinstance(x, ScaledRows) and not takes_scaled_rows(x.shape[0], weight):
         raise KernelError(f"linear: scaled rows are not taken for {x.shape[0]} rows and this weight")
     if isinstance(weight, LinearWeight):
-        weight, tiled, order = weight.rows, weight.tiled, weight.order
+        weight, tiled, order, tile_rows = weight.rows, weight.tiled, weight.order, weight.tile_rows
     if weight.dtype == torch.float32:
         return gemm_f32(x, weight, None, out_dtype or x.dtype)
     if weight.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
@@ -563,9 +598,9 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, kee
     M, K = x.shape
     kind = _small_m_kernel(M, weight.shape[0], K, tiled is not None)
     if kind == "skinny":
-        return skinny_gemm(x, weight, out_dtype, tiled=tiled, order=order)
+        return skinny_gemm(x, weight, out_dtype, tiled=tiled, order=order, tile_rows=tile_rows)
     if kind == "wide":
-        return wide_gemm(x, LinearWeight(weight, tiled, order), out_dtype, keep_slices=keep_slices)
+        return wide_gemm(x, LinearWeight(weight, tiled, order, tile_rows), out_dtype, keep_slices=keep_slices)
     if kind == "staged":
         return staged_gemm(x, weight, out_dtype)
     if out_dtype == torch.float32:
@@ -597,13 +632,14 @@ def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
     M, K = x.shape
     if isinstance(x, ScaledRows) and not takes_scaled_rows(M, weight_pairs):
         raise KernelError(f"linear_swiglu: scaled rows are not taken for {M} rows and this weight")
-    rows, tiled = (weight_pairs.rows, weight_pairs.tiled) if isinstance(weight_pairs, LinearWeight) else (weight_pairs, None)
+    rows, tiled, tile_rows = ((weight_pairs.rows, weight_pairs.tiled, weight_pairs.tile_rows) if isinstance(weight_pairs, LinearWeight)
+                              else (weight_pairs, None, 16))
     if isinstance(weight_pairs, LinearWeight) and weight_pairs.order is not None:
         raise KernelError("linear_swiglu: a tile order is not supported for gate/up pairs")
     if rows.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
         kind = _small_m_kernel(M, rows.shape[0], K, tiled is not None)
         if kind == "skinny":
-            return skinny_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, tiled=tiled)
+            return skinny_gemm(x, rows, torch.bfloat16, swiglu_pairs=True, tiled=tiled, tile_rows=tile_rows)
         if kind == "wide":
             return wide_gemm(x, weight_pairs, torch.bfloat16, swiglu_pairs=True)
         if kind == "staged":

@@ -442,22 +442,55 @@ def test_tile_weights_layout():
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K", [(50, 64), (3, 8), (130, 200), (577, 1000), (4608, 3584)])
-def test_skinny_gemm_from_the_tiled_copy_equals_from_rows(M, N, K):
+@pytest.mark.parametrize("tile_rows", [16, 14, 8])
+def test_skinny_gemm_from_the_tiled_copy_equals_from_rows(M, N, K, tile_rows):
     g = gen(16)
     x = torch.randn(M, K, generator=g).to(BF16).to(DEV)
     w = torch.randn(N, K, generator=g).to(BF16).to(DEV)
-    tiled = ops.tile_weights(w)
+    tiled = ops.tile_weights(w, tile_rows=tile_rows)
     want = x.double().cpu() @ w.double().cpu().t()
-    out = ops.skinny_gemm(x, w, F32, tiled=tiled).cpu().double()
+    skinny = ops.skinny_gemm
+    ops_skinny = lambda *a, **kw: skinny(*a, tile_rows=tile_rows, **kw)
+    out = ops_skinny(x, w, F32, tiled=tiled).cpu().double()
     assert torch.allclose(out, want, rtol=1e-4, atol=1e-4 * math.sqrt(K)), float((out - want).abs().max())
     mt = (M + 15) // 16
     for nt, waves, unroll in [(1, 1, 4), (2, 4, 2), (1, 16, 2)]:
         if (mt >= 3 and unroll == 4) or (mt == 4 and nt == 2):     # shapes the kernel is not built for
             with pytest.raises(ops.KernelError, match="no kernel"):
-                ops.skinny_gemm(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled)
+                ops_skinny(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled)
             continue
-        a = ops.skinny_gemm(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled).cpu().double()
+        a = ops_skinny(x, w, F32, nt=nt, waves=waves, unroll=unroll, tiled=tiled).cpu().double()
         assert torch.allclose(a, want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
+    if N % 2 == 0 and M <= 16:                     # gate/up pairs from the same copy
+        pairs = ops_skinny(x, w, F32, swiglu_pairs=True, tiled=tiled).cpu().double()
+        assert torch.allclose(pairs, torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], rtol=1e-4, atol=1e-3 * math.sqrt(K))
+
+
+def test_tiled_copies_of_other_tile_heights():
+    """A tile of p rows is stored as 4 runs of p 16-byte pieces per 32 k-values; p is chosen below 16 where 16-row
+    tiles would leave compute units without a tile; what is not a height, or a height with an order, is refused."""
+    g = gen(21)
+    N, K = 30, 72                                      # K pads to 128: 4 k-tiles
+    w = torch.randn(N, K, generator=g).to(BF16).to(DEV)
+    for p in ops.TILE_ROWS:
+        t = ops.tile_weights(w, tile_rows=p).cpu()
+        n_tiles = -(-N // p)
+        assert t.numel() == n_tiles * p * 128
+        t = t.view(n_tiles, 4, 4, p, 8)                # [row tile][k-tile][group of 8 k][row][8 k-values]
+        full = torch.zeros(n_tiles * p, 128, dtype=BF16)
+        full[:N, :K] = w.cpu()
+        assert torch.equal(t.permute(0, 3, 1, 2, 4).reshape(n_tiles * p, 128), full)
+    assert [ops.choose_tile_rows(n) for n in (3584, 2048, 5120, 37888, 152064, 4096, 3000, 64)] == [14, 8, 16, 16, 16, 16, 12, 8]
+    with pytest.raises(ops.KernelError, match="rows to a tile"):
+        ops.tile_weights(w, tile_rows=7)
+    with pytest.raises(ops.KernelError, match="rows to a tile"):
+        ops.tile_weights(w, torch.arange(3, dtype=torch.int32, device=DEV), tile_rows=10)
+    x = torch.randn(4, K, generator=g).to(BF16).to(DEV)
+    with pytest.raises(ops.KernelError, match="tiled"):
+        ops.skinny_gemm(x, w, F32, tiled=ops.tile_weights(w, tile_rows=10), tile_rows=12)    # not that copy's size
+    lw = ops.prepare_linear(w)
+    assert lw.tile_rows == 8 and ops.prepare_linear(w, tile_rows=12).tile_rows == 12
+    assert ops.prepare_linear(w, torch.tensor([1, 0], dtype=torch.int32, device=DEV)).tile_rows == 16
 
 
 def test_tiled_copy_in_another_row_tile_order():
@@ -526,12 +559,14 @@ def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, 
 @pytest.mark.parametrize("M", [9, 17, 32, 33, 50, 64])
 @pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136)])
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
-def test_wide_gemm(M, N, K, out_dtype):
+@pytest.mark.parametrize("tile_rows", [16, 14, 10])
+def test_wide_gemm(M, N, K, out_dtype, tile_rows):
     g = gen(40)
     x = torch.randn(M, K, generator=g).to(BF16)
     w = (torch.randn(N, K, generator=g) * 0.3).to(BF16)
     want = x.double() @ w.double().t()
-    lw = ops.prepare_linear(w.to(DEV))
+    lw = ops.prepare_linear(w.to(DEV), tile_rows=tile_rows)
+    assert lw.tile_rows == tile_rows
     t = dict(rtol=1e-4, atol=3e-3) if out_dtype == F32 else dict(rtol=1e-2, atol=0.1)
     got = ops.wide_gemm(x.to(DEV), lw, out_dtype).cpu().double()
     assert got.shape == (M, N) and torch.allclose(got, want, **t), float((got - want).abs().max())
@@ -676,34 +711,37 @@ def test_linear_swiglu_pairs(M):
 
 
 def _stream_case(M, N, K, seed, copy):
+    """``copy``: False (the weight's rows) or the rows to a tile of the streamed copy."""
     g = gen(seed)
     x = torch.randn(M, K, generator=g).to(BF16)
     w = (torch.randn(N, K, generator=g) * 0.1).to(BF16)
     stream = torch.randn(M, N, generator=g) * 2.0
     nw = (1 + 0.3 * torch.randn(N, generator=g)).to(BF16)
-    lw = ops.LinearWeight(w.to(DEV), ops.tile_weights(w.to(DEV)) if copy else None)
+    p = 16 if copy in (False, True) else copy
+    lw = ops.LinearWeight(w.to(DEV), ops.tile_weights(w.to(DEV), tile_rows=p) if copy else None, None, p)
     return x, w, stream, nw, lw
 
 
 @pytest.mark.parametrize("M", [1, 7, 16])
 @pytest.mark.parametrize("N,K", [(100, 72), (3584, 512), (36, 1000), (4100, 64)])
-@pytest.mark.parametrize("copy", [False, True])
+@pytest.mark.parametrize("copy", [False, True, 14, 8])
 def test_product_added_to_the_stream_with_the_next_norm_prepared(M, N, K, copy):
     x, w, stream, nw, lw = _stream_case(M, N, K, 30, copy)
+    p = lw.tile_rows
     s = stream.to(DEV)
     got = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), 1e-5)
     want = stream.double() + x.double() @ w.double().t()
     assert torch.allclose(s.cpu().double(), want, rtol=1e-5, atol=1e-5)               # float sums, no rounding of the delta
     assert got.rows.dtype == BF16 and got.width == N
     assert torch.allclose(got.rows.cpu().double(), want * nw.double(), **tol(BF16))   # one rounding
-    assert got.pieces.shape == (-(-N // 16), 16)
-    sq = torch.nn.functional.pad(want ** 2, (0, -N % 16)).reshape(M, -1, 16).sum(-1)   # [M, pieces]
+    assert got.pieces.shape == (-(-N // p), 16)                                        # one piece per row tile of the weight
+    sq = torch.nn.functional.pad(want ** 2, (0, -N % p)).reshape(M, -1, p).sum(-1)     # [M, pieces]
     assert torch.allclose(got.pieces.cpu().double()[:, :M], sq.t(), rtol=1e-5, atol=1e-7)
     assert float(got.pieces[:, M:].abs().max()) == 0.0 if M < 16 else True
 
 
 @pytest.mark.parametrize("M", [1, 5, 16])
-@pytest.mark.parametrize("copy", [False, True])
+@pytest.mark.parametrize("copy", [False, True, 10])
 def test_row_factors_are_applied_by_the_product_that_reads_the_rows(M, copy):
     """The norm's factor per row, applied to sums instead of to the input: the same as norm, then product."""
     H, I, eps = 200, 300, 1e-3
@@ -716,7 +754,7 @@ def test_row_factors_are_applied_by_the_product_that_reads_the_rows(M, copy):
     assert torch.allclose(rows * factor, normed, **tol(BF16))
     g = gen(32)
     w2 = (torch.randn(I, H, generator=g) * 0.2).to(BF16)
-    lw2 = ops.LinearWeight(w2.to(DEV), ops.tile_weights(w2.to(DEV)) if copy else None)
+    lw2 = ops.LinearWeight(w2.to(DEV), ops.tile_weights(w2.to(DEV), tile_rows=lw.tile_rows) if copy else None, None, lw.tile_rows)
     assert ops.takes_scaled_rows(M, lw2) and not ops.takes_scaled_rows(17, lw2)
     got = ops.linear(scaled, lw2).cpu().double()
     assert torch.allclose(got, (rows @ w2.double().t()) * factor, **tol(BF16))         # same rounded inputs: one rounding
