@@ -19,10 +19,11 @@ IFX_DEFINE_LAST_ERROR()
 template <typename T>
 __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
                                  float* __restrict__ out, int H) {
-  const int t = blockIdx.x;
+  // (a row is cut into runs of 4,096 columns, one workgroup each: rows as wide as a vocabulary then fill the chip too)
+  const int t = blockIdx.x, i0 = blockIdx.y * 4096, i1 = min(H, i0 + 4096);
   const T* src = table + (size_t)ids[t] * H;
   float* dst = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f(src[i]);
+  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) dst[i] = to_f(src[i]);
 }
 
 extern "C" int ifx_embedding(const int* ids, const void* table, int table_dtype, float* out, int T,
@@ -31,9 +32,9 @@ extern "C" int ifx_embedding(const int* ids, const void* table, int table_dtype,
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (table_dtype == DT_F32)
-    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T), dim3(256), 0, s, ids, (const float*)table, out, H);
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T, (H + 4095) / 4096), dim3(256), 0, s, ids, (const float*)table, out, H);
   else if (table_dtype == DT_BF16)
-    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids, (const bf16_t*)table, out, H);
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T, (H + 4095) / 4096), dim3(256), 0, s, ids, (const bf16_t*)table, out, H);
   else
     IFX_FAIL("embedding: unknown dtype %d", table_dtype);
   IFX_LAUNCH_CHECK();

@@ -32,6 +32,9 @@ def test_embedding(dtype):
     ids = torch.tensor([0, 76, 5, 5, 33], dtype=torch.int32)
     out = ops.embedding(ids.to(DEV), table.to(DEV))
     assert out.dtype == F32 and torch.equal(out.cpu(), table.float()[ids.long()])
+    wide = torch.randn(6, 9001, generator=g).to(dtype)              # rows of more than one run of 4,096 columns
+    pick = torch.tensor([5, 0, 3], dtype=torch.int32)
+    assert torch.equal(ops.embedding(pick.to(DEV), wide.to(DEV)).cpu(), wide.float()[pick.long()])
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
