@@ -85,6 +85,38 @@ def test_steps_got_ready_and_started_ahead_change_no_token_and_are_used(model_fo
     assert [o.token_ids for o in run(stop)] == [o.token_ids for o in stopped]
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_more_requests_than_slots_with_limits_stops_and_few_pages(seed, model_folders):
+    """Requests come in as others finish, each with its own limit, some stopping on a token, with so few pages that
+    some are preempted: in float32 every request's tokens are those of the plain model whether steps are started
+    early or not (rows dropped from a step, steps made void by an arrival and computed afresh)."""
+    folder, V = model_folders["C"], TINY["C"]["vocab_size"]
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(2, 60, 14).tolist()
+    limits = rng.integers(1, 28, 14).tolist()
+    prompts = [seeded_ids(300 + 20 * seed + i, n, V) for i, n in enumerate(lens)]
+    want = [plain_greedy(folder, p, n) for p, n in zip(prompts, limits)]
+    stops = {i: [want[i][len(want[i]) // 2]] for i in range(0, 14, 3) if len(want[i]) > 3}    # stop half-way (or earlier)
+    for i, st in stops.items():
+        want[i] = want[i][: want[i].index(st[0]) + 1]
+
+    def run(early, pages):
+        eng = Engine.load(folder, dtype="float32", kv_pages=pages, max_batch_size=4, chunked_prefill_tokens=16,
+                          start_steps_early=early)
+        params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True, stop_token_ids=stops.get(i, ()))
+                  for i, n in enumerate(limits)]
+        outs = eng.generate(prompts, params)
+        eng.runner.manager.check()
+        assert eng.runner.manager.free_pages() == [pages] * len(eng.runner.manager.groups)
+        return [o.token_ids for o in outs], eng.stats.preemptions
+
+    for early in (True, False):
+        got, _ = run(early, 64)
+        assert got == want
+    got, preempted = run(True, 9)                          # four requests of up to 87 tokens need up to 24 pages
+    assert got == want and preempted >= 1
+
+
 def _count(taken, ctx):
     taken.append(ctx is not None)
     return ctx
