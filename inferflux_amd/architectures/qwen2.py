@@ -45,7 +45,7 @@ def qwen2_plan(cfg: Qwen2Config) -> ModelPlan:
         lm_head=PartSpec("linear_head", {
             "name": "lm_head", "vocab_size": cfg.vocab_size,
             "tied_to": "model.embed_tokens.weight" if cfg.tie_word_embeddings else None}),
-        eos_token_id=cfg.eos_token_id,
+        eos_token_ids=tuple(cfg.eos_token_id),
     )
 
 

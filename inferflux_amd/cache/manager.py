@@ -180,6 +180,10 @@ class CacheManager:
         self._slot: Dict[Hashable, int] = {}        # live request -> its slot, which is how the native side knows it
         self._need = (ctypes.c_int * max(len(counts), 1))()
         self._fail = (ctypes.c_int * 3)()
+        # Called with the slot of every request that is added, whoever adds it (the runner for a replayed
+        # trace, the scheduler for an admission or a re-admission after preemption): the storage hangs the
+        # clearing of per-request state here, so that no path can hand out a slot with its last owner's state.
+        self.on_add = None
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -200,6 +204,8 @@ class CacheManager:
         if slot < 0:
             raise OutOfSlots(f"all {self.max_requests} request slots are in use")
         self._slot[rid] = slot
+        if self.on_add is not None:
+            self.on_add(slot)
         return slot
 
     def _slot_of(self, rid: Hashable) -> int:

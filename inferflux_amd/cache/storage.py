@@ -69,6 +69,8 @@ class CacheStorage:
             st = m.state_spec()
             if st is not None:
                 self._states[i] = torch.zeros((max_requests, *st.shape), dtype=_STATE_DTYPES[st.dtype], device=device)
+        if self._states:
+            self.manager.on_add = self.reset_state       # every admission path starts a request with zero state
         self._bindings: List[MixerBinding] = []
         for i, e in enumerate(schedule):
             owner = i if e.cache_from is None else e.cache_from

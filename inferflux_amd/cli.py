@@ -5,7 +5,8 @@ engine probe (tests/tools/first_token_probe.cpp:38-126: --model, --prompt / --pr
 The reference's inferctl talks to a server; this one drives the engine in the same process.
 
     inferctl completion --model DIR --prompt-ids 1,2,3 --max-tokens 16 [--stream]
-    inferctl random-weights --config config.json --out DIR --seed 0
+    inferctl completion --random-weights config.json --seed 0 --prompt-ids 1,2,3
+    inferctl random-weights --config config.json --out DIR --seed 0 [--shards N]
     inferctl inspect --model DIR
 """
 from __future__ import annotations
@@ -34,14 +35,16 @@ def _read_ids(args) -> List[List[int]]:
     if texts:
         tok = _tokenizer(args.model)
         if tok is None:
-            raise SystemExit(f"--prompt needs {args.model}/tokenizer.json; pass token ids with --prompt-ids instead")
+            raise SystemExit(f"--prompt needs tokenizer.json in the model folder ({args.model}); pass token ids with --prompt-ids instead")
         prompts += [tok.encode(t).ids for t in texts]
     if not prompts:
         raise SystemExit("--prompt-ids, --prompt-ids-file or --prompt is required")
     return prompts
 
 
-def _tokenizer(folder: str):
+def _tokenizer(folder: Optional[str]):
+    if not folder:
+        return None
     path = os.path.join(folder, "tokenizer.json")
     if not os.path.isfile(path):
         return None
@@ -49,18 +52,30 @@ def _tokenizer(folder: str):
     return Tokenizer.from_file(path)
 
 
+def load_spec_from_args(args):
+    """The ``ModelLoadSpec`` the options of ``completion`` describe (a complaint about them ends the program)."""
+    from .engine.load_spec import LoadSpecError, ModelLoadSpec
+    try:
+        return ModelLoadSpec(path=args.model, random_weights=args.random_weights, seed=args.seed, dtype=args.dtype,
+                             device=args.device, context_size=args.ctx_size, max_parallel_sequences=args.max_parallel_sequences,
+                             kv_pages=args.kv_pages, page_size=args.page_size, max_batch_tokens=args.batch_size,
+                             chunked_prefill_tokens=args.chunked_prefill_tokens,
+                             decode_weight_copy=not args.no_decode_weight_copy,
+                             strict_weights=not args.allow_unused_tensors, phase_timing=args.phase_timing).checked()
+    except LoadSpecError as e:
+        raise SystemExit(f"inferctl: {e}")
+
+
 def cmd_completion(args) -> int:
     from . import SamplingParams
     from .engine.engine import Engine
+    spec = load_spec_from_args(args)
     prompts = _read_ids(args)
-    engine = Engine.load(args.model, dtype=args.dtype, kv_pages=args.kv_pages, ctx_size=args.ctx_size,
-                         max_batch_size=args.max_parallel_sequences, max_batch_tokens=args.batch_size,
-                         chunked_prefill_tokens=args.chunked_prefill_tokens, phase_timing=args.phase_timing,
-                         decode_weight_copy=not args.no_decode_weight_copy)
+    engine = Engine.load(spec)
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p,
                             frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
                             repetition_penalty=args.repetition_penalty, penalty_last_n=args.penalty_last_n,
-                            seed=args.seed if args.seed is not None else 0xFFFFFFFF, max_tokens=args.max_tokens,
+                            seed=args.sample_seed if args.sample_seed is not None else 0xFFFFFFFF, max_tokens=args.max_tokens,
                             ignore_eos=args.ignore_eos, logprobs=args.top_n)
     tok = _tokenizer(args.model)
 
@@ -70,7 +85,7 @@ def cmd_completion(args) -> int:
 
     outs = engine.generate(prompts, params, on_token)
     for o in outs:
-        rec = {"model": args.model, "request": o.request_id, "prompt_tokens": len(o.prompt_token_ids),
+        rec = {"model": args.model or args.random_weights, "request": o.request_id, "prompt_tokens": len(o.prompt_token_ids),
                "completion_tokens": len(o.token_ids), "token_ids": o.token_ids, "finish_reason": o.finish_reason}
         if o.logprobs is not None:
             rec["logprobs"] = [{"token": l.token_id, "logprob": round(l.logprob, 6),
@@ -90,8 +105,9 @@ def cmd_random_weights(args) -> int:
     from .weights import write_random_model
     with open(args.config) as f:
         cfg = config_from_dict(json.load(f))
-    write_random_model(args.out, cfg, args.seed, {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype])
-    print(json.dumps({"written": args.out, "seed": args.seed, "dtype": args.dtype}))
+    write_random_model(args.out, cfg, args.seed, {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype],
+                       shards=args.shards)
+    print(json.dumps({"written": args.out, "seed": args.seed, "dtype": args.dtype, "shards": args.shards}))
     return 0
 
 
@@ -113,7 +129,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap = argparse.ArgumentParser(prog="inferctl", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="command", required=True)
     c = sub.add_parser("completion", help="generate tokens for one or more prompts")
-    c.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    c.add_argument("--model", help="folder with config.json and model.safetensors (or its shards and their index)")
+    c.add_argument("--random-weights", metavar="CONFIG_JSON",
+                   help="instead of --model: make seeded random weights for the model this config.json describes")
+    c.add_argument("--seed", type=int, default=0, help="seed of --random-weights")
     c.add_argument("--prompt", action="append", help="text (needs tokenizer.json in the model folder)")
     c.add_argument("--prompt-file")
     c.add_argument("--prompt-ids", action="append", help="comma-separated token ids; may be given several times")
@@ -128,7 +147,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     c.add_argument("--presence-penalty", type=float, default=0.0)
     c.add_argument("--repetition-penalty", type=float, default=1.0)
     c.add_argument("--penalty-last-n", type=int, default=64)
-    c.add_argument("--seed", type=int, default=None)
+    c.add_argument("--sample-seed", type=int, default=None, help="seed of the sampler's draws (default: a fresh one per request)")
     c.add_argument("--ignore-eos", action="store_true")
     c.add_argument("--top-n", type=int, default=None,
                    help="report each token's log-probability with the N most probable alternatives (0: the token's only)")
@@ -137,7 +156,11 @@ def main(argv: Optional[List[str]] = None) -> int:
     c.add_argument("--batch-size", type=int, default=16384, help="most tokens in one step (max_batch_tokens)")
     c.add_argument("--max-parallel-sequences", type=int, default=32, help="most requests in one step (max_batch_size)")
     c.add_argument("--chunked-prefill-tokens", type=int, default=512)
-    c.add_argument("--kv-pages", type=int, default=None, help="pages of 16 tokens in the cache (overrides --ctx-size)")
+    c.add_argument("--kv-pages", type=int, default=None, help="pages in the cache (overrides --ctx-size)")
+    c.add_argument("--page-size", type=int, default=16, help="tokens per page of the cache")
+    c.add_argument("--device", default=None, help="rocm:N or cuda:N (the same ordinal); default: the current device")
+    c.add_argument("--allow-unused-tensors", action="store_true",
+                   help="tensors in the file that the model does not read are a warning instead of an error")
     c.add_argument("--no-decode-weight-copy", action="store_true",
                    help="keep one copy of the weights only (saves their size in memory, decoding is slower)")
     c.add_argument("--phase-timing", action="store_true",
@@ -148,6 +171,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     r.add_argument("--out", required=True)
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    r.add_argument("--shards", type=int, default=1, help="write this many safetensors files and an index")
     r.set_defaults(fn=cmd_random_weights)
     i = sub.add_parser("inspect", help="print a model folder's config and check its tensors against it")
     i.add_argument("--model", required=True)

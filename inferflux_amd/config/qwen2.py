@@ -42,7 +42,7 @@ class Qwen2Config(ModelConfig):
     max_window_layers: int = 0
     hidden_act: str = "silu"
     torch_dtype: str = "bfloat16"
-    eos_token_id: Optional[int] = None
+    eos_token_id: Tuple[int, ...] = ()      # config.json gives one id or a list; every one of them ends a request
     bos_token_id: Optional[int] = None
 
     model_type: ClassVar[str] = "qwen2"
@@ -69,8 +69,9 @@ class Qwen2Config(ModelConfig):
         if rope_scaling not in (None, {}):
             raise ConfigError(f"config.json: 'rope_scaling' = {rope_scaling!r} is not supported (only null)")
         eos = d.get("eos_token_id")
-        if isinstance(eos, list):
-            eos = eos[0] if eos else None
+        eos = [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+        if any(isinstance(e, bool) or not isinstance(e, int) or e < 0 for e in eos):
+            raise ConfigError(f"config.json: 'eos_token_id' must be a token id or a list of them, got {d.get('eos_token_id')!r}")
         cfg = cls(
             vocab_size=read_key(d, "vocab_size", int),
             hidden_size=hidden,
@@ -89,11 +90,17 @@ class Qwen2Config(ModelConfig):
             max_window_layers=read_key(d, "max_window_layers", int, 0),
             hidden_act=read_key(d, "hidden_act", str, "silu"),
             torch_dtype=read_key(d, "torch_dtype", str, "bfloat16"),
-            eos_token_id=eos if isinstance(eos, int) and not isinstance(eos, bool) else None,
+            eos_token_id=tuple(dict.fromkeys(eos)),
             bos_token_id=read_key(d, "bos_token_id", int, None),
         )
         cfg.validate()
         return cfg
+
+    def to_dict(self):
+        out = super().to_dict()
+        eos = list(self.eos_token_id)       # as config.json files spell it: null, one id, or a list
+        out["eos_token_id"] = None if not eos else (eos[0] if len(eos) == 1 else eos)
+        return out
 
     def validate(self) -> None:
         def positive(name):
@@ -109,6 +116,8 @@ class Qwen2Config(ModelConfig):
                 f"num_key_value_heads {self.num_key_value_heads}")
         if self.head_dim % 2:
             raise ConfigError(f"config.json: head_dim {self.head_dim} must be even (rotary pairs)")
+        if any(e >= self.vocab_size for e in self.eos_token_id):
+            raise ConfigError(f"config.json: eos_token_id {list(self.eos_token_id)} outside the vocabulary of {self.vocab_size}")
         if not (self.rope_theta > 0):
             raise ConfigError(f"config.json: rope_theta must be positive, got {self.rope_theta}")
         if not (self.rms_norm_eps >= 0):

@@ -7,6 +7,7 @@ import torch
 
 from ..config.registry import load_config
 from ..kernels import ops
+from .load_spec import ModelLoadSpec
 from .model import Model
 from .runner import ModelRunner
 
@@ -17,20 +18,36 @@ def require_gpu() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device())
 
 
-def load_model(folder: str, dtype: torch.dtype = torch.bfloat16, device=None, decode_weight_copy: bool = True) -> Model:
+def load_model(folder, dtype: torch.dtype = torch.bfloat16, device=None, decode_weight_copy: bool = True,
+               strict_weights: bool = True) -> Model:
     """The model class is chosen by config.json; weights are read by tensor name.  With
     ``decode_weight_copy`` every bfloat16 projection also keeps the tiled copy that products with few
-    rows stream from (twice the weights' memory for about a fifth off a decode step)."""
+    rows stream from (twice the weights' memory for about a fifth off a decode step).  ``folder`` may be
+    a ``ModelLoadSpec`` (then the other arguments are taken from it, and a spec that names ``random_weights``
+    gets them made on the device, seeded, with no folder written)."""
+    spec = folder if isinstance(folder, ModelLoadSpec) else ModelLoadSpec(
+        path=folder, dtype={torch.bfloat16: "bfloat16", torch.float32: "float32"}[dtype],
+        decode_weight_copy=decode_weight_copy, strict_weights=strict_weights)
+    spec.checked()
+    if isinstance(folder, ModelLoadSpec):
+        dtype = spec.torch_dtype
+        if spec.device_index is not None:
+            device = torch.device("cuda", spec.device_index)
     device = device or require_gpu()
     if dtype == torch.float32:
         # The 32-bit path never uses a reduced-precision matrix mode; the engine's own float32
         # kernels do not consult these switches, they are set for any library call a part makes.
         torch.backends.cuda.matmul.allow_tf32 = False
-    config = load_config(folder)
     before = ops.decode_weight_copy
-    ops.decode_weight_copy = bool(decode_weight_copy)
+    ops.decode_weight_copy = bool(spec.decode_weight_copy)
     try:
-        return Model(config).load_folder(folder, dtype, device)
+        if spec.random_weights:
+            import json
+            from ..config.registry import config_from_dict
+            with open(spec.random_weights) as f:
+                config = config_from_dict(json.load(f))
+            return Model(config).init_random(spec.seed, dtype, device)
+        return Model(load_config(spec.path)).load_folder(spec.path, dtype, device, strict=spec.strict_weights)
     finally:
         ops.decode_weight_copy = before
 
@@ -57,10 +74,20 @@ def plan_kv_pages(model: Model, page_size: int, wanted_tokens: int, memory_fract
     return min(want, fit)
 
 
-def load_runner(folder: str, dtype: torch.dtype = torch.bfloat16, num_pages: Optional[int] = 256, page_size: int = 16,
+def load_runner(folder, dtype: torch.dtype = torch.bfloat16, num_pages: Optional[int] = 256, page_size: int = 16,
                 max_requests: int = 64, device=None, cache_tokens: Optional[int] = None,
                 phase_timing: bool = False, decode_weight_copy: bool = True) -> ModelRunner:
-    """``num_pages`` None: as many pages as ``cache_tokens`` need, within the free device memory."""
+    """A model with its cache and step function.  ``folder`` is a ``ModelLoadSpec`` (every other argument is then
+    taken from it) or a model folder with the arguments given here.  ``num_pages`` None: as many pages as
+    ``cache_tokens`` need, within the free device memory."""
+    if isinstance(folder, ModelLoadSpec):
+        spec = folder.checked()
+        model = load_model(spec)
+        num_pages = spec.kv_pages
+        if num_pages is None:
+            num_pages = plan_kv_pages(model, spec.page_size, spec.cache_tokens)
+        return ModelRunner(model, num_pages=num_pages, page_size=spec.page_size, max_requests=spec.max_parallel_sequences,
+                           phase_timing=spec.phase_timing)
     model = load_model(folder, dtype, device, decode_weight_copy)
     if num_pages is None:
         num_pages = plan_kv_pages(model, page_size, cache_tokens or 4096 * max_requests)

@@ -19,6 +19,7 @@ from .. import log
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler, SamplingState
 from .api import load_runner
+from .load_spec import ModelLoadSpec
 from .context import StepEntry
 from .runner import ModelRunner
 from .scheduler import RequestRefused, Scheduler, SchedulerConfig, Sequence_
@@ -65,30 +66,37 @@ class Engine:
         self.config.max_batch_size = min(self.config.max_batch_size, runner.manager.max_requests)
         self.scheduler = Scheduler(runner.manager, self.config, runner.max_position)
         self.sampler = Sampler(runner.device)
-        self.eos_token_id = runner.model.plan.eos_token_id
+        self.eos_token_ids = frozenset(runner.model.plan.eos_token_ids)
         self._live: Dict[Hashable, _Live] = {}
         self._next_id = 0
         self.stats = EngineStats()
 
     @classmethod
-    def load(cls, model: str, dtype: str = "bfloat16", kv_pages: Optional[int] = None, page_size: int = 16,
+    def load(cls, model, dtype: str = "bfloat16", kv_pages: Optional[int] = None, page_size: int = 16,
              max_batch_size: int = 32, max_batch_tokens: int = 16384, chunked_prefill_tokens: int = 512,
              ctx_size: int = 4096, phase_timing: bool = False, decode_weight_copy: bool = True,
              start_steps_early: bool = True) -> "Engine":
-        """``kv_pages`` None sizes the cache for ``ctx_size`` tokens for each of ``max_batch_size``
-        requests, within the device memory that is free once the weights are loaded.
-        ``decode_weight_copy`` False saves the second, tiled copy of the weights at the price of slower decoding."""
-        dt = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}[dtype]
-        runner = load_runner(model, dt, num_pages=kv_pages, page_size=page_size, max_requests=max_batch_size,
-                             cache_tokens=ctx_size * max_batch_size, phase_timing=phase_timing,
-                             decode_weight_copy=decode_weight_copy)
-        log.info("engine", "model loaded", model=model, dtype=dtype, kv_pages=runner.manager.pools[0].num_pages
-                 if runner.manager.pools else 0, page_size=page_size, max_batch_size=max_batch_size)
-        return cls(runner, SchedulerConfig(max_batch_size, max_batch_tokens, chunked_prefill_tokens), start_steps_early)
+        """``model`` is a ``ModelLoadSpec``, or a model folder with the other arguments standing for the spec's
+        fields (``max_batch_size`` = max_parallel_sequences, ``ctx_size`` = context_size).  ``kv_pages`` None sizes
+        the cache for ``ctx_size`` tokens for each of ``max_batch_size`` requests, within the device memory that is
+        free once the weights are loaded.  ``decode_weight_copy`` False saves the second, tiled copy of the weights
+        at the price of slower decoding."""
+        spec = model if isinstance(model, ModelLoadSpec) else ModelLoadSpec(
+            path=model, dtype=dtype, kv_pages=kv_pages, page_size=page_size, max_parallel_sequences=max_batch_size,
+            max_batch_tokens=max_batch_tokens, chunked_prefill_tokens=chunked_prefill_tokens, context_size=ctx_size,
+            phase_timing=phase_timing, decode_weight_copy=decode_weight_copy)
+        runner = load_runner(spec.checked())
+        log.info("engine", "model loaded", model=spec.path or spec.random_weights, dtype=spec.dtype,
+                 kv_pages=runner.manager.pools[0].num_pages if runner.manager.pools else 0, page_size=spec.page_size,
+                 max_batch_size=spec.max_parallel_sequences)
+        return cls(runner, SchedulerConfig(spec.max_parallel_sequences, spec.max_batch_tokens, spec.chunked_prefill_tokens),
+                   start_steps_early)
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
-                    request_id: Optional[Hashable] = None) -> Hashable:
+                    request_id: Optional[Hashable] = None, priority: int = 0) -> Hashable:
+        """Queue a request; it joins the running batch at the next ``step`` that has room for it.  ``priority``:
+        higher is admitted earlier and preempted later (equal priorities: first come first served)."""
         params = params or SamplingParams()
         params.validate()
         prompt = [int(t) for t in prompt_token_ids]
@@ -98,7 +106,7 @@ class Engine:
         if request_id is None:
             request_id = self._next_id
             self._next_id += 1
-        seq = self.scheduler.add(request_id, prompt, params.max_tokens)
+        seq = self.scheduler.add(request_id, prompt, params.max_tokens, priority)
         self._live[request_id] = _Live(seq, params, prompt)
         self.stats.prompt_tokens += len(prompt)
         return request_id
@@ -116,7 +124,7 @@ class Engine:
     # ---- one step -------------------------------------------------------------------
     def _finish_reason(self, live: _Live, token: int) -> Optional[str]:
         p = live.params
-        if not p.ignore_eos and self.eos_token_id is not None and token == self.eos_token_id:
+        if not p.ignore_eos and token in self.eos_token_ids:
             return "stop"
         if token in p.stop_token_ids:
             return "stop"
@@ -149,9 +157,9 @@ class Engine:
             staying = [i.seq.rid for i in plan.items if len(i.seq.generated) + 1 < self._live[i.seq.rid].params.max_tokens]
             early = self.start_steps_early and self.runner.starts_steps_early and bool(staying)
 
-            def ahead(chosen):
+            def ahead(chosen, host_tokens):
                 if early:
-                    if self.runner.prepare_decode(everyone) and self.runner.launch_prepared(chosen):
+                    if self.runner.prepare_decode(everyone) and self.runner.launch_prepared(chosen, host_tokens):
                         return
                     if len(staying) == len(everyone):
                         return                      # what was got ready stands

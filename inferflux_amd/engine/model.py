@@ -74,16 +74,22 @@ class Model:
         self.dtype, self.device = dtype, torch.device(device)
         return self
 
-    def load_folder(self, folder: str, dtype: torch.dtype, device) -> "Model":
-        return self.bind(load_weights(folder, self.param_specs(), dtype, device), dtype, device)
+    def load_folder(self, folder: str, dtype: torch.dtype, device, strict: bool = True) -> "Model":
+        return self.bind(load_weights(folder, self.param_specs(), dtype, device, strict=strict), dtype, device)
 
-    def init_random(self, seed: int, dtype: torch.dtype, device) -> "Model":
-        """Random weights made on the device, tensor by tensor (for sizes whose folder would take
-        long to write).  Values follow each spec's rule, rounded to bfloat16 in both modes so the
-        two modes see the same numbers."""
+    def init_random(self, seed: int, dtype: torch.dtype, device, on_host: Optional[bool] = None) -> "Model":
+        """Random weights without a folder.  Values follow each spec's rule, rounded to bfloat16 in both modes
+        so the two modes see the same numbers.  ``on_host`` True draws them with the host's generator, tensor by
+        tensor, which gives exactly the values ``write_random_model`` writes for the same seed; False draws them
+        on the device (another stream of numbers, but no minutes of waiting for billions of weights).  None: on
+        the host for models of up to 2**28 weights."""
+        import math
+        specs = self.param_specs()
+        if on_host is None:
+            on_host = sum(math.prod(s.shape) for s in specs.values()) <= (1 << 28)
         tensors = {}
-        for n, s in self.param_specs().items():
-            t = random_tensor(n, s, seed, torch.bfloat16, device=device)
+        for n, s in specs.items():
+            t = random_tensor(n, s, seed, torch.bfloat16, device="cpu" if on_host else device).to(device)
             tensors[n] = t if (dtype == torch.bfloat16 or s.integer) else t.float()
         return self.bind(tensors, dtype, device)
 

@@ -72,8 +72,7 @@ class ModelRunner:
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, rid: Hashable) -> None:
-        slot = self.manager.add(rid)
-        self.storage.reset_state(slot)
+        self.manager.add(rid)          # (the storage clears the slot's per-request state as the manager hands it out)
 
     def free_request(self, rid: Hashable) -> None:
         self.manager.free(rid)
@@ -132,14 +131,15 @@ class ModelRunner:
         """Whether ``launch_prepared`` can ever start a step (graphs are on and no mixer keeps state of its own)."""
         return self.decode_graphs and not self.storage.has_state
 
-    def launch_prepared(self, tokens: torch.Tensor) -> bool:
+    def launch_prepared(self, tokens: torch.Tensor, host_tokens: Optional[torch.Tensor] = None) -> bool:
         """Start the step ``prepare_decode`` got ready, now, with its tokens taken on the GPU from ``tokens`` (int32,
         one per request of that step, in its order: the sampler's output for the step before), so that the GPU goes
         on while the host reads those tokens and does its bookkeeping.  ``step`` hands out the logits if it is then
-        given these requests with one token each (it trusts that they are the tokens of ``tokens``), or a part of
-        them in the same order (the others' rows are dropped: a request that has just stopped).  Any other step
-        makes it void and is computed afresh; keys and values written early are written again with the same
-        contents, which is why nothing is started early for a model whose mixers keep state of their own.
+        given these requests with one token each, the very tokens of ``tokens``, or a part of them in the same
+        order (the others' rows are dropped: a request that has just stopped).  ``host_tokens`` is a host copy of
+        ``tokens`` that is complete by the time ``step`` is called (the sampler's pinned one); without it a copy
+        is made here.  Any other step, or other tokens, makes the early step void and is computed afresh; keys and values written early are written again, which is
+        why nothing is started early for a model whose mixers keep state of their own.
         Returns False, the prepared step kept for ``step``, when it cannot (no captured graph of this layout yet)."""
         prep = self._prepared
         if prep is None or self.storage.has_state:
@@ -152,23 +152,33 @@ class ModelRunner:
         self._replay_inputs(g, ctx)
         g.ctx.token_ids.copy_(tokens)          # (the copy above brought placeholder tokens; both precede the graph on the stream)
         g.graph.replay()
-        self._launched = (snapshot, g)
+        copied = None
+        if host_tokens is None:
+            host_tokens = torch.empty(tokens.shape, dtype=torch.int32, pin_memory=True).copy_(tokens, non_blocking=True)
+            copied = torch.cuda.Event()
+            copied.record()
+        self._launched = (snapshot, g, host_tokens, copied)
         return True
 
     def _take_launched(self, entries):
         """The logits of the step started early, if ``entries`` are its requests or a part of them; else None."""
-        (snapshot, g), self._launched = self._launched, None
+        (snapshot, g, host_tokens, copied), self._launched = self._launched, None
         if any(len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0 for e in entries):
             return None
+        if copied is not None:
+            copied.synchronize()
+        started_with = host_tokens.tolist()                 # the tokens the early step ran on
         rids, was = [e.rid for e in entries], snapshot[0]
         if len(rids) == len(was):
-            if not self.manager.unchanged(snapshot, rids):
+            if [int(e.tokens[0]) for e in entries] != started_with or not self.manager.unchanged(snapshot, rids):
                 return None
             self.manager.commit_each(rids, 1)
             return g.logits
         place = {r: i for i, r in enumerate(was)}
         rows = [place.get(r, -1) for r in rids]
         if min(rows) < 0 or any(a >= b for a, b in zip(rows, rows[1:])):
+            return None
+        if [int(e.tokens[0]) for e in entries] != [started_with[i] for i in rows]:
             return None
         if not self.manager.unchanged(self.manager.snapshot_rows(snapshot, rows), rids):
             return None

@@ -18,12 +18,23 @@ recently admitted running request is preempted: its pages are given back and it 
 front of the waiting queue with prompt + generated tokens as its new prompt (recomputation).
 A request that could never fit the pool alone, or whose prompt + max_tokens exceeds the model's
 positions, is refused when it is added (the reference: context_overflow, scheduler.cpp:2303-2324).
+
+Order of admission.  The reference sorts its queues by a score, priority + age_ms / 2000, ties by
+arrival (scheduler/batch_selection_policy.cpp:10-20; scheduler/scheduler.cpp:2013-2031).  Here a
+request carries a ``priority`` (0 unless given) and the scheduler a ``score`` function of the
+waiting request; the waiting request with the highest score is admitted next, the earlier arrival
+among equals.  The default score is the priority alone, which is first come first served while
+nobody sets one; ``priority_age_score`` is the reference's.  The best-scoring request that does
+not fit blocks those behind it (no overtaking by smaller requests, hence no starvation).  When
+pages run out the victim is the running request of lowest priority, the most recently admitted
+among those.
 """
 from __future__ import annotations
 
 import collections
 import dataclasses
-from typing import Deque, Dict, Hashable, List, Optional, Sequence
+import time
+from typing import Callable, Deque, Dict, Hashable, List, Optional, Sequence
 
 from ..cache.manager import CacheManager, OutOfPages
 
@@ -62,6 +73,8 @@ class Sequence_:
     preemptions: int = 0
     n_prompt_original: int = 0
     folded: int = 0
+    priority: int = 0                  # higher is admitted earlier and preempted later
+    arrival_time: float = 0.0          # the scheduler's clock when the request was added
 
     @property
     def is_prefilling(self) -> bool:
@@ -86,17 +99,35 @@ class StepPlan:
         return sum(len(i.tokens) for i in self.items)
 
 
+def priority_score(seq: "Sequence_", now: float) -> float:
+    """The default: the request's priority; equal priorities are served in arrival order."""
+    return float(seq.priority)
+
+
+def priority_age_score(aging_divisor_ms: float = 2000.0) -> Callable[["Sequence_", float], float]:
+    """The reference's policy: every ``aging_divisor_ms`` of waiting adds one to the effective priority
+    (scheduler/batch_selection_policy.cpp:10-20)."""
+    def score(seq: "Sequence_", now: float) -> float:
+        return float(seq.priority) + (now - seq.arrival_time) * 1e3 / aging_divisor_ms
+    return score
+
+
 class Scheduler:
-    def __init__(self, manager: CacheManager, config: SchedulerConfig, max_position: int):
+    def __init__(self, manager: CacheManager, config: SchedulerConfig, max_position: int,
+                 score: Optional[Callable[["Sequence_", float], float]] = None,
+                 clock: Callable[[], float] = time.monotonic):
+        """``score(request, now)``: the waiting request with the highest is admitted next (``priority_score`` unless
+        given); ``clock`` gives ``now`` and the requests' arrival times, in seconds."""
         config.validate()
         self.manager, self.config, self.max_position = manager, config, max_position
+        self.score, self.clock = score or priority_score, clock
         self.waiting: Deque[Sequence_] = collections.deque()
         self.running: List[Sequence_] = []
         self._arrivals = 0
         self._admissions = 0
 
     # ---- requests -----------------------------------------------------------------
-    def add(self, rid: Hashable, prompt: Sequence[int], max_new: int) -> Sequence_:
+    def add(self, rid: Hashable, prompt: Sequence[int], max_new: int, priority: int = 0) -> Sequence_:
         prompt = [int(t) for t in prompt]
         if not prompt:
             raise RequestRefused(f"request {rid!r}: empty prompt")
@@ -114,7 +145,8 @@ class Scheduler:
                 k = min(k, -(-(window + self.config.chunked_prefill_tokens) // P) + 2)
             if k > pool.num_pages:
                 raise RequestRefused(f"request {rid!r} can never fit: {k} pages needed in cache group {g}, the pool has {pool.num_pages}")
-        seq = Sequence_(rid, prompt, max_new, arrival=self._arrivals, n_prompt_original=len(prompt))
+        seq = Sequence_(rid, prompt, max_new, arrival=self._arrivals, n_prompt_original=len(prompt),
+                        priority=int(priority), arrival_time=self.clock())
         self._arrivals += 1
         self.waiting.append(seq)
         return seq
@@ -144,20 +176,23 @@ class Scheduler:
         victim.preemptions += 1
         self.waiting.appendleft(victim)
 
-    def _reserve_or_preempt(self, seq: Sequence_, n: int, plan: StepPlan) -> bool:
-        """Pages for ``seq``'s next n tokens, preempting the youngest running requests if needed.
-        False when ``seq`` itself had to go."""
+    def _reserve_or_preempt(self, seq: Sequence_, n: int, plan: StepPlan):
+        """Pages for ``seq``'s next n tokens, preempting running requests if needed (the lowest priority first, the
+        most recently admitted among equals).  Returns (whether ``seq`` got its pages: False when it had to go
+        itself, the tokens of this step that victims already planned in it had been charged)."""
+        refund = 0
         while True:
             try:
                 self.manager.reserve(seq.rid, n)
-                return True
+                return True, refund
             except OutOfPages:
-                victim = max(self.running, key=lambda s: s.admitted_at)
+                victim = max(self.running, key=lambda s: (-s.priority, s.admitted_at))
+                refund += sum(len(i.tokens) for i in plan.items if i.seq is victim)
                 plan.items = [i for i in plan.items if i.seq is not victim]
                 plan.preempted.append(victim.rid)
                 self._preempt(victim)
                 if victim is seq:
-                    return False
+                    return False, refund
 
     def schedule(self) -> StepPlan:
         cfg = self.config
@@ -174,19 +209,23 @@ class Scheduler:
                 wants = seq.computed + n == len(seq.prompt)
             else:
                 n, toks, wants = 1, [seq.generated[-1]], True
-            if self._reserve_or_preempt(seq, n, plan):
+            ok, refund = self._reserve_or_preempt(seq, n, plan)
+            budget += refund               # what a victim had been charged in this step is free again
+            if ok:
                 plan.items.append(PlannedItem(seq, toks, wants))
                 budget -= n
-        # 2. admissions, first come first served; a request preempted in this step waits for the next
+        # 2. admissions, best score first (first come first served among equals); a request preempted in this step
+        #    waits for the next
+        now = self.clock()
         while self.waiting and len(self.running) < cfg.max_batch_size and budget > 0:
-            seq = self.waiting[0]
+            seq = min(self.waiting, key=lambda q: (-self.score(q, now), q.arrival))
             if seq.rid in plan.preempted:
                 break
             n = min(len(seq.prompt), cfg.chunked_prefill_tokens, budget)
             need = self.manager.pages_needed_fresh(n)
             if any(k > f for k, f in zip(need, self.manager.free_pages())) or self.manager.free_slots() == 0:
                 break
-            self.waiting.popleft()
+            self.waiting.remove(seq)
             self.manager.add(seq.rid)
             seq.admitted_at = self._admissions
             self._admissions += 1

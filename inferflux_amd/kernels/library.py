@@ -35,6 +35,12 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
 
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
+# INFERFLUX_HOST_SANITIZE=1 builds the host-only modules (the cache's bookkeeping) with the address and
+# undefined-behaviour sanitizers, for test runs on the CPU (the process then needs libasan preloaded:
+# LD_PRELOAD=$(g++ -print-file-name=libasan.so)).  Device code is never built with a sanitizer.
+HOST_SANITIZE = os.environ.get("INFERFLUX_HOST_SANITIZE", "") == "1"
+if HOST_SANITIZE:
+    HOST_FLAGS = ["-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined", "-std=c++17", "-shared", "-fPIC"]
 
 Variant = Tuple[Tuple[str, int], ...]
 
@@ -76,19 +82,44 @@ def _digest(name: str, variant: Variant) -> str:
     return h.hexdigest()[:12]
 
 
-def _fallback_dir() -> str:
+def _fallback_dir(create: bool = False) -> Optional[str]:
+    """The per-user folder under the temporary directory that libraries go to when the source folder cannot be
+    written.  Libraries are loaded from it, so it must be this user's own and closed to everyone else: a folder
+    of that name that somebody else made, or that others may write, is refused.  Without ``create`` a folder
+    that does not exist is None."""
     d = os.path.join(tempfile.gettempdir(), f"inferflux_amd-{os.getuid()}")
-    os.makedirs(d, mode=0o700, exist_ok=True)
+    if create:
+        try:
+            os.mkdir(d, 0o700)
+        except FileExistsError:
+            pass
+    try:
+        st = os.lstat(d)
+    except FileNotFoundError:
+        return None
+    import stat
+    if not stat.S_ISDIR(st.st_mode) or st.st_uid != os.getuid() or st.st_mode & 0o077:
+        raise KernelBuildError(f"{d} is not a private folder of this user (owner {st.st_uid}, mode {stat.S_IMODE(st.st_mode):o}): "
+                               f"refusing to build into or load libraries from it")
     return d
 
 
+def _stem(name: str, variant: Variant) -> str:
+    """A library's file name up to its hash (a sanitized host build has a name of its own, so that it and the
+    ordinary build do not take each other for stale)."""
+    san = "-hostsan" if HOST_SANITIZE and _is_host_module(name) else ""
+    return f"{name}{san}{_variant_tag(variant)}"
+
+
 def _lib_filename(name: str, variant: Variant) -> str:
-    return f"{name}{_variant_tag(variant)}.{_digest(name, variant)}.so"
+    return f"{_stem(name, variant)}.{_digest(name, variant)}.so"
 
 
 def find_library(name: str, variant: Variant = ()) -> Optional[str]:
     fn = _lib_filename(name, variant)
     for d in (CSRC, _fallback_dir()):
+        if d is None:
+            continue
         p = os.path.join(d, fn)
         if os.path.isfile(p):
             return p
@@ -109,7 +140,7 @@ def compile_module(name: str, variant: Variant = (), force: bool = False) -> str
     src = os.path.join(CSRC, f"{name}.cpp" if host else f"{name}.hip")
     if not os.path.isfile(src):
         raise KernelBuildError(f"no kernel source {src}")
-    out_dir = CSRC if os.access(CSRC, os.W_OK) else _fallback_dir()
+    out_dir = CSRC if os.access(CSRC, os.W_OK) else _fallback_dir(create=True)
     fn = _lib_filename(name, variant)
     out = os.path.join(out_dir, fn)
     lock_path = os.path.join(out_dir, f".{name}{_variant_tag(variant)}.lock")
@@ -141,7 +172,7 @@ def compile_module(name: str, variant: Variant = (), force: bool = False) -> str
                 raise KernelBuildError(f"{os.path.basename(cmd[0])} failed for {label} (exit {proc.returncode}):\n{' '.join(cmd)}\n{log}")
             os.replace(tmp, out)
             # Drop libraries of the same module built from older sources.
-            prefix = f"{name}{_variant_tag(variant)}."
+            prefix = f"{_stem(name, variant)}."
             for old in os.listdir(out_dir):
                 if old.startswith(prefix) and old.endswith(".so") and old != fn:
                     try:

@@ -55,7 +55,7 @@ class ModelPlan:
     schedule: Tuple[ScheduleEntry, ...]
     final_norm: PartSpec
     lm_head: PartSpec
-    eos_token_id: Optional[int] = None
+    eos_token_ids: Tuple[int, ...] = ()      # every token id that ends a request (a model may name several)
 
     def validate(self) -> None:
         if not self.layers:

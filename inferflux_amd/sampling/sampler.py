@@ -70,7 +70,8 @@ class Sampler:
     def sample(self, logits: torch.Tensor, states: Sequence[SamplingState], while_waiting=None) -> List[int]:
         """One token per row of float32 ``logits`` [R, V]; row i belongs to ``states[i]``.  The
         logits are modified in place by penalties and bias.  States are advanced (draw counter,
-        history).  ``while_waiting`` is called with the chosen tokens (int32 [R], on the GPU) once the kernels and
+        history).  ``while_waiting`` is called with the chosen tokens (int32 [R], on the GPU) and the pinned host
+        tensor their copy is on its way to (valid once this function has returned) once the kernels and
         the copies of their results to the host are launched, before these are waited for: host work that needs no
         token goes there, and so may GPU work that takes the tokens where they are; the wait is for the copies
         only, not for what ``while_waiting`` launched."""
@@ -113,7 +114,7 @@ class Sampler:
         host_tokens = self._to_host(chosen, keep=True)
         self._copied.record()
         if while_waiting is not None:
-            while_waiting(chosen)
+            while_waiting(chosen, host_tokens)
         self._copied.synchronize()
         tokens = host_tokens.tolist()
         for r, (st, t) in enumerate(zip(states, tokens)):

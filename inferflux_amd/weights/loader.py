@@ -21,7 +21,8 @@ from typing import Dict, Iterable, List, Mapping, Optional, Tuple
 import torch
 
 from ..parts.plan import ParamSpec
-from .safetensors_io import SafetensorsError, SafetensorsFile, open_model_files, write_safetensors
+from .. import log
+from .safetensors_io import SafetensorsError, SafetensorsFile, open_model_files, write_safetensors, write_sharded
 
 
 class WeightError(ValueError):
@@ -53,7 +54,11 @@ def storage_dtype(file_dtype: torch.dtype, mode: torch.dtype, integer: bool) -> 
     raise ValueError(f"engine dtype must be float32 or bfloat16, got {mode}")
 
 
-def check_against_specs(folder: str, files: List[SafetensorsFile], specs: Mapping[str, ParamSpec]) -> Dict[str, SafetensorsFile]:
+def check_against_specs(folder: str, files: List[SafetensorsFile], specs: Mapping[str, ParamSpec],
+                        strict: bool = True, unused: Optional[List[str]] = None) -> Dict[str, SafetensorsFile]:
+    """Where each tensor lives, or ``WeightError`` with everything that is wrong.  Tensors nobody asked for are an
+    error when ``strict``; otherwise they are reported through ``unused`` (older exports carry buffers such as
+    ``rotary_emb.inv_freq`` that no part reads) and everything else is still checked."""
     where: Dict[str, SafetensorsFile] = {}
     other: List[str] = []
     for f in files:
@@ -72,19 +77,29 @@ def check_against_specs(folder: str, files: List[SafetensorsFile], specs: Mappin
                 wrong.append((n, tuple(got), tuple(s.shape)))
             if s.integer == where[n].dtype(n).is_floating_point:
                 other.append(f"tensor '{n}' is {where[n].dtype(n)}, expected {'an integer' if s.integer else 'a floating'} type")
-    if missing or unexpected or wrong or other:
+    if missing or (unexpected and strict) or wrong or other:
         raise WeightError(folder, missing, unexpected, sorted(wrong), other)
+    if unused is not None:
+        unused[:] = unexpected
     return where
 
 
-def load_weights(folder: str, specs: Mapping[str, ParamSpec], mode: torch.dtype, device) -> Dict[str, torch.Tensor]:
-    """All tensors ``specs`` names that the folder holds, on ``device``, stored by the rule above."""
+def load_weights(folder: str, specs: Mapping[str, ParamSpec], mode: torch.dtype, device, strict: bool = True,
+                 report: Optional[Dict[str, List[str]]] = None) -> Dict[str, torch.Tensor]:
+    """All tensors ``specs`` names that the folder holds, on ``device``, stored by the rule above.  With ``strict``
+    False tensors that no part asked for are left alone, logged as a warning and listed in ``report["unused"]``."""
     try:
         files = open_model_files(folder)
     except SafetensorsError as e:
         raise WeightError(folder, [], [], [], [str(e)]) from None
     try:
-        where = check_against_specs(folder, files, specs)
+        unused: List[str] = []
+        where = check_against_specs(folder, files, specs, strict, unused)
+        if unused:
+            log.warn("weights", f"{folder}: {len(unused)} tensors are not used by the model: " + ", ".join(unused[:8])
+                     + (" ..." if len(unused) > 8 else ""))
+        if report is not None:
+            report["unused"] = unused
         out: Dict[str, torch.Tensor] = {}
         for n, s in specs.items():
             if n not in where:
@@ -126,12 +141,13 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, dev
 
 
 def write_random_model(folder: str, config, seed: int, dtype: torch.dtype = torch.bfloat16,
-                       float32_tensors: Iterable[str] = (), include_optional: bool = True) -> None:
+                       float32_tensors: Iterable[str] = (), include_optional: bool = True, shards: int = 1) -> None:
     """Write ``config.json`` and ``model.safetensors`` with seeded random weights.
 
     Matrices, tables and biases are N(0, 0.02) and norm weights 1.0, as each part's specs say.
     Tensors named in ``float32_tensors`` (exact names or suffixes) are stored in float32
-    instead of ``dtype``.
+    instead of ``dtype``.  With ``shards`` > 1 the tensors go into that many files with an index, as large
+    checkpoints are laid out; a tensor's values do not depend on the layout.
     """
     from ..engine.model import Model
     specs = Model.param_specs_for(config)
@@ -144,5 +160,8 @@ def write_random_model(folder: str, config, seed: int, dtype: torch.dtype = torc
         tensors[name] = random_tensor(name, spec, seed, dt)
     os.makedirs(folder, exist_ok=True)
     config.save(folder)
-    write_safetensors(os.path.join(folder, "model.safetensors"), tensors,
-                      metadata={"format": "pt", "seed": str(seed)})
+    meta = {"format": "pt", "seed": str(seed)}
+    if shards > 1:
+        write_sharded(folder, tensors, shards, meta)
+    else:
+        write_safetensors(os.path.join(folder, "model.safetensors"), tensors, metadata=meta)

@@ -71,6 +71,13 @@ class SafetensorsFile:
             if self.data_start + e > size:
                 raise SafetensorsError(f"{path}: tensor '{name}' reaches past the end of the file (truncated?)")
             self.entries[name] = (tdt, shape, b, e)
+        # No two tensors may share bytes: a header whose ranges overlap is not something a writer produces.
+        last_end, last_name = 0, None
+        for name, (_, _, b, e) in sorted(self.entries.items(), key=lambda kv: (kv[1][2], kv[1][3])):
+            if e > b:
+                if b < last_end:
+                    raise SafetensorsError(f"{path}: tensors '{last_name}' and '{name}' overlap in the file")
+                last_end, last_name = e, name
 
     def names(self) -> List[str]:
         return list(self.entries)
@@ -138,6 +145,14 @@ def open_model_files(folder: str) -> List[SafetensorsFile]:
             shards = sorted(set(wm.values()))
         except (json.JSONDecodeError, KeyError, AttributeError, TypeError) as e:
             raise SafetensorsError(f"{index}: not a safetensors index ({e})") from None
+        if not shards:
+            raise SafetensorsError(f"{index}: the weight map names no files")
+        root = os.path.realpath(folder)
+        for s in shards:
+            inside = isinstance(s, str) and s and not os.path.isabs(s) and \
+                os.path.commonpath([root, os.path.realpath(os.path.join(root, s))]) == root
+            if not inside:
+                raise SafetensorsError(f"{index}: shard name {s!r} does not stay inside the model folder")
         missing = [s for s in shards if not os.path.isfile(os.path.join(folder, s))]
         if missing:
             raise SafetensorsError(f"{index} names shard files that do not exist: {missing}")
@@ -146,3 +161,29 @@ def open_model_files(folder: str) -> List[SafetensorsFile]:
     if os.path.isfile(single):
         return [SafetensorsFile(single)]
     raise SafetensorsError(f"{folder}: no safetensors files found (model.safetensors or model.safetensors.index.json)")
+
+
+def write_sharded(folder: str, tensors: Mapping[str, torch.Tensor], n_shards: int, metadata: Mapping[str, str] = None) -> List[str]:
+    """Write ``tensors`` as ``n_shards`` files ``model-0000i-of-0000n.safetensors`` (names dealt out in sorted order, by
+    bytes) plus ``model.safetensors.index.json``, the layout of large checkpoints; returns the shard names."""
+    if n_shards < 1:
+        raise SafetensorsError("a model needs at least one shard")
+    names = sorted(tensors)
+    total = sum(tensors[n].numel() * tensors[n].element_size() for n in names)
+    shards: List[Dict[str, torch.Tensor]] = [{} for _ in range(n_shards)]
+    seen = 0
+    for n in names:
+        shards[min(n_shards - 1, seen * n_shards // max(total, 1))][n] = tensors[n]
+        seen += tensors[n].numel() * tensors[n].element_size()
+    files, weight_map = [], {}
+    for i, part in enumerate(shards):
+        fn = f"model-{i + 1:05d}-of-{n_shards:05d}.safetensors"
+        write_safetensors(os.path.join(folder, fn), part, metadata)
+        files.append(fn)
+        for n in part:
+            weight_map[n] = fn
+    tmp = os.path.join(folder, "model.safetensors.index.json.tmp")
+    with open(tmp, "w") as f:
+        json.dump({"metadata": {"total_size": total}, "weight_map": weight_map}, f, indent=1)
+    os.replace(tmp, os.path.join(folder, "model.safetensors.index.json"))
+    return files

@@ -342,6 +342,17 @@ def test_a_decode_step_started_before_the_host_has_its_tokens(sharp_folders):
     assert not runner.launch_prepared(torch.zeros(2, dtype=torch.int32, device="cuda"))
     assert not runner.launch_prepared(torch.zeros(1, dtype=torch.int64, device="cuda"))
     assert not runner.launch_prepared(torch.zeros(1, dtype=torch.int32))
+    # a step that brings other tokens than the early one ran on is computed afresh, with its own tokens
+    started_on = torch.tensor([ids["a"][31]], dtype=torch.int32, device="cuda")
+    assert runner.launch_prepared(started_on)
+    other = (ids["a"][31] + 1) % V
+    got = runner.step([StepEntry("x", [other], [0])]).cpu()
+    fresh = load_runner(folder, torch.float32, num_pages=24)
+    fresh.add_request("y")
+    fresh.step([StepEntry("y", ids["a"][:31], [])])
+    assert torch.equal(got, fresh.step([StepEntry("y", [other], [0])]).cpu())
+    assert runner.length("x") == 32
+    assert runner.prepare_decode(["x"])
     runner.storage._states[0] = torch.zeros(1, device="cuda")
     assert not runner.launch_prepared(torch.zeros(1, dtype=torch.int32, device="cuda")) and runner._prepared is not None
 

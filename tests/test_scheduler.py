@@ -172,3 +172,81 @@ def test_random_workloads_finish_with_the_right_tokens(seed):
     for i, p in prompts.items():
         assert out[i] == expected(p, news[i])
     assert m.free_pages() == [m.pools[0].num_pages]
+
+
+def test_priority_decides_admission_and_the_default_is_first_come_first_served():
+    # one place in the batch: the order of admission is the order of service
+    m, s = make(pages=64, max_batch_size=1)
+    s.add("low", [1, 2, 3], 2)
+    s.add("high", [4, 5, 6], 2, priority=5)
+    s.add("mid", [7, 8], 2, priority=2)
+    s.add("high2", [9], 2, priority=5)
+    log = []
+    drive(m, s, log=log)
+    order = []
+    for step in log:
+        for rid, _, _ in step:
+            if rid not in order:
+                order.append(rid)
+    assert order == ["high", "high2", "mid", "low"]            # by priority, arrival among equals
+
+
+def test_the_score_hook_is_the_references_priority_plus_age():
+    # scheduler/batch_selection_policy.cpp:10-20: every 2 s of waiting count as one step of priority
+    from inferflux_amd.engine.scheduler import priority_age_score
+    now = [0.0]
+    m = CacheManager([GroupSpec(None, (0,))], 16, 64, 8)
+    s = Scheduler(m, SchedulerConfig(max_batch_size=1), 4096, score=priority_age_score(2000.0), clock=lambda: now[0])
+    old = s.add("old", [1, 2], 1)                               # priority 0, arrives at t = 0
+    now[0] = 3.0
+    new = s.add("new", [3, 4], 1, priority=1)                   # priority 1, arrives at t = 3
+    assert s.score(old, 3.0) == 1.5 and s.score(new, 3.0) == 1.0
+    plan = s.schedule()                                         # at t = 3 the old request has aged past the new one
+    assert [i.seq.rid for i in plan.items] == ["old"]
+    m2 = CacheManager([GroupSpec(None, (0,))], 16, 64, 8)
+    s2 = Scheduler(m2, SchedulerConfig(max_batch_size=1), 4096, score=priority_age_score(2000.0), clock=lambda: now[0])
+    now[0] = 0.0
+    s2.add("old", [1, 2], 1)
+    now[0] = 1.0
+    s2.add("new", [3, 4], 1, priority=1)
+    assert [i.seq.rid for i in s2.schedule().items] == ["new"]  # one second of age does not outweigh a priority step
+
+
+def test_the_victim_is_the_lowest_priority_then_the_youngest():
+    m, s = make(pages=4, page_size=16)
+    a = s.add("a", list(range(30)), 30)                         # oldest, priority 0
+    b = s.add("b", list(range(100, 120)), 30, priority=3)       # younger but more important
+    plan = s.schedule()
+    assert [i.seq.rid for i in plan.items] == ["b", "a"] and m.free_pages() == [0]
+    for it in plan.items:
+        m.commit(it.seq.rid, len(it.tokens)); s.advance(it); it.seq.generated.append(1)
+    # b reaches its page edge (32 tokens) and needs a third page: a, of lower priority, has to go although it is older
+    for _ in range(12):
+        m.reserve("b", 1); m.commit("b", 1); b.computed += 1; b.generated.append(2)
+    plan = s.schedule()
+    assert plan.preempted == ["a"] and [i.seq.rid for i in plan.items] == ["b"]
+    assert s.waiting[0] is a and not m.has("a")
+
+
+def test_a_victims_tokens_return_to_the_steps_budget():
+    """A running request of low priority is planned, then a more important one needs a page and takes the first
+    one's: the token the victim had been charged is free again for an admission in the same step."""
+    m, s = make(pages=3, page_size=16, max_batch_tokens=2)
+    a = s.add("a", list(range(16)), 30)                         # priority 0, admitted first
+    s.config.max_batch_tokens = 64
+    plan = s.schedule()
+    for it in plan.items:
+        m.commit("a", len(it.tokens)); s.advance(it); a.generated.append(1)
+    b = s.add("b", list(range(100, 116)), 30, priority=5)
+    plan = s.schedule()                                         # a decodes (its 17th token: a second page), b is admitted
+    assert [(i.seq.rid, len(i.tokens)) for i in plan.items] == [("a", 1), ("b", 16)] and m.free_pages() == [0]
+    for it in plan.items:
+        m.commit(it.seq.rid, len(it.tokens)); s.advance(it); it.seq.generated.append(2)
+    s.add("c", [7, 8, 9, 10, 11], 4, priority=1)
+    s.config.max_batch_tokens = 2
+    plan = s.schedule()
+    # a was dealt its token, then b needed a page for its 17th and a, of lower priority, had to go; the token a had
+    # been charged went to c, which outranks the preempted a in the queue
+    assert plan.preempted == ["a"]
+    assert [(i.seq.rid, len(i.tokens)) for i in plan.items] == [("b", 1), ("c", 1)] and plan.n_tokens == 2
+    assert s.waiting[0] is a

@@ -132,3 +132,99 @@ def test_config_and_file_are_cross_checked(tmp_path, model_folders):
 def test_missing_files(tmp_path):
     with pytest.raises(WeightError, match="no safetensors files"):
         load_weights(str(tmp_path), {}, torch.float32, "cpu")
+
+
+def test_shards_with_an_index_load_bit_equal(tmp_path, model_folders):
+    """The layout of large checkpoints (the reference's rule: index's weight_map -> set of shard files,
+    runtime/backends/cuda/inferflux_cuda_executor.cpp:366-402): same tensors, bit for bit, as one file."""
+    cfg = tiny_config("B")
+    specs = Model.param_specs_for(cfg)
+    d = tmp_path / "sharded"
+    write_random_model(str(d), cfg, seed=101, dtype=torch.bfloat16, shards=3)
+    index = json.load(open(d / "model.safetensors.index.json"))
+    shards = sorted(set(index["weight_map"].values()))
+    assert len(shards) == 3 and all(os.path.isfile(d / s) for s in shards) and not os.path.exists(d / "model.safetensors")
+    assert sorted(index["weight_map"]) == sorted(specs)
+    sizes = [os.path.getsize(d / s) for s in shards]
+    assert min(sizes) > 0.15 * sum(sizes)                               # dealt out by bytes, not all in one
+    one = load_weights(model_folders["B"], specs, torch.bfloat16, "cpu")   # conftest wrote this one with the same seed
+    many = load_weights(str(d), specs, torch.bfloat16, "cpu")
+    assert sorted(one) == sorted(many) and all(torch.equal(one[k], many[k]) and one[k].dtype == many[k].dtype for k in one)
+    # the independent reader sees the same tensors in the files the index names
+    from safetensors.torch import load_file
+    for s in shards:
+        for k, v in load_file(str(d / s)).items():
+            assert index["weight_map"][k] == s and torch.equal(v, one[k])
+
+
+def test_broken_shard_sets_are_errors_that_name_the_file(tmp_path, model_folders):
+    import shutil
+    cfg = tiny_config("A")
+    specs = Model.param_specs_for(cfg)
+    d = tmp_path / "s"
+    write_random_model(str(d), cfg, seed=1, shards=2)
+    index_path = d / "model.safetensors.index.json"
+    index = json.load(open(index_path))
+    shards = sorted(set(index["weight_map"].values()))
+    # a shard the index names is not there
+    os.rename(d / shards[1], d / "elsewhere.safetensors")
+    with pytest.raises(WeightError, match="shard files that do not exist.*" + shards[1].replace(".", r"\.")):
+        load_weights(str(d), specs, torch.bfloat16, "cpu")
+    os.rename(d / "elsewhere.safetensors", d / shards[1])
+    # a tensor in two shards
+    from safetensors.torch import load_file
+    first = load_file(str(d / shards[0]))
+    second = load_file(str(d / shards[1]))
+    dup = next(iter(first))
+    write_safetensors(str(d / shards[1]), {**second, dup: first[dup]})
+    with pytest.raises(WeightError, match=f"'{dup}' appears in both"):
+        load_weights(str(d), specs, torch.bfloat16, "cpu")
+    write_safetensors(str(d / shards[1]), second)
+    # shard names that leave the folder
+    outside = tmp_path / "outside.safetensors"
+    shutil.copy(d / shards[1], outside)
+    for bad in ("../outside.safetensors", str(outside)):
+        json.dump({"weight_map": {**index["weight_map"], dup: bad}}, open(index_path, "w"))
+        with pytest.raises(WeightError, match="does not stay inside the model folder"):
+            load_weights(str(d), specs, torch.bfloat16, "cpu")
+    json.dump({"weight_map": {}}, open(index_path, "w"))
+    with pytest.raises(WeightError, match="names no files"):
+        load_weights(str(d), specs, torch.bfloat16, "cpu")
+    json.dump(["not", "an", "index"], open(index_path, "w"))
+    with pytest.raises(WeightError, match="not a safetensors index"):
+        load_weights(str(d), specs, torch.bfloat16, "cpu")
+
+
+def test_tensors_that_overlap_in_the_file_are_refused(tmp_path):
+    p = str(tmp_path / "o.safetensors")
+    hdr = json.dumps({"a": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]},
+                      "b": {"dtype": "F32", "shape": [4], "data_offsets": [8, 24]}}).encode()
+    open(p, "wb").write(struct.pack("<Q", len(hdr)) + hdr + b"\0" * 24)
+    with pytest.raises(SafetensorsError, match="'a' and 'b' overlap"):
+        SafetensorsFile(p)
+
+
+def test_unused_tensors_are_an_error_or_a_reported_warning(tmp_path, model_folders, capfd):
+    """Older exports carry buffers no part reads (rotary_emb.inv_freq): an error by default, a warning that lists
+    them when the caller says so; what is missing or misshapen stays an error either way."""
+    from safetensors.torch import load_file
+    cfg = tiny_config("A")
+    specs = Model.param_specs_for(cfg)
+    raw = load_file(os.path.join(model_folders["A"], "model.safetensors"))
+    raw["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    d = tmp_path / "old"
+    d.mkdir()
+    cfg.save(str(d))
+    write_safetensors(str(d / "model.safetensors"), raw)
+    with pytest.raises(WeightError) as ei:
+        load_weights(str(d), specs, torch.bfloat16, "cpu")
+    assert ei.value.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    report = {}
+    got = load_weights(str(d), specs, torch.bfloat16, "cpu", strict=False, report=report)
+    assert report["unused"] == ["model.layers.0.self_attn.rotary_emb.inv_freq"] and sorted(got) == sorted(specs)
+    assert "1 tensors are not used by the model" in capfd.readouterr().err
+    del raw["model.norm.weight"]
+    write_safetensors(str(d / "model.safetensors"), raw)
+    with pytest.raises(WeightError) as ei:
+        load_weights(str(d), specs, torch.bfloat16, "cpu", strict=False)
+    assert ei.value.missing == ["model.norm.weight"]
