@@ -228,3 +228,138 @@ def test_logprobs_through_the_engine(model_folders):
         assert l.top_logprobs[0][0] == l.token_id and len(l.top_logprobs) == 3          # greedy: the sampled token is the top one
         assert all(abs(v - float(want[t])) < 1e-4 for t, v in l.top_logprobs)
     assert engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))[0].logprobs is None
+
+
+def _stateful_toy_runner(pages, slots):
+    """A two-layer model made outside the package: attention, then a mixer that keeps a decayed sum per request in a
+    state slot (no cache).  A state that is not zero when a request starts changes every token after it."""
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.parts import LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec, ScheduleEntry, StateSpec, register_part
+    from inferflux_amd.parts.base import registered_parts
+
+    H, V, kind = 32, 61, "toy_decay_sum_for_generation"
+    if kind not in registered_parts("mixer"):
+        @register_part("mixer", kind)
+        class DecaySum(Mixer):
+            def __init__(self, name, hidden_size, decay):
+                self.name, self.H, self.decay = name, hidden_size, decay
+            def param_specs(self):
+                return {f"{self.name}.mix.weight": ParamSpec((self.H, self.H), ("normal", 0.3))}
+            def load(self, tensors):
+                self.w = tensors[f"{self.name}.mix.weight"]
+            def state_spec(self):
+                return StateSpec((self.H,), "float32")
+            def forward(self, h, ctx, binding):
+                out = torch.empty_like(h)
+                for r in range(ctx.n_requests):
+                    s = binding.state[int(ctx.h_state_slots[r])]
+                    a, n = int(ctx.h_q_start[r]), int(ctx.h_q_len[r])
+                    for t in range(a, a + n):
+                        s.mul_(self.decay).add_(h[t].float())
+                        out[t] = s.to(h.dtype)
+                return out @ self.w.t()
+
+    def layer(i, mixer):
+        p = f"toy.layers.{i}"
+        return LayerSpec(p, PartSpec("prenorm"), PartSpec("rmsnorm", {"name": f"{p}.n1", "eps": 1e-5}), mixer,
+                         PartSpec("rmsnorm", {"name": f"{p}.n2", "eps": 1e-5}),
+                         PartSpec("swiglu", {"name": f"{p}.mlp", "intermediate_size": 48}))
+
+    attn = PartSpec("paged_attention", {"name": "toy.layers.0.attn", "n_heads": 2, "n_kv_heads": 1, "head_dim": 16,
+                                        "bias": False, "position": PartSpec("rotary", {"head_dim": 16, "theta": 100.0})})
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=256,
+                     embedding=PartSpec("token_embedding", {"name": "toy.embed", "vocab_size": V}),
+                     layers=(layer(0, attn), layer(1, PartSpec(kind, {"name": "toy.layers.1.mixer", "decay": 0.95}))),
+                     schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+                     final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
+    model = Model(plan=plan).init_random(4, torch.float32, "cuda")
+    return ModelRunner(model, num_pages=pages, max_requests=slots), V
+
+
+def test_per_request_state_is_zero_for_every_admission_through_the_engine():
+    """Requests admitted by the scheduler (not through the runner's add_request): into a slot another request has
+    left, and again after a preemption.  Each one's tokens must be those of the same request alone in a fresh engine."""
+    from inferflux_amd.engine.engine import Engine as Eng
+    from inferflux_amd.engine.scheduler import SchedulerConfig
+    lens, n_new = [30, 9, 40, 22, 35], 24
+    sp = SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True)
+    want = []
+    for i, n in enumerate(lens):
+        runner, V = _stateful_toy_runner(pages=16, slots=1)
+        want.append(Eng(runner, SchedulerConfig(1, 4096, 512)).generate([seeded_ids(500 + i, n, V)], sp)[0].token_ids)
+    assert len({tuple(w) for w in want}) == len(want)
+    prompts = [seeded_ids(500 + i, n, V) for i, n in enumerate(lens)]
+    # two slots for five requests: three of them start in a slot that holds another request's last state
+    runner, _ = _stateful_toy_runner(pages=32, slots=2)
+    eng = Eng(runner, SchedulerConfig(2, 4096, 16))
+    assert not runner.starts_steps_early                      # a step over state cannot be run twice
+    outs = eng.generate(prompts, sp)
+    assert [o.token_ids for o in outs] == want and eng.stats.preemptions == 0
+    # three slots and 7 pages: 30+24, 9+24 and 40+24 tokens need 4 + 3 + 4 pages, so somebody is preempted and
+    # admitted again (its slot may be the one it had: the state it left there must not survive)
+    runner, _ = _stateful_toy_runner(pages=7, slots=3)
+    eng = Eng(runner, SchedulerConfig(3, 4096, 16))
+    outs = eng.generate(prompts, sp)
+    assert eng.stats.preemptions >= 1 and any(o.preemptions for o in outs)
+    assert [o.token_ids for o in outs] == want
+    runner.manager.check()
+    assert runner.manager.free_pages() == [7]
+
+
+@pytest.mark.parametrize("early", [True, False])
+def test_requests_added_and_aborted_between_steps_by_hand(early, model_folders):
+    """The engine driven step by step: a request arrives between two decode steps (the step that was started early
+    for the others is void), a running request is aborted right after a step that started the next one early (its
+    row of that step is dropped), a waiting one is aborted before it ever ran, greedy requests run beside a seeded
+    one.  Survivors' tokens are the plain model's; aborted requests return what they had."""
+    folder, V = model_folders["B"], TINY["B"]["vocab_size"]
+    P = {k: seeded_ids(600 + i, n, V) for i, (k, n) in enumerate({"a": 21, "b": 5, "c": 33, "d": 12, "w": 8, "s": 17, "x": 9}.items())}
+    greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)
+    eng = Engine.load(folder, dtype="float32", kv_pages=40, max_batch_size=4, chunked_prefill_tokens=16,
+                      start_steps_early=early)
+    runner = eng.runner
+    done = {}
+
+    def step(n=1):
+        for _ in range(n):
+            for o in eng.step():
+                done[o.request_id] = o
+
+    eng.add_request(P["a"], greedy(30), "a")
+    eng.add_request(P["b"], greedy(30), "b")
+    eng.add_request(P["s"], SamplingParams(temperature=0.9, top_p=0.95, seed=77, max_tokens=12, ignore_eos=True), "s")
+    step(6)                                                    # prompts are in, everyone decodes
+    if early:
+        assert runner._launched is not None                    # the next step of a, b, s is already running
+    eng.add_request(P["c"], greedy(10), "c")                   # an arrival: that step is void
+    step(1)
+    assert runner.has_request("c")
+    step(5)
+    if early:
+        assert runner._launched is not None and "b" in runner._launched[0][0]
+    out_b = eng.abort("b")                                     # b's row of the step that is running is dropped
+    assert out_b.finish_reason == "abort" and not runner.has_request("b") and len(out_b.token_ids) >= 5
+    step(2)
+    # s has reached its limit; d and w fill the batch (a, c, d, w), x waits and is aborted before it ever ran
+    assert "s" in done and len(eng.scheduler.running) == 2
+    eng.add_request(P["d"], greedy(8), "d")
+    eng.add_request(P["w"], greedy(8), "w")
+    eng.add_request(P["x"], greedy(8), "x")
+    step(1)
+    assert runner.has_request("d") and runner.has_request("w") and not runner.has_request("x") and len(eng.scheduler.waiting) == 1
+    out_x = eng.abort("x")
+    assert out_x.finish_reason == "abort" and out_x.token_ids == [] and not eng.scheduler.waiting
+    assert eng.abort("x") is None and eng.abort("nobody") is None
+    while eng.has_unfinished():
+        step(1)
+    runner.manager.check()
+    assert runner.manager.free_pages() == [40] and not runner.manager.live()
+    for k, n in (("a", 30), ("c", 10), ("d", 8), ("w", 8)):
+        assert done[k].finish_reason == "length" and done[k].token_ids == plain_greedy(folder, P[k], n), k
+    assert out_b.token_ids == plain_greedy(folder, P["b"], 30)[: len(out_b.token_ids)]
+    # the seeded request alone gives the same tokens: neither the batch nor the arrivals and aborts around it matter
+    alone = Engine.load(folder, dtype="float32", kv_pages=40, max_batch_size=4)
+    assert alone.generate([P["s"]], SamplingParams(temperature=0.9, top_p=0.95, seed=77, max_tokens=12, ignore_eos=True))[0].token_ids \
+        == done["s"].token_ids
