@@ -2,7 +2,7 @@
 per-request state tensors, laid out from what the model's mixers declare.
 
 K pages are [page][kv head][offset][d] (a key's elements contiguous, as the score needs them);
-V pages are [page][kv head][d][offset] (a page's values of one element contiguous, as the
+V pages are [page][kv head][dv][offset] (a page's values of one element contiguous, as the
 weighted sum needs them).  Validity is defined by block tables and lengths, so pages are never
 cleared when they change hands; they are zero when first allocated so that a masked key can
 never contribute a NaN.  The reference keeps one contiguous [max_seq][nKV*d] slab per sequence
@@ -40,7 +40,7 @@ def plan_groups(schedule, mixers) -> Tuple[List[GroupSpec], Dict[int, int]]:
         if e.cache_from is not None and mixers[i].cache_spec() is not None:
             owner = mixers[e.cache_from].cache_spec()
             mine = mixers[i].cache_spec()
-            if owner is None or (owner.n_kv_heads, owner.head_dim) != (mine.n_kv_heads, mine.head_dim):
+            if owner is None or (owner.n_kv_heads, owner.k_dim, owner.v_dim) != (mine.n_kv_heads, mine.k_dim, mine.v_dim):
                 raise ValueError(f"schedule[{i}] reads the cache of entry {e.cache_from}, whose shape differs")
             if owner.window is not None and (mine.window is None or mine.window > owner.window):
                 raise ValueError(f"schedule[{i}] reads further back than entry {e.cache_from} keeps (window {owner.window})")
@@ -63,8 +63,8 @@ class CacheStorage:
             if spec is not None and e.cache_from is None:
                 g = self.entry_group[i]
                 n = counts[g]
-                k = torch.zeros((n, spec.n_kv_heads, page_size, spec.head_dim), dtype=dtype, device=device)
-                v = torch.zeros((n, spec.n_kv_heads, spec.head_dim, page_size), dtype=dtype, device=device)
+                k = torch.zeros((n, spec.n_kv_heads, page_size, spec.k_dim), dtype=dtype, device=device)
+                v = torch.zeros((n, spec.n_kv_heads, spec.v_dim, page_size), dtype=dtype, device=device)
                 self._caches[i] = LayerCache(k, v, g, page_size)
             st = m.state_spec()
             if st is not None:
@@ -91,4 +91,4 @@ class CacheStorage:
             t[slot].zero_()
 
     def bytes_per_token(self) -> int:
-        return sum(c.k[0].numel() * c.k.element_size() * 2 // self.page_size for c in self._caches.values())
+        return sum((c.k[0].numel() + c.v[0].numel()) * c.k.element_size() // self.page_size for c in self._caches.values())

@@ -11,7 +11,8 @@
 // the query at position p sees keys j with max(0, p - window + 1) <= j <= p; s_j = (q . k_j) *
 // scale; o = sum_j softmax(s)_j v_j.
 //
-// Cache layouts: K [page][kv head][offset][d], V [page][kv head][d][offset].
+// Cache layouts: K [page][kv head][offset][d], V [page][kv head][dv][offset].  Values may have another width
+// than keys (dv != d): the output row of a head then has dv elements.
 #include "common.h"
 
 IFX_DEFINE_LAST_ERROR()
@@ -29,7 +30,7 @@ struct AttnArgs {
   const int* positions;
   const int* block_table;
   int max_blocks;
-  int T, nH, nKV, d, page_size, window;
+  int T, nH, nKV, d, dv, page_size, window;
   float scale;
 };
 
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
   // barrier follows.
   if (item >= (long long)a.T * a.nH) return;
   const int row = (int)(item / a.nH), head = (int)(item % a.nH);
-  const int d = a.d, P = a.page_size;
+  const int d = a.d, dv = a.dv, P = a.page_size;
   const int kvh = head / (a.nH / a.nKV);
   const int pos = a.positions[row];
   const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
@@ -84,33 +85,34 @@ __global__ __launch_bounds__(WAVE * WAVES_PER_BLOCK) void attn_plain_kernel(Attn
       const float pj = __shfl(p, jj, WAVE);
       const int pg = __shfl(page, jj, WAVE), of = __shfl(off, jj, WAVE);
       if (pj == 0.f) continue;  // uniform over the wave; keys outside the range are never read
-      const T* vb = Vc + ((size_t)pg * a.nKV + kvh) * d * P + of;
+      const T* vb = Vc + ((size_t)pg * a.nKV + kvh) * dv * P + of;
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
         const int e = lane + c * WAVE;
-        if (e < d) acc[c] = fmaf(pj, to_f(vb[(size_t)e * P]), acc[c]);
+        if (e < dv) acc[c] = fmaf(pj, to_f(vb[(size_t)e * P]), acc[c]);
       }
     }
     m = m_new;
   }
-  T* orow = (T*)a.out + ((size_t)row * a.nH + head) * d;
+  T* orow = (T*)a.out + ((size_t)row * a.nH + head) * dv;
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
   for (int c = 0; c < DC; ++c) {
     const int e = lane + c * WAVE;
-    if (e < d) orow[e] = from_f<T>(acc[c] * inv);
+    if (e < dv) orow[e] = from_f<T>(acc[c] * inv);
   }
 }
 
 extern "C" int ifx_attn_plain(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                               const int* row_req, const int* positions, const int* block_table,
-                              int max_blocks, int T, int nH, int nKV, int d, int page_size, int window,
+                              int max_blocks, int T, int nH, int nKV, int d, int dv, int page_size, int window,
                               float scale, void* stream) {
   IFX_REQUIRE(T >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_plain: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(d > 0 && d <= MAX_D, "attn_plain: head_dim %d outside 1..%d", d, MAX_D);
+  IFX_REQUIRE(dv > 0 && dv <= MAX_D, "attn_plain: value head_dim %d outside 1..%d", dv, MAX_D);
   IFX_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attn_plain: bad page_size/max_blocks/window");
   if (T == 0) return 0;
-  AttnArgs a{q, k_cache, v_cache, out, row_req, positions, block_table, max_blocks, T, nH, nKV, d, page_size, window, scale};
+  AttnArgs a{q, k_cache, v_cache, out, row_req, positions, block_table, max_blocks, T, nH, nKV, d, dv, page_size, window, scale};
   const long long items = (long long)T * nH;
   const unsigned blocks = (unsigned)((items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
   hipStream_t s = (hipStream_t)stream;

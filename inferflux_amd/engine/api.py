@@ -63,7 +63,7 @@ def plan_kv_pages(model: Model, page_size: int, wanted_tokens: int, memory_fract
     for e, mixer in zip(model.plan.schedule, model.schedule_mixers()):
         spec = mixer.cache_spec()
         if spec is not None and e.cache_from is None:
-            per_token += 2 * spec.n_kv_heads * spec.head_dim * esz
+            per_token += spec.bytes_per_token(esz)
     want = max(1, -(-wanted_tokens // page_size))
     if per_token == 0:
         return want

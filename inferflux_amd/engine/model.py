@@ -100,7 +100,7 @@ class Model:
         if t is not None:
             t.begin()
             t.enter("embed")
-        residual = self.embedding.forward(ctx.token_ids)
+        residual = self.embedding.forward(ctx)
         if t is not None:
             t.mark("embed")
         pending = None

@@ -651,19 +651,21 @@ def linear_swiglu(x: torch.Tensor, weight_pairs) -> torch.Tensor:
 def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_req: torch.Tensor,
                     positions: torch.Tensor, block_table: torch.Tensor, window: Optional[int],
                     scale: float) -> torch.Tensor:
-    """Causal (optionally windowed) attention of q [T, nH, d] over the paged cache; returns [T, nH*d]."""
+    """Causal (optionally windowed) attention of q [T, nH, d] over the paged cache (K [pages, nKV, page, d],
+    V [pages, nKV, dv, page]; dv may differ from d); returns [T, nH*dv]."""
     _check(q, "q", (None, None, None))
     T, nH, d = q.shape
     _check(k_cache, "k_cache", (None, None, None, d), q.dtype)
     n_pages, nKV, page_size, _ = k_cache.shape
-    _check(v_cache, "v_cache", (n_pages, nKV, d, page_size), q.dtype)
+    _check(v_cache, "v_cache", (n_pages, nKV, None, page_size), q.dtype)
+    dv = v_cache.shape[2]
     _check(row_req, "row_req", (T,), torch.int32)
     _check(positions, "positions", (T,), torch.int32)
     _check(block_table, "block_table", (None, None), torch.int32)
-    out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
-    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P),
+    out = torch.empty((T, nH * dv), dtype=q.dtype, device=q.device)
+    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q), row_req.data_ptr(),
-          positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, page_size,
+          positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, dv, page_size,
           int(window or 0), float(scale), _stream())
     return out
 

@@ -18,7 +18,8 @@ Categories and what each must provide beyond ``param_specs`` / ``load``:
   ffn       forward(h, ctx) -> delta [T, H].
   block     the arrangement: forward(residual, pending, ctx, binding) -> (residual, pending),
             where ``pending`` is a delta not yet added to the stream (the next norm adds it).
-  embedding forward(token_ids) -> float32 stream [T, H].
+  embedding forward(ctx) -> float32 stream [T, H] of the step's rows (``ctx.token_ids``, and whatever else of the
+            step it needs: ``ctx.positions`` for a learned position table, ...).
   head      forward(normalised rows) -> float32 logits [R, V].
 
 A norm's kernel can be saved for steps of few rows, where a launch costs as much as the work.  This is
@@ -102,7 +103,8 @@ class Part:
 @dataclasses.dataclass
 class LayerCache:
     """The cache tensors of one schedule entry: K [pages, kv heads, page_size, d] and
-    V [pages, kv heads, d, page_size], and the cache group whose block tables index them."""
+    V [pages, kv heads, dv, page_size] (dv = d unless the mixer's ``CacheSpec`` says otherwise), and the cache
+    group whose block tables index them."""
     k: torch.Tensor
     v: torch.Tensor
     group: int

@@ -42,6 +42,8 @@ class PreNormBlock(Block):
     graph_safe = True
 
     def __init__(self, layer: LayerSpec, hidden_size: int):
+        if layer.norm_in is None or layer.norm_post is None or layer.ffn is None or layer.extra:
+            raise ValueError(f"layer {layer.prefix}: the prenorm block is two norms, a mixer and a feed-forward, no more and no less")
         self.prefix = layer.prefix
         self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)
         self.mixer = build_part("mixer", layer.mixer, hidden_size=hidden_size)

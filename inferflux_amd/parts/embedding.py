@@ -32,8 +32,8 @@ class TokenEmbedding(Part):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.table = tensors[f"{self.name}.weight"]
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        return ops.embedding(token_ids, self.table)
+    def forward(self, ctx) -> torch.Tensor:
+        return ops.embedding(ctx.token_ids, self.table)
 
 
 @register_part("head", "linear_head")

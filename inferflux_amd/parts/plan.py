@@ -21,16 +21,26 @@ class PartSpec:
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    """One layer: an arrangement (``block``) of two norms, a mixer and a feed-forward.
+    """One layer: an arrangement (``block``) of parts.  The arrangement decides which of them it uses: the
+    built-in "prenorm" block takes two norms, a mixer and a feed-forward; another block may leave the norms or
+    the feed-forward out (None) and take further parts by name from ``extra`` (category, spec): a third and
+    fourth norm, a second feed-forward, ...  Every layer has a mixer: it is what owns cache and state.
 
     ``prefix`` is the tensor-name prefix of the layer's weights ("model.layers.3").
     """
     prefix: str
     block: PartSpec
-    norm_in: PartSpec
+    norm_in: Optional[PartSpec]
     mixer: PartSpec
-    norm_post: PartSpec
-    ffn: PartSpec
+    norm_post: Optional[PartSpec] = None
+    ffn: Optional[PartSpec] = None
+    extra: Tuple[Tuple[str, str, PartSpec], ...] = ()      # (name, category, spec) of further parts
+
+    def extra_part(self, name: str) -> Tuple[str, PartSpec]:
+        for n, category, spec in self.extra:
+            if n == name:
+                return category, spec
+        raise KeyError(f"layer {self.prefix}: no extra part named '{name}' (has: {[n for n, _, _ in self.extra]})")
 
 
 @dataclasses.dataclass(frozen=True)
@@ -86,7 +96,8 @@ class ParamSpec:
 
 @dataclasses.dataclass(frozen=True)
 class CacheSpec:
-    """What a mixer keeps per token: keys and values of ``n_kv_heads`` x ``head_dim``.
+    """What a mixer keeps per token: keys of ``n_kv_heads`` x ``head_dim`` and values of ``n_kv_heads`` x
+    ``v_head_dim`` (None: as wide as the keys).
 
     ``window`` is None when every past token stays readable, or the number of most recent
     positions (the current one included) that the mixer reads; older pages are given back.
@@ -94,6 +105,18 @@ class CacheSpec:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def k_dim(self) -> int:
+        return self.head_dim
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    def bytes_per_token(self, element_size: int) -> int:
+        return self.n_kv_heads * (self.k_dim + self.v_dim) * element_size
 
 
 @dataclasses.dataclass(frozen=True)

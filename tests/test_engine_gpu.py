@@ -121,7 +121,7 @@ def test_parts_alone(sharp_folders):
     x = torch.randn(40, 144, generator=g)
     blk, p = model.blocks[1], "model.layers.1"
     # embedding
-    assert torch.equal(model.embedding.forward(ctx.token_ids).cpu().double(), W["model.embed_tokens.weight"][ids])
+    assert torch.equal(model.embedding.forward(ctx).cpu().double(), W["model.embed_tokens.weight"][ids])
     # norm (with and without a pending delta)
     delta = torch.randn(40, 144, generator=g)
     res = x.to(dev).clone()
@@ -639,3 +639,177 @@ def test_sizes_that_are_multiples_of_little(name, dtype, tmp_path):
            runner.step([StepEntry("a", ids[70:87], list(range(17)))]).cpu()]        # 17 rows: one more than a tile
     got += [runner.step([StepEntry("a", [ids[p]], [0])]).cpu() for p in range(87, 120)]
     assert rel_err(torch.cat(got), want) < REL_TOL[dtype]
+
+
+def test_a_toy_embedding_that_reads_positions_and_a_toy_mixer_with_narrow_values(tmp_path):
+    """Two parts from outside the package that need more of the step than the built-in ones: an embedding that adds
+    a learned table of absolute positions (it is given the step's context, not just the token ids), and an
+    attention whose values are narrower than its keys (d = 24, dv = 8: the cache spec, the storage, the planner's
+    bytes per token and the plain attention kernel all take the two widths).  Whole against cut, and against the
+    formulas written out."""
+    from inferflux_amd.engine.api import plan_kv_pages
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.kernels import ops
+    from inferflux_amd.parts import CacheSpec, LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec, ScheduleEntry, register_part
+    from inferflux_amd.parts.base import Part
+
+    H, V, nH, d, dv, MAXP = 40, 70, 2, 24, 8, 96
+
+    @register_part("embedding", "toy_token_plus_position")
+    class TokenPlusPosition(Part):
+        def __init__(self, name, vocab_size, hidden_size, max_position):
+            self.name, self.V, self.H, self.maxp = name, vocab_size, hidden_size, max_position
+        def param_specs(self):
+            return {f"{self.name}.tokens.weight": ParamSpec((self.V, self.H)),
+                    f"{self.name}.positions.weight": ParamSpec((self.maxp, self.H), ("normal", 0.05))}
+        def load(self, tensors):
+            self.tokens, self.positions = tensors[f"{self.name}.tokens.weight"], tensors[f"{self.name}.positions.weight"]
+        def forward(self, ctx):
+            return ops.embedding(ctx.token_ids, self.tokens) + ops.embedding(ctx.positions, self.positions)
+
+    @register_part("mixer", "toy_narrow_value_attention")
+    class NarrowValues(Mixer):
+        def __init__(self, name, hidden_size):
+            self.name, self.H = name, hidden_size
+        def cache_spec(self):
+            return CacheSpec(n_kv_heads=1, head_dim=d, v_head_dim=dv)
+        def param_specs(self):
+            n = self.name
+            return {f"{n}.q.weight": ParamSpec((nH * d, self.H), ("normal", 0.3)), f"{n}.k.weight": ParamSpec((d, self.H), ("normal", 0.3)),
+                    f"{n}.v.weight": ParamSpec((dv, self.H), ("normal", 0.3)), f"{n}.o.weight": ParamSpec((self.H, nH * dv), ("normal", 0.3))}
+        def load(self, tensors):
+            self.wq, self.wk, self.wv, self.wo = (tensors[f"{self.name}.{p}.weight"] for p in "qkvo")
+        def forward(self, h, ctx, binding):
+            cache = binding.cache
+            P = cache.page_size
+            slots = ctx.write_slots(cache.group).long()
+            k, v = h @ self.wk.t(), h @ self.wv.t()
+            cache.k[slots // P, 0, slots % P] = k                          # K [page][head][offset][d]
+            cache.v[slots // P, 0, :, slots % P] = v                       # V [page][head][dv][offset]
+            q = (h @ self.wq.t()).view(-1, nH, d).contiguous()
+            out = ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, ctx.block_table(cache.group), None, d ** -0.5)
+            return out @ self.wo.t()
+
+    p = "toy.layers.0"
+    layer = LayerSpec(p, PartSpec("prenorm"), PartSpec("rmsnorm", {"name": f"{p}.n1", "eps": 1e-5}),
+                      PartSpec("toy_narrow_value_attention", {"name": f"{p}.attn"}),
+                      PartSpec("rmsnorm", {"name": f"{p}.n2", "eps": 1e-5}),
+                      PartSpec("swiglu", {"name": f"{p}.mlp", "intermediate_size": 56}))
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=MAXP,
+                     embedding=PartSpec("toy_token_plus_position", {"name": "toy.embed", "vocab_size": V, "max_position": MAXP}),
+                     layers=(layer,), schedule=(ScheduleEntry(0),),
+                     final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
+    model = Model(plan=plan).init_random(9, torch.float32, "cuda")
+    runner = ModelRunner(model, num_pages=8, max_requests=2)
+    cache = runner.storage.binding(0).cache
+    assert tuple(cache.k.shape) == (8, 1, 16, d) and tuple(cache.v.shape) == (8, 1, dv, 16)
+    assert runner.storage.bytes_per_token() == (d + dv) * 4
+    assert plan_kv_pages(model, 16, 16 * 5) == 5                        # (sized by tokens; the bytes only cap it)
+    ids = seeded_ids(31, 60, V)
+    runner.add_request("w")
+    whole = runner.step([StepEntry("w", ids, list(range(60)))]).cpu()
+    runner.free_request("w")
+    runner.add_request("o"); runner.add_request("c")
+    rows, at = [], 0
+    for m in (13, 1, 2, 30, 1, 13):
+        rows.append(runner.step([StepEntry("o", ids[at:at + 1], []), StepEntry("c", ids[at:at + m], list(range(m)))]).cpu()[:m])
+        at += m
+    assert torch.allclose(torch.cat(rows), whole, rtol=1e-4, atol=1e-5)
+    # the formulas, plainly
+    emb, att, blk = model.embedding, model.blocks[0].mixer, model.blocks[0]
+    D = lambda t: t.double().cpu()
+    x = D(emb.tokens)[ids] + D(emb.positions)[:60]
+    h = pm.rms_norm(x, D(blk.norm_in.weight), 1e-5)
+    q, k, v = (h @ D(att.wq).t()).view(60, nH, d), (h @ D(att.wk).t()).view(60, 1, d), (h @ D(att.wv).t()).view(60, 1, dv)
+    s = torch.einsum("ihd,jd->hij", q, k[:, 0]) * d ** -0.5
+    s = s.masked_fill(torch.triu(torch.ones(60, 60, dtype=torch.bool), 1), float("-inf"))
+    o = torch.einsum("hij,je->ihe", torch.softmax(s, -1), v[:, 0]).reshape(60, nH * dv)
+    x = x + o @ D(att.wo).t()
+    h = pm.rms_norm(x, D(blk.norm_post.weight), 1e-5)
+    x = x + pm.swiglu(h, D(blk.ffn.w_gate_up.rows)[0::2], D(blk.ffn.w_gate_up.rows)[1::2], D(blk.ffn.w_down.rows))
+    want = pm.rms_norm(x, D(model.final_norm.weight), 1e-5) @ D(model.head.weight.rows).t()
+    assert torch.allclose(whole.double(), want, rtol=1e-3, atol=1e-4)
+    # the position table matters: without it the logits are others
+    emb.positions.zero_()
+    runner.free_request("o")
+    runner.add_request("z")
+    assert not torch.allclose(runner.step([StepEntry("z", ids[:10], list(range(10)))]).cpu(), whole[:10], rtol=1e-2, atol=1e-3)
+
+
+def test_a_toy_block_with_four_norms_and_no_feed_forward():
+    """An arrangement from outside the package that the built-in one does not cover: pre-norm, attention, a norm on
+    the attention's output before the add, a norm on the skip path, and no feed-forward at all; the two further
+    norms come from the layer spec's named extras.  It is registered, built and stepped; whole equals cut; and
+    the formulas written out."""
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.parts import Block, LayerSpec, ModelPlan, PartSpec, ScheduleEntry, build_part, register_part
+
+    H, V, nH, d = 48, 80, 3, 16
+
+    @register_part("block", "toy_sandwich_without_ffn")
+    class Sandwich(Block):
+        def __init__(self, layer, hidden_size):
+            assert layer.ffn is None and layer.norm_post is None
+            self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)
+            self.mixer = build_part("mixer", layer.mixer, hidden_size=hidden_size)
+            self.norm_out = build_part(*layer.extra_part("norm_out"), hidden_size=hidden_size)
+            self.norm_skip = build_part(*layer.extra_part("norm_skip"), hidden_size=hidden_size)
+        def children(self):
+            return (self.norm_in, self.mixer, self.norm_out, self.norm_skip)
+        def forward(self, residual, pending, ctx, binding):
+            h = self.norm_in.forward(residual, pending, ctx.act_dtype)            # (adds what the block before left pending)
+            delta = self.mixer.forward(h, ctx, binding).float()
+            normed = self.norm_out.forward(delta, None, torch.float32)            # a norm on the sub-block's output
+            skip = self.norm_skip.forward(residual.clone(), None, torch.float32)  # and one on the skip path
+            residual.copy_(skip)
+            return residual, normed.to(ctx.act_dtype)
+
+    def layer(i):
+        p = f"toy.layers.{i}"
+        return LayerSpec(p, PartSpec("toy_sandwich_without_ffn"), PartSpec("rmsnorm", {"name": f"{p}.n_in", "eps": 1e-5}),
+                         PartSpec("paged_attention", {"name": f"{p}.attn", "n_heads": nH, "n_kv_heads": 1, "head_dim": d, "bias": False,
+                                                      "position": PartSpec("rotary", {"head_dim": d, "theta": 100.0})}),
+                         extra=(("norm_out", "norm", PartSpec("rmsnorm", {"name": f"{p}.n_out", "eps": 1e-5})),
+                                ("norm_skip", "norm", PartSpec("rmsnorm", {"name": f"{p}.n_skip", "eps": 1e-4}))))
+
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=128,
+                     embedding=PartSpec("token_embedding", {"name": "toy.embed", "vocab_size": V}),
+                     layers=(layer(0), layer(1)), schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+                     final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
+    with pytest.raises(KeyError, match="no extra part named 'nope'"):
+        plan.layers[0].extra_part("nope")
+    model = Model(plan=plan).init_random(12, torch.float32, "cuda")
+    names = set(model.param_specs())
+    assert {"toy.layers.0.n_out.weight", "toy.layers.1.n_skip.weight"} <= names and not any(".mlp." in n for n in names)
+    runner = ModelRunner(model, num_pages=8, max_requests=2)
+    ids = seeded_ids(41, 50, V)
+    runner.add_request("w")
+    whole = runner.step([StepEntry("w", ids, list(range(50)))]).cpu()
+    runner.free_request("w")
+    runner.add_request("c")
+    rows, at = [], 0
+    for m in (20, 1, 2, 26, 1):
+        rows.append(runner.step([StepEntry("c", ids[at:at + m], list(range(m)))]).cpu()); at += m
+    assert torch.allclose(torch.cat(rows), whole, rtol=1e-4, atol=1e-5)
+    D = lambda t: t.double().cpu()
+    x, pending = D(model.embedding.table)[ids], 0.0
+    for b in model.blocks:
+        x = x + pending
+        h = pm.rms_norm(x, D(b.norm_in.weight), 1e-5)
+        att = b.mixer
+        qkv = h @ D(att.w_qkv.rows).t()
+        q, k, v = qkv[:, :nH * d].view(50, nH, d), qkv[:, nH * d:(nH + 1) * d].view(50, 1, d), qkv[:, (nH + 1) * d:].view(50, 1, d)
+        pos = list(range(50))
+        q, k = pm.rope_split_half(q, pos, 100.0), pm.rope_split_half(k, pos, 100.0)
+        delta = pm.attention(q, k, v).reshape(50, nH * d) @ D(att.w_o.rows).t()
+        pending = pm.rms_norm(delta, D(b.norm_out.weight), 1e-5)
+        x = pm.rms_norm(x, D(b.norm_skip.weight), 1e-4)
+    want = pm.rms_norm(x + pending, D(model.final_norm.weight), 1e-5) @ D(model.head.weight.rows).t()
+    assert torch.allclose(whole.double(), want, rtol=1e-3, atol=1e-4)
+    # the built-in arrangement refuses a layer it cannot be
+    with pytest.raises(ValueError, match="no more and no less"):
+        build_part("block", PartSpec("prenorm"), layer=plan.layers[0], hidden_size=H)
