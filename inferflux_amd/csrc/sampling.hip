@@ -13,6 +13,9 @@
 // a filter keeps every token whose weight is >= its threshold, found by bisection over the
 // bit patterns of positive floats, so tokens of equal weight are kept or dropped together.
 #include "common.h"
+#include "sampling.h"
+
+#include <mutex>
 
 IFX_DEFINE_LAST_ERROR()
 
@@ -100,6 +103,48 @@ extern "C" int ifx_argmax(const float* logits, int R, int V, int* out, float* sc
     hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, s, logits, V, out);
   }
   IFX_LAUNCH_CHECK();
+}
+
+// The same two stages with their scratch in a file-scope device array instead of a workspace of the caller's: the entry
+// point for callers that cannot allocate (see sampling.h).  In host code the array's name is only a stand-in for the
+// symbol: the address the kernels are given is looked up per device with hipGetSymbolAddress, once, and kept.
+#define ARGMAX_STATIC_BYTES (IFX_ARGMAX_STATIC_MAX_ROWS * ARGMAX_SLICES * (sizeof(float) + sizeof(int)))
+static __device__ __align__(256) unsigned char scratch[ARGMAX_STATIC_BYTES];
+
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static void* g_scratch_ptr[ARGMAX_STATIC_MAX_DEVICES];   // per device: that device's copy of `scratch`, or null before its first call
+static std::mutex g_scratch_mutex;
+
+// The address of the current device's `scratch` (each GPU holds its own copy at its own address).
+static int argmax_static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) IFX_FAIL("argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  IFX_REQUIRE(dev >= 0 && dev < ARGMAX_STATIC_MAX_DEVICES, "argmax_static: device %d outside 0..%d", dev, ARGMAX_STATIC_MAX_DEVICES - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      IFX_FAIL("argmax_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int ifx_argmax_static(const float* logits, int R, int V, int* out, void* stream) {
+  IFX_REQUIRE(R >= 0 && V > 0, "argmax_static: bad sizes R=%d V=%d", R, V);
+  IFX_REQUIRE(R <= IFX_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows, the static scratch holds at most %d", R,
+              IFX_ARGMAX_STATIC_MAX_ROWS);
+  if (R == 0) return 0;
+  IFX_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: null logits or out");
+  void* ptr = nullptr;
+  if (const int rc = argmax_static_scratch(&ptr)) return rc;
+  // the floats of all R rows first, then the ints (both 4 bytes wide, so both parts stay aligned)
+  float* pv = (float*)ptr;
+  int* pi = (int*)((unsigned char*)ptr + (size_t)IFX_ARGMAX_STATIC_MAX_ROWS * ARGMAX_SLICES * sizeof(float));
+  return ifx_argmax(logits, R, V, out, pv, pi, stream);
 }
 
 // ---------------------------------------------------------------------------------------

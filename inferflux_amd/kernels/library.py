@@ -74,7 +74,9 @@ def _cxx() -> str:
 def _digest(name: str, variant: Variant) -> str:
     h = hashlib.sha256()
     host = _is_host_module(name)
-    for fn in ((f"{name}.cpp",) if host else (f"{name}.hip", "common.h")):
+    for fn in ((f"{name}.cpp",) if host else (f"{name}.hip", "common.h", f"{name}.h")):
+        if fn == f"{name}.h" and not os.path.isfile(os.path.join(CSRC, fn)):
+            continue                    # a module's own header (its public entry points), where it has one
         with open(os.path.join(CSRC, fn), "rb") as f:
             h.update(f.read())
     h.update(" ".join(HOST_FLAGS if host else FLAGS).encode())
