@@ -132,10 +132,40 @@ def seeded_ids(seed, n, vocab):
 
 # Logits are compared relative to the largest logit of the row set: a float32 engine differs from
 # the float64 plain model by rounding that accumulates over a few hundred operations; a bfloat16
-# engine rounds every activation to 8 bits of mantissa.
-REL_TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+# engine rounds every activation to 8 bits of mantissa.  The bfloat16 bounds are per configuration: the
+# largest error any test of that configuration shows (A 0.96 %, B 1.33 %, C 2.51 %: its window makes single
+# scores count for more; other shapes up to 1.3 %) and half as much again.  INFERFLUX_REL_ERR_LOG (below)
+# writes what a run shows.
+REL_TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+BF16_TOL = {"A": 1.5e-2, "B": 2e-2, "C": 3.7e-2}
+
+
+def tol(dtype, name=None):
+    """The bound for logits of configuration ``name`` (a key of TINY, or None for any other shape) in ``dtype``."""
+    if dtype == "bfloat16":
+        return BF16_TOL.get(name, REL_TOL["bfloat16"])
+    return REL_TOL[dtype]
+
+
+_REL_ERRS = []      # (test id, error) of every comparison of a run, for the summary below
 
 
 def rel_err(got, want):
     want = want.double()
-    return float((got.double() - want).abs().max() / want.abs().max())
+    e = float((got.double() - want).abs().max() / want.abs().max())
+    _REL_ERRS.append((os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0], e))
+    return e
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """With INFERFLUX_REL_ERR_LOG=path: the largest relative error each test saw, one line a test, into that file
+    (what the tolerances above are set from)."""
+    path = os.environ.get("INFERFLUX_REL_ERR_LOG")
+    if not path or not _REL_ERRS:
+        return
+    worst = {}
+    for test, e in _REL_ERRS:
+        worst[test] = max(worst.get(test, 0.0), e)
+    with open(path, "w") as f:
+        for test, e in sorted(worst.items()):
+            f.write(f"{e:.3e}  {test}\n")

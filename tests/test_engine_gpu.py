@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import plain_model as pm
-from conftest import REL_TOL, TINY, plain_logits, rel_err, seeded_ids
+from conftest import REL_TOL, TINY, plain_logits, rel_err, seeded_ids, tol
 
 pytestmark = pytest.mark.gpu
 
@@ -34,7 +34,7 @@ def test_whole_prompt(name, dtype, sharp_folders):
     for n in (1, 2, 29, 200):
         ids = seeded_ids(n, n, TINY[name]["vocab_size"])
         got = run_whole(runner, "a", ids)
-        assert rel_err(got, plain_logits(folder, ids)) < REL_TOL[dtype], (name, n)
+        assert rel_err(got, plain_logits(folder, ids)) < tol(dtype, name), (name, n)
     runner.manager.check()
     assert runner.manager.free_pages() == [32] * len(runner.manager.groups)
 
@@ -62,7 +62,7 @@ def test_long_decoding_stays_on_the_plain_model(dtype, sharp_folders):
     for p in range(5, 300):
         got.append(runner.step([StepEntry("d", [ids[p]], [0])]).cpu()[0])
         runner.manager.check()
-    assert rel_err(torch.stack(got), want[4:]) < REL_TOL[dtype]
+    assert rel_err(torch.stack(got), want[4:]) < tol(dtype, name)
     # the windowed group kept only the pages a window of 24 can still see
     held = sum(1 for p in runner.manager.block_table("d", 1) if p >= 0)
     assert held <= 24 // 16 + 2 and sum(1 for p in runner.manager.block_table("d", 0) if p >= 0) == -(-300 // 16)
@@ -283,8 +283,8 @@ def test_steps_of_few_rows_need_no_kernel_for_the_norms_between_products(name, s
     yield_calls = []
     separate = run(load_runner(folder, torch.bfloat16, num_pages=16))
     assert all(n == 2 * L + 1 for _, n in yield_calls), yield_calls
-    assert rel_err(fused, want[:60]) < REL_TOL["bfloat16"] and rel_err(separate, want[:60]) < REL_TOL["bfloat16"]
-    assert rel_err(fused, separate) < REL_TOL["bfloat16"]
+    assert rel_err(fused, want[:60]) < tol("bfloat16", name) and rel_err(separate, want[:60]) < tol("bfloat16", name)
+    assert rel_err(fused, separate) < tol("bfloat16", name)
 
 
 def test_a_decode_step_started_before_the_host_has_its_tokens(sharp_folders):
@@ -424,7 +424,7 @@ def test_portions_of_every_product_size_with_and_without_the_decode_copy(name, c
     got, at = [], 0
     for m in (40, 17, 3, 64, 1, 16, 70, 1):
         got.append(runner.step([StepEntry("p", ids[at:at + m], list(range(m)))]).cpu()); at += m
-    assert at == 212 and rel_err(torch.cat(got), want) < REL_TOL["bfloat16"]
+    assert at == 212 and rel_err(torch.cat(got), want) < tol("bfloat16", name)
     runner.free_request("p")
 
 
@@ -467,7 +467,7 @@ def test_replayed_decode_graphs_equal_eager_steps(name, dtype, sharp_folders):
             assert torch.allclose(got, want, rtol=0, atol=0), (who, pos)   # same kernels, same order: equal bits
     assert replays > 60 and len(graphed._graphs) >= 4
     want = plain_logits(folder, seqs["a"][: pos["a"]])[-1]
-    assert rel_err(got[0], want) < REL_TOL[dtype]
+    assert rel_err(got[0], want) < tol(dtype, name)
 
 
 # ---- other toy parts: a position encoding of its own, a feed-forward with routing --------------------
@@ -575,7 +575,7 @@ def test_other_page_sizes(page_size, dtype, sharp_folders):
         got = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).cpu()
         if s["step"] in expected:
             want = torch.stack([plain_logits(folder, seqs[rid])[p] for rid, p in expected[s["step"]]])
-            assert rel_err(got, want) < REL_TOL[dtype], s["step"]
+            assert rel_err(got, want) < tol(dtype, "C"), s["step"]
         for rid in s["end"]:
             runner.free_request(rid)
         runner.manager.check()
@@ -599,7 +599,7 @@ def test_prompt_portions_with_a_long_past_split_their_keys(sharp_folders, monkey
         pos = 0
         for n in portions:
             got = runner.step([StepEntry("p", ids[pos:pos + n], list(range(n)))]).cpu()
-            assert rel_err(got, want[pos:pos + n]) < REL_TOL["bfloat16"], (name, pos)
+            assert rel_err(got, want[pos:pos + n]) < tol("bfloat16", name), (name, pos)
             pos += n
         runner.free_request("p")
     assert max(calls) > 1      # some portion did run in splits

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 import traces
-from conftest import REL_TOL, ROOT, TINY, plain_logits, rel_err, seeded_ids
+from conftest import REL_TOL, tol, ROOT, TINY, plain_logits, rel_err, seeded_ids
 
 pytestmark = pytest.mark.gpu
 
@@ -36,7 +36,7 @@ def replay(folder, dtype, steps, out_dir, max_tokens):
             proc.kill()
 
 
-def check(folder, dtype, seqs, expected, out_dir, vocab):
+def check(folder, dtype, seqs, expected, out_dir, vocab, name):
     worst = 0.0
     for step, rows in expected.items():
         got = np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4")
@@ -45,7 +45,7 @@ def check(folder, dtype, seqs, expected, out_dir, vocab):
         want = torch.stack([plain_logits(folder, seqs[rid])[p] for rid, p in rows])
         assert torch.isfinite(got).all(), f"step {step}"
         e = rel_err(got, want)
-        assert e < REL_TOL[dtype], f"step {step} rows {rows[:4]}...: relative error {e:.3g}"
+        assert e < tol(dtype, name), f"step {step} rows {rows[:4]}...: relative error {e:.3g}"
         worst = max(worst, e)
     return worst
 
@@ -71,4 +71,4 @@ def test_all_cuttings_match_the_plain_model(name, dtype, sharp_folders, tmp_path
     replay(folder, dtype, all_steps, out, max_tokens)
     files = sorted(int(f[:-4]) for f in os.listdir(out))
     assert files == sorted(all_expected), "a logits file for every step that wants something, and no other"
-    check(folder, dtype, seqs, all_expected, out, vocab)
+    check(folder, dtype, seqs, all_expected, out, vocab, name)
