@@ -4,8 +4,12 @@
 
 A step is one decode step of the whole engine (scheduler, step function, sampling).  Prints one
 JSON line: decoded tokens a second at batch 8 as ``value``, the same at batch 1 and 64 under
-``points``, a 2,048-token prefill under ``prefill`` and the decode step's share of the HBM
-roofline under ``roofline``.
+``points`` (with their step times and roofline shares under ``ms_per_step_b1`` / ``roofline_b1`` and
+``..._b64``), a 2,048-token prefill under ``prefill`` (the best of ``best_of`` runs with the library's
+kernels chosen by timing; ``prefill_untuned`` is the same with the library's default choice) and the
+decode step's share of the HBM roofline under ``roofline``.  Every share is given against the data
+sheet (``frac``) and, unless ``--no-ceilings``, against what this card gives a kernel that only reads
+memory or a large library product (``frac_measured``, the ceilings under ``ceilings``).
 """
 import argparse
 import json
@@ -29,6 +33,9 @@ SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, num_hidden_layers=48, num_attention
 WORKLOADS = {
     "mixed3b": dict(shape=SHAPE_3B, name="Qwen2.5-3B shape", requests=64, prompt=(128, 2048), new=256, chunk=512),
     "long14b": dict(shape=SHAPE_14B, name="Qwen2.5-14B shape", requests=32, prompt=(8192, 8192), new=512, chunk=2048),
+    # requests that finish one by one: the decode batch shrinks a request at a time, which is what captured decode
+    # steps (one graph per layout) like least
+    "staggered": dict(shape=SHAPE_7B, name="Qwen2.5-7B shape", requests=64, prompt=(512, 512), new=(32, 512), chunk=512),
 }
 CONTEXT = 4096
 PROMPT = 2048
@@ -51,10 +58,15 @@ def main() -> int:
                          "(for profiles); mixed3b / long14b: whole workloads through the scheduler")
     ap.add_argument("--no-decode-weight-copy", action="store_true",
                     help="decode from the weights' plain rows instead of the tiled copy")
+    ap.add_argument("--ceilings", action=argparse.BooleanOptionalAction, default=True,
+                    help="measure what the card gives (a 2 GB streaming read, an 8192^3 bf16 library product) once and "
+                         "report every share against it beside the data sheet's peak")
+    ap.add_argument("--context", type=int, default=DECODE_KV_START, help="tokens each request holds when the timed decode steps start")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    kv_start = args.context
 
     import torch
     from inferflux_amd import SamplingParams
@@ -103,14 +115,14 @@ def main() -> int:
         return Engine(runner, SchedulerConfig(max_batch_size=batch, max_batch_tokens=16384, chunked_prefill_tokens=2048))
 
     def decode_rate(batch, steps, warmup):
-        """tokens/s and ms/step of ``steps`` decode steps at ``batch`` with contexts from DECODE_KV_START."""
+        """tokens/s and ms/step of ``steps`` decode steps at ``batch`` with contexts from ``--context``."""
         # While the last prompts are still coming in, the first requests already decode: give every
         # request enough tokens (and pages) that none finishes before the timed steps are over.
-        slack = -(-batch * DECODE_KV_START // 16384) + 2
-        eng = make_engine(batch, DECODE_KV_START + steps + warmup + slack + 2)
+        slack = -(-batch * kv_start // 16384) + 2
+        eng = make_engine(batch, kv_start + steps + warmup + slack + 2)
         sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + slack + 1, ignore_eos=True)
         for _ in range(batch):
-            eng.add_request(torch.randint(0, V, (DECODE_KV_START,), generator=gen).tolist(), SamplingParams(**vars(sp)))
+            eng.add_request(torch.randint(0, V, (kv_start,), generator=gen).tolist(), SamplingParams(**vars(sp)))
         while any(s.is_prefilling for s in eng.scheduler.running) or eng.scheduler.waiting:
             eng.step()                                            # prompts in; every request now decodes
         note(f"batch {batch}: prompts are in, decoding")
@@ -125,15 +137,17 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         assert len(eng.scheduler.running) == batch and eng.stats.preemptions == 0, "a request finished or was preempted while timing"
-        kv_mean = DECODE_KV_START + warmup + steps / 2
+        kv_mean = kv_start + warmup + steps / 2
         del eng
         torch.cuda.empty_cache()
         return batch * steps / dt, dt / steps * 1e3, kv_mean
 
     def prefill_rate(tokens, reps=3):
+        """(tokens/s, ms, share of the matrix peak, mean ms) of a prompt of ``tokens`` in one step: the best of ``reps``
+        runs after one that warms up (and, with tuning on, lets the library time its kernels for these shapes)."""
         runner = ModelRunner(model, num_pages=-(-tokens // PAGE) + 1, page_size=PAGE, max_requests=2)
         ids = torch.randint(0, V, (tokens,), generator=gen).tolist()
-        best = None
+        times = []
         ops.pause_library_gemm_tuning(False)
         for i in range(reps + 1):
             runner.add_request(i)
@@ -146,13 +160,38 @@ def main() -> int:
             ops.pause_library_gemm_tuning(True)
             note(f"prefill of {tokens} tokens: {dt * 1e3:.1f} ms")
             if i > 0:
-                best = dt if best is None else min(best, dt)
+                times.append(dt)
+        best = min(times)
         linear = 2.0 * tokens * L * ((nH + 2 * nKV) * d * H + nH * d * H + 3 * I * H) + 2.0 * V * H
         attn = 4.0 * L * nH * d * tokens * (tokens + 1) / 2
-        return tokens / best, best * 1e3, (linear + attn) / best / 1e12 / PEAK_TFLOPS[args.dtype]
+        return tokens / best, best * 1e3, (linear + attn) / best / 1e12 / PEAK_TFLOPS[args.dtype], sum(times) / len(times) * 1e3
+
+    def measured_ceilings():
+        """What this card gives a kernel that only reads 2 GB (streaming loads), and the library's 8192^3 bfloat16
+        product: the yardsticks beside the data sheet's 8 TB/s and 2.5 PFLOP/s."""
+        from inferflux_amd.kernels.microbench import _time_us
+        pool = torch.zeros((6 << 30) // 4, dtype=torch.float32, device=dev)
+        n = (2 << 30) // 4
+        t = min(_time_us(lambda i: ops.stream_read(pool[(i % 3) * n:(i % 3 + 1) * n], 2048, True), 6) for _ in range(2))
+        read = (2 << 30) / t / 1e3                    # GB/s
+        del pool
+        a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        t = min(_time_us(lambda i: torch.matmul(a, b.t()), 6) for _ in range(2))
+        del a, b
+        torch.cuda.empty_cache()
+        return {"read_2GB_GBs": round(read, 1), "library_bf16_8192_TFLOPs": round(2 * 8192 ** 3 / t / 1e6, 1)}
+
+    def hbm_roofline(batch, ms, kv_mean, ceil):
+        step_bytes = weight_bytes + batch * kv_mean * kv_bytes_per_token
+        achieved = step_bytes / (ms * 1e-3) / 1e9
+        r = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)}
+        if ceil:
+            r["frac_measured"] = round(achieved / ceil["read_2GB_GBs"], 4)
+        return r
 
     if args.workload == "prefill":
-        ptps, pms, pfrac = prefill_rate(PROMPT, reps=args.steps)
+        ptps, pms, pfrac, _ = prefill_rate(PROMPT, reps=args.steps)
         print(json.dumps({"metric": f"prefill tok/s, {PROMPT} tokens (Qwen2.5-7B shape, {args.dtype}, random weights)",
                           "value": round(ptps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": 1,
                           "ms_per_step": round(pms, 3), "higher_is_better": True, "dtype": args.dtype,
@@ -160,10 +199,11 @@ def main() -> int:
                                      "prompt_len": PROMPT, "library_gemm_tuning": not args.no_gemm_tuning},
                           "frac_of_peak": round(pfrac, 4)}), flush=True)
         return 0
+    ceil = measured_ceilings() if (args.ceilings and args.dtype == "bf16") else None
+    if ceil:
+        note(f"this card: {ceil['read_2GB_GBs']:.0f} GB/s for a 2 GB read, {ceil['library_bf16_8192_TFLOPs']:.0f} TFLOP/s for the library's 8192^3 product")
     tps, ms, kv_mean = decode_rate(args.batch, args.steps, max(args.warmup, 1))
     note(f"batch {args.batch}: {tps:.0f} tokens/s")
-    step_bytes = weight_bytes + args.batch * kv_mean * kv_bytes_per_token
-    achieved = step_bytes / (ms * 1e-3) / 1e9
     out = {
         "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-7B shape, {args.dtype}, random weights)",
         "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -172,18 +212,36 @@ def main() -> int:
         "config": {"model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "1 GPU",
                    "num_hidden_layers": layers_full, "layers_run": L, "hidden_size": H, "num_attention_heads": nH,
                    "num_key_value_heads": nKV, "head_dim": d, "intermediate_size": I, "vocab_size": V,
-                   "prompt_len": PROMPT, "decode_kv_start": DECODE_KV_START, "kv_page_size": PAGE,
+                   "prompt_len": PROMPT, "decode_kv_start": kv_start, "kv_page_size": PAGE,
                    "tie_word_embeddings": False, "library_gemm_tuning": not args.no_gemm_tuning,
                    "decode_weight_copy": not args.no_decode_weight_copy},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_GBS, 4)},
+        "roofline": hbm_roofline(args.batch, ms, kv_mean, ceil),
     }
+    if ceil:
+        out["ceilings"] = ceil
     if not args.no_points:
-        ptps, pms, pfrac = prefill_rate(PROMPT)
-        out["prefill"] = {"value": round(ptps, 1), "tokens": PROMPT, "ms": round(pms, 3), "frac": round(pfrac, 4)}
-        b1 = decode_rate(1, min(args.steps, 32), min(args.warmup, 4))[0]
-        b64 = decode_rate(64, min(args.steps, 32), min(args.warmup, 4))[0]
-        out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+        reps = 3
+        ptps, pms, pfrac, pmean = prefill_rate(PROMPT, reps)
+        out["prefill"] = {"value": round(ptps, 1), "tokens": PROMPT, "ms": round(pms, 3), "frac": round(pfrac, 4),
+                          "best_of": reps, "mean_ms": round(pmean, 3), "library_gemm_tuning": not args.no_gemm_tuning}
+        if ceil:
+            out["prefill"]["frac_measured"] = round(pfrac * PEAK_TFLOPS[args.dtype] / ceil["library_bf16_8192_TFLOPs"], 4)
+        if not args.no_gemm_tuning:
+            # the same prefill with the library's own default choice of kernels (no timing of candidates, no file of
+            # earlier choices): what a first call gets
+            import torch.cuda.tunable as tunable
+            tunable.enable(False)
+            utps, ums, ufrac, umean = prefill_rate(PROMPT, reps)
+            tunable.enable(True)
+            out["prefill_untuned"] = {"value": round(utps, 1), "tokens": PROMPT, "ms": round(ums, 3), "frac": round(ufrac, 4),
+                                      "best_of": reps, "mean_ms": round(umean, 3)}
+        points = {}
+        for b in (1, 64):
+            btps, bms, bkv = decode_rate(b, min(args.steps, 32), min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(btps, 2)
+            out[f"ms_per_step_b{b}"] = round(bms, 4)
+            out[f"roofline_b{b}"] = hbm_roofline(b, bms, bkv, ceil)
+        out["points"] = points
     print(json.dumps(out), flush=True)
     return 0
 
@@ -209,7 +267,9 @@ def run_workload(args, w) -> int:
     lo, hi = w["prompt"]
     lens = torch.randint(lo, hi + 1, (w["requests"],), generator=gen).tolist()
     prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lens]
-    pages = sum(-(-(n + w["new"]) // PAGE) + 1 for n in lens)
+    new_lo, new_hi = w["new"] if isinstance(w["new"], tuple) else (w["new"], w["new"])
+    news = torch.randint(new_lo, new_hi + 1, (w["requests"],), generator=gen).tolist()
+    pages = sum(-(-(n + m) // PAGE) + 1 for n, m in zip(lens, news))
     runner = ModelRunner(model, num_pages=pages, page_size=PAGE, max_requests=w["requests"])
     eng = Engine(runner, SchedulerConfig(max_batch_size=w["requests"], max_batch_tokens=16384, chunked_prefill_tokens=w["chunk"]))
     first, t0 = {}, time.perf_counter()
@@ -218,27 +278,28 @@ def run_workload(args, w) -> int:
         if rid not in first:
             first[rid] = time.perf_counter() - t0
 
-    sp = SamplingParams(temperature=0.0, max_tokens=w["new"], ignore_eos=True)
+    sps = lambda: [SamplingParams(temperature=0.0, max_tokens=m, ignore_eos=True) for m in news]
     if args.warmup > 0:
         # One untimed pass of the same workload: the library loads a kernel the first time a shape asks
         # for it, which costs up to a second per shape and has nothing to do with the steady state.
-        eng.generate(prompts, SamplingParams(**vars(sp)))
+        eng.generate(prompts, sps())
         eng.stats = type(eng.stats)()
-        print("[bench] warm-up pass done", file=sys.stderr, flush=True)
+        print(f"[bench] warm-up pass done ({runner.graph_captures} decode layouts captured)", file=sys.stderr, flush=True)
+    captures_before, replays_before = runner.graph_captures, runner.graph_replays
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    outs = eng.generate(prompts, sp, on_token)
+    outs = eng.generate(prompts, sps(), on_token)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     n_gen = sum(len(o.token_ids) for o in outs)
     ttft = sorted(first.values())
     out = {
-        "metric": f"generated tok/s, {w['requests']} requests, prompts {lo}-{hi}, {w['new']} new tokens each ({w['name']}, {args.dtype}, random weights)",
+        "metric": f"generated tok/s, {w['requests']} requests, prompts {lo}-{hi}, {new_lo}-{new_hi} new tokens each ({w['name']}, {args.dtype}, random weights)",
         "value": round(n_gen / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": eng.stats.steps,
         "warmup": 1 if args.warmup > 0 else 0,
         "ms_per_step": round(dt / eng.stats.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (uniform random token ids, seeded N(0,0.02) weights)",
-        "config": {"model": w["name"], "global_batch": w["requests"], "seq_len": hi + w["new"], "parallelism": "1 GPU",
+        "config": {"model": w["name"], "global_batch": w["requests"], "seq_len": hi + new_hi, "parallelism": "1 GPU",
                    "num_hidden_layers": w["shape"]["num_hidden_layers"], "layers_run": cfg.num_hidden_layers,
                    "hidden_size": cfg.hidden_size, "num_attention_heads": cfg.num_attention_heads,
                    "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
@@ -247,6 +308,8 @@ def run_workload(args, w) -> int:
         "total_s": round(dt, 2), "prompt_tok_per_s_overall": round(sum(lens) / dt, 1),
         "ttft_s": {"min": round(ttft[0], 3), "median": round(ttft[len(ttft) // 2], 3), "max": round(ttft[-1], 3)},
         "preemptions": eng.stats.preemptions,
+        "decode_graphs": {"captured_in_timed_pass": runner.graph_captures - captures_before,
+                          "captured_in_all": runner.graph_captures, "replays_in_timed_pass": runner.graph_replays - replays_before},
         "steps_by_tokens": {f"<={k}": n for k, n in sorted(eng.stats.step_tokens.items())},
     }
     print(json.dumps(out), flush=True)

@@ -55,6 +55,9 @@ class CacheStorage:
         self.manager = CacheManager(self.groups, page_size, counts, max_requests) if self.groups else \
             CacheManager([], page_size, [], max_requests)
         self.page_size, self.dtype, self.device = page_size, dtype, device
+        # One page more than the manager hands out, at the end of every cache tensor: the scratch page, which rows
+        # that stand for nobody (padding of a captured decode step's batch) write to and read back.
+        self.scratch_pages = list(counts)
         self._caches: Dict[int, LayerCache] = {}
         self._states: Dict[int, torch.Tensor] = {}
         for i, e in enumerate(schedule):
@@ -63,8 +66,8 @@ class CacheStorage:
             if spec is not None and e.cache_from is None:
                 g = self.entry_group[i]
                 n = counts[g]
-                k = torch.zeros((n, spec.n_kv_heads, page_size, spec.k_dim), dtype=dtype, device=device)
-                v = torch.zeros((n, spec.n_kv_heads, spec.v_dim, page_size), dtype=dtype, device=device)
+                k = torch.zeros((n + 1, spec.n_kv_heads, page_size, spec.k_dim), dtype=dtype, device=device)
+                v = torch.zeros((n + 1, spec.n_kv_heads, spec.v_dim, page_size), dtype=dtype, device=device)
                 self._caches[i] = LayerCache(k, v, g, page_size)
             st = m.state_spec()
             if st is not None:

@@ -30,28 +30,66 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
+def _pad_arrays(arrays, n_pad: int, scratch_pages: Sequence[int], page_size: int):
+    """``arrays`` of a step (``CacheManager.step_arrays``) with ``n_pad`` rows that stand for nobody appended: each is
+    a request of its own with one token at position 0 whose key and value go to the group's scratch page (a page
+    outside every pool, which nobody's block table names) and which reads that one key back.  Such rows keep a
+    step's layout the same while the number of real requests changes; what they compute is thrown away."""
+    R, T = arrays["q_len"].shape[0], arrays["positions"].shape[0]
+    i32 = lambda v: np.asarray(v, dtype=np.int32)
+    out = dict(arrays)
+    out["start"] = np.concatenate([arrays["start"], np.zeros(n_pad, np.int32)])
+    out["q_start"] = np.concatenate([arrays["q_start"], i32(np.arange(T, T + n_pad))])
+    out["q_len"] = np.concatenate([arrays["q_len"], np.ones(n_pad, np.int32)])
+    out["kv_len"] = np.concatenate([arrays["kv_len"], np.ones(n_pad, np.int32)])
+    out["state_slots"] = np.concatenate([arrays["state_slots"], np.zeros(n_pad, np.int32)])
+    out["row_req"] = np.concatenate([arrays["row_req"], i32(np.arange(R, R + n_pad))])
+    out["positions"] = np.concatenate([arrays["positions"], np.zeros(n_pad, np.int32)])
+    tables, slots = [], []
+    for g, bt in enumerate(arrays["block_tables"]):
+        pad = np.full((n_pad, bt.shape[1]), -1, np.int32)
+        pad[:, 0] = scratch_pages[g]
+        tables.append(np.concatenate([bt, pad]))
+        slots.append(np.concatenate([arrays["write_slots"][g], i32(scratch_pages[g] * page_size + np.arange(n_pad) % page_size)]))
+    out["block_tables"], out["write_slots"] = tables, slots
+    return out
+
+
 class StepContext:
     """``width_multiple`` rounds the block tables' width up (a replayed graph needs the same layout
     for many steps).  ``slab`` is a device buffer to fill instead of a new one, ``pinned`` the host
-    buffer the copy goes through; ``layout_key`` tells whether two steps have the same layout."""
+    buffer the copy goes through; ``layout_key`` tells whether two steps have the same layout.
+    ``pad_requests`` appends that many rows that stand for nobody (see ``_pad_arrays``; ``scratch_pages``: per
+    cache group the page they write to); their logits come last and are the caller's to drop.  ``n_requests``
+    and ``n_tokens`` count them, ``n_real_requests`` and ``n_real_tokens`` do not."""
 
     def __init__(self, entries: Sequence[StepEntry], manager, act_dtype: torch.dtype, device,
-                 width_multiple: int = 8, slab: torch.Tensor = None, pinned: torch.Tensor = None, upload: bool = True):
+                 width_multiple: int = 8, slab: torch.Tensor = None, pinned: torch.Tensor = None, upload: bool = True,
+                 pad_requests: int = 0, scratch_pages: Sequence[int] = ()):
         self.act_dtype, self.device = act_dtype, device
         self.timer = None              # a tracing.PhaseTimer while per-phase timing is on
         self.entries = list(entries)
-        R = self.n_requests = len(self.entries)
+        self.n_real_requests = len(self.entries)
         # lengths, positions, block tables and write slots come from the cache manager's native side in one call
         arrays = manager.step_arrays([e.rid for e in self.entries], [len(e.tokens) for e in self.entries], width_multiple)
+        self.n_real_tokens = int(arrays["positions"].shape[0])
+        if pad_requests > 0:
+            if len(scratch_pages) != len(manager.groups):
+                raise ValueError("padding rows need a scratch page for every cache group")
+            arrays = _pad_arrays(arrays, pad_requests, scratch_pages, manager.page_size)
+        R = self.n_requests = self.n_real_requests + max(pad_requests, 0)
         q_len, q_start, start = arrays["q_len"], arrays["q_start"], arrays["start"]
         T = self.n_tokens = int(arrays["positions"].shape[0])
         self.h_q_len, self.h_q_start, self.h_start_pos = q_len, q_start, start
         self.h_kv_len = arrays["kv_len"]
-        self.h_token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in self.entries]) if R else np.zeros(0, np.int32)
+        self.h_token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in self.entries]
+                                          + [np.zeros(max(pad_requests, 0), np.int32)]) if R else np.zeros(0, np.int32)
         self.h_row_req, self.h_positions = arrays["row_req"], arrays["positions"]
         rows: List[int] = []
         for i, e in enumerate(self.entries):
             rows.extend(int(q_start[i]) + int(w) for w in e.want)
+        self.n_real_logit_rows = len(rows)
+        rows.extend(range(self.n_real_tokens, T))            # rows that stand for nobody: last, dropped by the caller
         self.h_logit_rows = np.asarray(rows, dtype=np.int32)
         self.n_logit_rows = len(rows)
         self.h_state_slots = arrays["state_slots"]
@@ -86,10 +124,10 @@ class StepContext:
     def set_tokens(self, entries: Sequence[StepEntry], tokens: Sequence[int]) -> None:
         """For a context built ahead of its tokens (one placeholder token per request): the step's entries and
         their tokens, before ``bind``."""
-        if len(tokens) != self.n_tokens or len(entries) != self.n_requests:
+        if len(tokens) != self.n_real_tokens or len(entries) != self.n_real_requests:
             raise ValueError("set_tokens: not the step this context was built for")
         self.entries = list(entries)
-        self.h_token_ids[:] = tokens
+        self.h_token_ids[:self.n_real_tokens] = tokens
 
     def bind(self, slab: torch.Tensor = None, pinned: torch.Tensor = None) -> None:
         """Put the step's arrays on the device: into ``slab`` through ``pinned`` when given (an

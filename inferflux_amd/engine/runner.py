@@ -41,7 +41,13 @@ class _DecodeGraph:
 
 class ModelRunner:
     GRAPH_WIDTH_MULTIPLE = 64     # block-table width (pages) a captured step is valid for, in steps of this
-    MAX_GRAPHS = 12
+    MAX_GRAPHS = 24               # captured layouts kept; the one unused longest goes first
+    # A captured step is valid for one number of rows.  A batch that shrinks a request at a time would need a capture
+    # (a wait for the GPU, an eager step, the capture: tens of milliseconds) for every size it passes through, so the
+    # batch of a captured step is filled up to the next of these sizes with rows that stand for nobody (they write
+    # to a scratch page and their logits are dropped).  The sizes follow the products' kernels (up to 16 rows one
+    # kernel, 17-64 another) and cost nothing there: a weight-streaming product reads the same bytes for 5 rows and 8.
+    GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64)
 
     def __init__(self, model: Model, num_pages: int, page_size: int = 16, max_requests: int = 64,
                  decode_graphs: bool = True, phase_timing: bool = False):
@@ -67,6 +73,8 @@ class ModelRunner:
             self.timer = PhaseTimer()
         self.decode_graphs = decode_graphs and model.graph_safe and self.timer is None
         self._graphs = {}
+        self.graph_captures = 0    # decode-step layouts captured so far (each costs an eager step, a wait for the GPU and a capture)
+        self.graph_replays = 0
         self._prepared = None      # (the manager's snapshot of the requests, the context) of a step got ready ahead of its tokens
         self._launched = None      # (that snapshot, the graph) of a step already started with tokens the host has not seen
 
@@ -121,10 +129,19 @@ class ModelRunner:
             return False
         for r in rids:
             self.manager.reserve(r, 1)
-        ctx = StepContext([StepEntry(r, [0], [0]) for r in rids], self.manager, self.dtype, self.device,
-                          width_multiple=self.GRAPH_WIDTH_MULTIPLE, upload=False)
+        ctx = self._decode_context([StepEntry(r, [0], [0]) for r in rids])
         self._prepared = (self.manager.snapshot(rids), ctx)
         return True
+
+    def _decode_context(self, entries) -> StepContext:
+        """The context of a step of single tokens in the layout its captured graph has: block tables as wide as the
+        next multiple of GRAPH_WIDTH_MULTIPLE pages, the batch filled up to the next of GRAPH_BATCH_SIZES."""
+        n, pad = len(entries), 0
+        if not self.storage.has_state:          # (a row that stands for nobody would still need a state slot to scribble on)
+            size = next((b for b in self.GRAPH_BATCH_SIZES if b >= n), -(-n // 16) * 16)
+            pad = size - n
+        return StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
+                           upload=False, pad_requests=pad, scratch_pages=self.storage.scratch_pages)
 
     @property
     def starts_steps_early(self) -> bool:
@@ -146,12 +163,13 @@ class ModelRunner:
             return False
         snapshot, ctx = prep
         g = self._graphs.get(ctx.layout_key)
-        if g is None or tokens.dtype != torch.int32 or tuple(tokens.shape) != (ctx.n_tokens,) or tokens.device != self.device:
+        if g is None or tokens.dtype != torch.int32 or tuple(tokens.shape) != (ctx.n_real_tokens,) or tokens.device != self.device:
             return False
         self._prepared = None
         self._replay_inputs(g, ctx)
-        g.ctx.token_ids.copy_(tokens)          # (the copy above brought placeholder tokens; both precede the graph on the stream)
+        g.ctx.token_ids[:ctx.n_real_tokens].copy_(tokens)   # (the copy above brought placeholder tokens; both precede the graph on the stream)
         g.graph.replay()
+        self.graph_replays += 1
         copied = None
         if host_tokens is None:
             host_tokens = torch.empty(tokens.shape, dtype=torch.int32, pin_memory=True).copy_(tokens, non_blocking=True)
@@ -173,7 +191,7 @@ class ModelRunner:
             if [int(e.tokens[0]) for e in entries] != started_with or not self.manager.unchanged(snapshot, rids):
                 return None
             self.manager.commit_each(rids, 1)
-            return g.logits
+            return g.logits[:len(rids)]
         place = {r: i for i, r in enumerate(was)}
         rows = [place.get(r, -1) for r in rids]
         if min(rows) < 0 or any(a >= b for a, b in zip(rows, rows[1:])):
@@ -244,13 +262,15 @@ class ModelRunner:
         and is then captured; later steps copy their arrays into the graph's buffer and replay it.
         The logits returned by a replay live in the graph's memory: they are valid until the next step."""
         if ctx is None:
-            ctx = StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
-                              upload=False)
+            ctx = self._decode_context(entries)
+        n = ctx.n_real_logit_rows
         g = self._graphs.get(ctx.layout_key)
         if g is not None:
+            self._graphs[ctx.layout_key] = self._graphs.pop(ctx.layout_key)      # used last: evicted last
             self._replay_inputs(g, ctx)
             g.graph.replay()
-            return g.logits
+            self.graph_replays += 1
+            return g.logits[:n]
         slab = torch.empty(ctx.slab_size, dtype=torch.int32, device=self.device)
         pinned = torch.empty(ctx.slab_size, dtype=torch.int32, pin_memory=True)
         ctx.bind(slab, pinned)
@@ -258,11 +278,11 @@ class ModelRunner:
         if len(self._graphs) >= self.MAX_GRAPHS:
             self._graphs.pop(next(iter(self._graphs)))
         torch.cuda.synchronize()
-        cap_ctx = StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
-                              upload=False)
+        cap_ctx = self._decode_context(entries)
         cap_ctx.use_slab(slab)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             cap_logits = self.model.forward(cap_ctx, self.storage)
         self._graphs[ctx.layout_key] = _DecodeGraph(slab, pinned, graph, cap_ctx, cap_logits)
-        return logits
+        self.graph_captures += 1
+        return logits[:n]

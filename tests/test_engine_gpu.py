@@ -704,7 +704,7 @@ def test_a_toy_embedding_that_reads_positions_and_a_toy_mixer_with_narrow_values
     model = Model(plan=plan).init_random(9, torch.float32, "cuda")
     runner = ModelRunner(model, num_pages=8, max_requests=2)
     cache = runner.storage.binding(0).cache
-    assert tuple(cache.k.shape) == (8, 1, 16, d) and tuple(cache.v.shape) == (8, 1, dv, 16)
+    assert tuple(cache.k.shape) == (8 + 1, 1, 16, d) and tuple(cache.v.shape) == (8 + 1, 1, dv, 16)     # (one scratch page beyond the pool)
     assert runner.storage.bytes_per_token() == (d + dv) * 4
     assert plan_kv_pages(model, 16, 16 * 5) == 5                        # (sized by tokens; the bytes only cap it)
     ids = seeded_ids(31, 60, V)
@@ -813,3 +813,39 @@ def test_a_toy_block_with_four_norms_and_no_feed_forward():
     # the built-in arrangement refuses a layer it cannot be
     with pytest.raises(ValueError, match="no more and no less"):
         build_part("block", PartSpec("prenorm"), layer=plan.layers[0], hidden_size=H)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_shrinking_batch_replays_few_layouts(dtype, sharp_folders):
+    """Seven requests decode and leave one by one.  A captured decode step is filled up to the next of a few batch
+    sizes with rows that stand for nobody (they write to a scratch page outside the pool), so the batch passes
+    through sizes 7..1 on three captured layouts (8, 4, 2; 1 alone makes a fourth) instead of seven; every step's
+    logits are those of the same steps run eagerly without any such rows, bit for bit."""
+    folder, V = sharp_folders["C", dtype], TINY["C"]["vocab_size"]
+    eager = load_runner(folder, DT[dtype], num_pages=40, max_requests=8)
+    eager.decode_graphs = False
+    graphed = load_runner(folder, DT[dtype], num_pages=40, max_requests=8)
+    seqs = {r: seeded_ids(700 + i, 30 + 5 * i, V) for i, r in enumerate("abcdefg")}
+    at = {}
+    for rid, ids in seqs.items():
+        for r in (eager, graphed):
+            r.add_request(rid)
+            r.step([StepEntry(rid, ids[:20], [])])
+        at[rid] = 20
+    live = list(seqs)
+    while live:
+        for _ in range(3):
+            entries = [StepEntry(r, [seqs[r][at[r]]], [0]) for r in live]
+            want, got = eager.step(entries).cpu(), graphed.step(entries).cpu()
+            assert got.shape == (len(live), V) and torch.equal(got, want), (len(live), at)
+            for r in live:
+                at[r] += 1
+        gone = live.pop(0)
+        for r in (eager, graphed):
+            r.free_request(gone)
+            r.manager.check()
+    assert graphed.graph_captures == 4 and graphed.graph_replays == 21 - 4
+    assert sorted(k[0] for k in graphed._graphs) == [1, 2, 4, 8]
+    assert graphed.manager.free_pages() == eager.manager.free_pages() == [40, 40]
+    # the scratch page lies beyond every pool: no block table ever names it
+    assert graphed.storage.scratch_pages == [40, 40] and graphed.storage.binding(0).cache.k.shape[0] == 41
