@@ -33,83 +33,13 @@ IFX_DEFINE_LAST_ERROR()
 #endif
 static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "HEAD_DIM must be a multiple of 16 in 16..256");
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-
-constexpr int D = HEAD_DIM;
-constexpr int KS = (D + 31) / 32;  // 32-wide steps of the QK product (the last one half empty when D % 32 == 16)
-constexpr int DT = D / 16;         // 16-wide tiles of the output's head dimension
+#include "attn_shared.h"
 
 extern "C" int ifx_attn_head_dim() { return D; }
-
-__device__ __forceinline__ bf16x8 zero8() {
-  bf16x8 z;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
-  return z;
-}
-
-__device__ __forceinline__ bf16x8 join4(bf16x4 a, bf16x4 b) {
-  bf16x8 r;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { r[i] = a[i]; r[i + 4] = b[i]; }
-  return r;
-}
-
-__device__ __forceinline__ bf16x4 zero4() {
-  bf16x4 z;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) z[i] = (__bf16)0.f;
-  return z;
-}
-
-// 2^x on the hardware's exponent unit.  Arguments are <= 0 here and results below the smallest
-// normal float may flush to zero, which a softmax weight of that size may.
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// The four lanes that hold the same query column are lane, lane^16, lane^32, lane^48: one lane of each
-// row of 16.  gfx950 exchanges rows between two registers in one VALU instruction (permlane16_swap: odd
-// rows of the first with even rows of the second; permlane32_swap: rows 2, 3 of the first with rows 0, 1
-// of the second); given the same value twice, the two results hold v and v from the partner lane.
-__device__ __forceinline__ void swap16(float v, float& a, float& b) {
-  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
-}
-__device__ __forceinline__ void swap32(float v, float& a, float& b) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
-}
-__device__ __forceinline__ float col_max(float v) {
-  float a, b;
-  swap16(v, a, b); v = fmaxf(a, b);
-  swap32(v, a, b); return fmaxf(a, b);
-}
-__device__ __forceinline__ float col_sum(float v) {
-  float a, b;
-  swap16(v, a, b); v = a + b;
-  swap32(v, a, b); return a + b;
-}
 
 // =======================================================================================
 // rows
 // =======================================================================================
-struct RowArgs {
-  const bf16_t* q;        // [T, nH, D]
-  const bf16_t* k_cache;  // [pages, nKV, P, D]
-  const bf16_t* v_cache;  // [pages, nKV, D, P]
-  const int* rows;        // [n_rows] rows of the batch this launch handles (nullptr: rows 0..n_rows-1)
-  const int* row_req;     // [T]
-  const int* positions;   // [T]
-  const int* block_table; // [R, max_blocks], -1 where no page
-  float* part_o;          // [n_rows, nH, max_splits, D]
-  float* part_ml;         // [n_rows, nH, max_splits, 2]
-  bf16_t* out;            // [T, nH * D]
-  int max_blocks, n_rows, nH, nKV, P, window, chunk, max_splits;
-  float scale_log2e;
-  int part_by_row;        // partial results lie at the batch row's number (the tile kernel's), not at its place in ``rows``
-};
-
 // The operands of one block of 32 keys (two pages' worth of 16): loaded together, K and V at once,
 // so that a block costs one trip to memory, and one block ahead of the arithmetic.  The page numbers come
 // from a register: lane i of ``pages`` holds entry ``page_base + i`` of the request's block table, read once
@@ -247,75 +177,6 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = o[dt];
     }
-  }
-}
-
-// out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s.
-// One wave per (row, head): lane s first weighs split s, then every lane sums its elements over
-// the splits in ascending order.
-__global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
-  __shared__ float w_s[WAVE];
-  const int ri = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int row = a.rows ? a.rows[ri] : ri;
-  const int pos = a.positions[row];
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int s0 = lo / a.chunk, s1 = pos / a.chunk;  // first and last split that hold a visible key
-  const size_t pi = a.part_by_row ? row : ri;
-  const float* po = a.part_o + (pi * a.nH + head) * a.max_splits * D;
-  const float* pml = a.part_ml + (pi * a.nH + head) * a.max_splits * 2;
-  float acc[(D + WAVE - 1) / WAVE];
-#pragma unroll
-  for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = 0.f;
-  float L = 0.f;
-  // Lane s of a round holds split sb + s; rows with more than 64 splits take further rounds.  The first
-  // round's maxima and sums are kept from the pass that finds the maximum (the usual case is one round).
-  float M = -INFINITY, m_first = -INFINITY, l_first = 0.f;
-  for (int sb = s0; sb <= s1; sb += WAVE) {
-    const int s = sb + lane;
-    const float2 ml = s <= s1 ? *(const float2*)(pml + 2 * s) : float2{-INFINITY, 0.f};
-    if (sb == s0) { m_first = ml.x; l_first = ml.y; }
-    M = fmaxf(M, ml.x);
-  }
-  M = wave_max(M);
-  for (int sb = s0; sb <= s1; sb += WAVE) {
-    const int s = sb + lane;
-    float ms = m_first, ls = l_first;
-    if (sb != s0) {
-      const float2 ml = s <= s1 ? *(const float2*)(pml + 2 * s) : float2{-INFINITY, 0.f};
-      ms = ml.x; ls = ml.y;
-    }
-    const float w = ms == -INFINITY ? 0.f : exp2f(ms - M);
-    L += w * ls;
-    __syncthreads();
-    w_s[lane] = w;
-    __syncthreads();
-    const int n = min(WAVE, s1 - sb + 1);
-    // sixteen splits at a time, so that their loads are in flight together (a step of a loop that waits
-    // for its own loads costs a trip to the L2 each); an empty split (weight 0) is never read, its
-    // scratch may hold anything
-    for (int i = 0; i < n; i += 16) {
-      float wi[16], val[16][(D + WAVE - 1) / WAVE];
-#pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        wi[u] = i + u < n ? w_s[i + u] : 0.f;
-#pragma unroll
-        for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
-          const int e = lane + c * WAVE;
-          val[u][c] = (wi[u] != 0.f && e < D) ? po[(size_t)(sb + i + u) * D + e] : 0.f;
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 16; ++u)
-#pragma unroll
-        for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = fmaf(wi[u], val[u][c], acc[c]);
-    }
-  }
-  L = wave_sum(L);
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-#pragma unroll
-  for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
-    const int e = lane + c * WAVE;
-    if (e < D) a.out[((size_t)row * a.nH + head) * D + e] = (bf16_t)(acc[c] * inv);
   }
 }
 

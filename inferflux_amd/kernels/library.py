@@ -71,12 +71,25 @@ def _cxx() -> str:
     return _hipcc()          # hipcc compiles plain C++ too
 
 
+def _sources(name: str) -> Tuple[str, ...]:
+    """The files a module is built from: its source, the header of the same name (its public entry points) where it
+    has one, and every header of this folder that the source includes."""
+    import re
+    if _is_host_module(name):
+        return (f"{name}.cpp",)
+    files = [f"{name}.hip"]
+    with open(os.path.join(CSRC, files[0])) as f:
+        included = re.findall(r'^\s*#\s*include\s+"([^"]+)"', f.read(), flags=re.M)
+    for fn in ["common.h", f"{name}.h", *included]:
+        if fn not in files and os.path.isfile(os.path.join(CSRC, fn)):
+            files.append(fn)
+    return tuple(files)
+
+
 def _digest(name: str, variant: Variant) -> str:
     h = hashlib.sha256()
     host = _is_host_module(name)
-    for fn in ((f"{name}.cpp",) if host else (f"{name}.hip", "common.h", f"{name}.h")):
-        if fn == f"{name}.h" and not os.path.isfile(os.path.join(CSRC, fn)):
-            continue                    # a module's own header (its public entry points), where it has one
+    for fn in _sources(name):
         with open(os.path.join(CSRC, fn), "rb") as f:
             h.update(f.read())
     h.update(" ".join(HOST_FLAGS if host else FLAGS).encode())

@@ -46,13 +46,14 @@ def attention_tiles(args) -> None:
     vc = torch.randn(nb, nKV, d, P, device=dev, dtype=torch.bfloat16)
     table = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
-    for qt in ([args.query_tiles] if args.query_tiles else list(ops.TILE_QTS)):
-        tiles = list(range(0, T, ops.attention_tile_rows(d, qt)))
+    kernels = [("tiles", ops.attention_tiles, ops.attention_tile_rows(d, qt), qt) for qt in ([args.query_tiles] if args.query_tiles else list(ops.TILE_QTS))]
+    for name, fn, tile_rows, qt in kernels:
+        tiles = list(range(0, T, tile_rows))
         out = torch.empty(T, nH * d, device=dev, dtype=torch.bfloat16)
         call = (q, kc, vc, out, i32([0] * len(tiles)), i32(tiles), i32([0]), i32([T]), i32([T]), table, None, 1 / math.sqrt(d), qt)
-        t = _time_us(lambda i: ops.attention_tiles(*call), args.iters)
+        t = _time_us(lambda i: fn(*call), args.iters)
         flops = 4.0 * nH * d * T * (T + 1) / 2
-        print(f"attention-tiles rows={T} query_tiles={qt}: {t:9.1f} us  {flops / t / 1e6:7.1f} TFLOP/s (causal half only)", flush=True)
+        print(f"attention-tiles rows={T} {name}, query_tiles={qt}: {t:9.1f} us  {flops / t / 1e6:7.1f} TFLOP/s (causal half only)", flush=True)
 
 
 def attention_rows(args) -> None:
