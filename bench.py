@@ -62,6 +62,9 @@ def main() -> int:
                     help="measure what the card gives (a 2 GB streaming read, an 8192^3 bf16 library product) once and "
                          "report every share against it beside the data sheet's peak")
     ap.add_argument("--context", type=int, default=DECODE_KV_START, help="tokens each request holds when the timed decode steps start")
+    ap.add_argument("--shape", choices=["7b", "3b", "14b"], default="7b", help="layer sizes of the decode / prefill measurement (the headline is 7b)")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT, help="--workload prefill: tokens of the prompt")
+    ap.add_argument("--prefill-chunk", type=int, default=0, help="--workload prefill: the prompt in portions of this many tokens, one step each (0: whole)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -89,7 +92,8 @@ def main() -> int:
     ops.decode_weight_copy = not args.no_decode_weight_copy
     if args.workload in WORKLOADS:
         return run_workload(args, WORKLOADS[args.workload])
-    shape = dict(SHAPE_7B)
+    shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B}[args.shape])
+    shape_name = f"Qwen2.5-{args.shape.upper()} shape"
     layers_full = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
@@ -105,7 +109,7 @@ def main() -> int:
     L, H, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     nH, nKV, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     layer_params = (nH + 2 * nKV) * d * H + (nH + 2 * nKV) * d + nH * d * H + 3 * I * H + 2 * H
-    weight_bytes = (L * layer_params + H + V * H) * esz          # every weight a decode step uses, once
+    weight_bytes = (L * layer_params + H + V * H) * esz          # every weight a decode step uses, once (a tied head reads the table)
     kv_bytes_per_token = 2 * L * nKV * d * esz
     gen = torch.Generator().manual_seed(1)
 
@@ -142,23 +146,27 @@ def main() -> int:
         torch.cuda.empty_cache()
         return batch * steps / dt, dt / steps * 1e3, kv_mean
 
-    def prefill_rate(tokens, reps=3):
-        """(tokens/s, ms, share of the matrix peak, mean ms) of a prompt of ``tokens`` in one step: the best of ``reps``
-        runs after one that warms up (and, with tuning on, lets the library time its kernels for these shapes)."""
+    def prefill_rate(tokens, reps=3, chunk=0):
+        """(tokens/s, ms, share of the matrix peak, mean ms) of a prompt of ``tokens`` in one step (or in portions of
+        ``chunk`` tokens, one step each): the best of ``reps`` runs after one that warms up (and, with tuning on, lets
+        the library time its kernels for these shapes)."""
         runner = ModelRunner(model, num_pages=-(-tokens // PAGE) + 1, page_size=PAGE, max_requests=2)
         ids = torch.randint(0, V, (tokens,), generator=gen).tolist()
+        cuts = list(range(0, tokens, chunk or tokens))
         times = []
         ops.pause_library_gemm_tuning(False)
         for i in range(reps + 1):
             runner.add_request(i)
             torch.cuda.synchronize()
             t = time.perf_counter()
-            runner.step([StepEntry(i, ids, [tokens - 1])])
+            for a0 in cuts:
+                part = ids[a0:a0 + (chunk or tokens)]
+                runner.step([StepEntry(i, part, [len(part) - 1] if a0 == cuts[-1] else [])])
             torch.cuda.synchronize()
             dt = time.perf_counter() - t
             runner.free_request(i)
             ops.pause_library_gemm_tuning(True)
-            note(f"prefill of {tokens} tokens: {dt * 1e3:.1f} ms")
+            note(f"prefill of {tokens} tokens{f' in portions of {chunk}' if chunk else ''}: {dt * 1e3:.1f} ms")
             if i > 0:
                 times.append(dt)
         best = min(times)
@@ -191,12 +199,13 @@ def main() -> int:
         return r
 
     if args.workload == "prefill":
-        ptps, pms, pfrac, _ = prefill_rate(PROMPT, reps=args.steps)
-        print(json.dumps({"metric": f"prefill tok/s, {PROMPT} tokens (Qwen2.5-7B shape, {args.dtype}, random weights)",
+        ptps, pms, pfrac, _ = prefill_rate(args.prompt_len, reps=args.steps, chunk=args.prefill_chunk)
+        print(json.dumps({"metric": f"prefill tok/s, {args.prompt_len} tokens (" + shape_name + f", {args.dtype}, random weights)",
                           "value": round(ptps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": 1,
                           "ms_per_step": round(pms, 3), "higher_is_better": True, "dtype": args.dtype,
-                          "config": {"model": "Qwen2.5-7B shape", "num_hidden_layers": layers_full, "layers_run": L,
-                                     "prompt_len": PROMPT, "library_gemm_tuning": not args.no_gemm_tuning},
+                          "config": {"model": shape_name, "num_hidden_layers": layers_full, "layers_run": L,
+                                     "prompt_len": args.prompt_len, "prefill_chunk": args.prefill_chunk or args.prompt_len,
+                                     "library_gemm_tuning": not args.no_gemm_tuning},
                           "frac_of_peak": round(pfrac, 4)}), flush=True)
         return 0
     ceil = measured_ceilings() if (args.ceilings and args.dtype == "bf16") else None
@@ -205,15 +214,15 @@ def main() -> int:
     tps, ms, kv_mean = decode_rate(args.batch, args.steps, max(args.warmup, 1))
     note(f"batch {args.batch}: {tps:.0f} tokens/s")
     out = {
-        "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-7B shape, {args.dtype}, random weights)",
+        "metric": f"decode tok/s at batch {args.batch} (" + shape_name + f", {args.dtype}, random weights)",
         "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (uniform random token ids, seeded N(0,0.02) weights)",
-        "config": {"model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "1 GPU",
+        "config": {"model": shape_name, "global_batch": args.batch, "seq_len": max(CONTEXT, kv_start + args.steps + args.warmup), "parallelism": "1 GPU",
                    "num_hidden_layers": layers_full, "layers_run": L, "hidden_size": H, "num_attention_heads": nH,
                    "num_key_value_heads": nKV, "head_dim": d, "intermediate_size": I, "vocab_size": V,
                    "prompt_len": PROMPT, "decode_kv_start": kv_start, "kv_page_size": PAGE,
-                   "tie_word_embeddings": False, "library_gemm_tuning": not args.no_gemm_tuning,
+                   "tie_word_embeddings": bool(shape["tie_word_embeddings"]), "library_gemm_tuning": not args.no_gemm_tuning,
                    "decode_weight_copy": not args.no_decode_weight_copy},
         "roofline": hbm_roofline(args.batch, ms, kv_mean, ceil),
     }

@@ -18,16 +18,53 @@ from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
 TILE_QT2_MIN_WORKGROUPS = 512   # two workgroups of the tile kernel for each of the 256 compute units
-TILE_SPLIT_BELOW = 256          # fewer workgroups than compute units: the tile kernel splits the keys
-TILE_SPLIT_TARGET = 512         # ... aiming at this many workgroups,
-TILE_SPLIT_MIN_KEYS = 256       # with at least this many keys to a split
+TILE_QT2_MIN_KEYS = 2048        # ... or keys enough that reading them from LDS half as often decides (see choose_tiling)
+TILE_SPLIT_BELOW = 384          # fewer workgroups than this: the tile kernel splits the keys
+TILE_SPLIT_TARGET = 448         # ... aiming at this many workgroups,
+TILE_SPLIT_MIN_KEYS = 512       # with at least this many keys to a split
+TILE_SPLIT_MIN_LONGEST = 1536   # and only when the longest request has this many keys: writing and merging partial
+                                # results costs about 20 us
+TILE_SPLIT_FEW = 128            # at most this many workgroups: splits pay from
+TILE_SPLIT_FEW_MIN_LONGEST = 1024   # this many keys on, and may be as short as
+TILE_SPLIT_FEW_MIN_KEYS = 256       # this while the walk is short
 TILE_MAX_SPLITS = 16
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 128  # and until a row has at most this many splits (one row over 131,072 keys: 91 us against 133 at 64)
 
 
-def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads):
+def choose_tiling(tiled_rows, longest: int, n_heads: int, rows_of):
+    """(query tiles per wave, key splits, keys per split) for a launch of the tile kernel: ``tiled_rows`` the row
+    counts of the requests it covers, ``longest`` the most keys any of them sees, ``rows_of(qt)`` a tile's rows.
+
+    Measured at head size 128 (28, 16 and 40 query heads; portions of 256-2,048 rows after pasts of 0-7,680 keys):
+    two query tiles per wave are level with one at 2,048 rows without a past and 20-30 % faster behind a past
+    (2,048 rows after 2,048 / 4,096 / 6,144 keys: 185 / 271 / 354 us against 236 / 379 / 494), as long as the rows
+    fill the taller tiles; about 448 workgroups are the best number to cut the keys for (1,024 rows after 7,168
+    keys: 292 us whole, 199 in two splits, 208 in four), and a cut pays only when the walk it shortens is long
+    (512 rows after 512 keys: 34 us whole, 40 in two splits)."""
+    total = int(sum(tiled_rows))
+    n_big = sum(-(-int(n) // rows_of(2)) for n in tiled_rows)
+    qt = 1
+    if n_big * n_heads >= TILE_QT2_MIN_WORKGROUPS:
+        qt = 2
+    elif longest >= TILE_QT2_MIN_KEYS and n_big * rows_of(2) * 2 <= total * 3:
+        qt = 2
+    groups = sum(-(-int(n) // rows_of(qt)) for n in tiled_rows) * n_heads
+    splits, chunk = 1, 0
+    if groups < TILE_SPLIT_BELOW and longest >= (TILE_SPLIT_FEW_MIN_LONGEST if groups <= TILE_SPLIT_FEW else TILE_SPLIT_MIN_LONGEST):
+        want = min(max(1, (2 * TILE_SPLIT_TARGET + groups) // (2 * groups)), longest // TILE_SPLIT_MIN_KEYS, TILE_MAX_SPLITS)
+        if groups <= TILE_SPLIT_FEW and longest < 2 * TILE_SPLIT_MIN_LONGEST:
+            want = max(want, min(4, longest // TILE_SPLIT_FEW_MIN_KEYS))
+        if want > 1:
+            chunk = (-(-longest // want) + 63) // 64 * 64
+            splits = -(-longest // chunk)
+            if splits <= 1:
+                splits, chunk = 1, 0
+    return qt, splits, chunk
+
+
+def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk=0):
     """What the kernels need beyond the step's own arrays, computed once per step (and per number of
     kv heads, which decides how many waves a launch has)."""
     q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
@@ -44,15 +81,10 @@ def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads):
         out["tile_req"] = ctx.upload(np.asarray(tile_req, np.int32))
         out["tile_q0"] = ctx.upload(np.asarray(tile_q0, np.int32))
         # Few tiles with many keys each (portions of prompts with a long past) leave most of the chip idle
-        # and each workgroup walking its keys alone: cut the keys into splits that run side by side.
-        groups = len(tile_req) * n_heads
-        longest = int(kv_len[tiled].max())
-        if groups < TILE_SPLIT_BELOW and longest >= 2 * TILE_SPLIT_MIN_KEYS:
-            want = min(-(-TILE_SPLIT_TARGET // groups), longest // TILE_SPLIT_MIN_KEYS, TILE_MAX_SPLITS)
-            chunk = (-(-longest // want) + 63) // 64 * 64
-            out["tile_splits"], out["tile_chunk"] = -(-longest // chunk), chunk
-            if out["tile_splits"] > 1:
-                out["tile_row_list"] = ctx.upload(np.nonzero(~row_mask)[0].astype(np.int32))
+        # and each workgroup walking its keys alone: the keys are cut into splits that run side by side.
+        if tile_splits > 1:
+            out["tile_splits"], out["tile_chunk"] = tile_splits, tile_chunk
+            out["tile_row_list"] = ctx.upload(np.nonzero(~row_mask)[0].astype(np.int32))
     if rows.size:
         if rows.size != ctx.n_tokens:
             out["rows"] = ctx.upload(rows)
@@ -73,14 +105,15 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
     n_kv = cache.k.shape[1]
-    # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often;
-    # they win once they still give two workgroups for each compute unit (measured with 28 heads: equal
-    # at 2,048 rows, 5 % faster at 4,096, 30 % at 8,192; one tile per wave is ahead below).
-    big = ops.attention_tile_rows(d, 2)
-    n_big = sum(-(-int(n) // big) for n in ctx.h_q_len if n >= TILE_MIN)
-    qt = 2 if n_big * nH >= TILE_QT2_MIN_WORKGROUPS else 1
+    # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often.
+    tiled = ctx.h_q_len >= TILE_MIN
+    qt, splits, chunk = 1, 1, 0
+    if tiled.any():
+        qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], int(ctx.h_kv_len[tiled].max()), nH,
+                                          lambda t: ops.attention_tile_rows(d, t))
     tile_rows = ops.attention_tile_rows(d, qt)
-    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH), lambda: _work_lists(ctx, n_kv, tile_rows, nH))
+    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk),
+                    lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,

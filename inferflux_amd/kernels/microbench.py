@@ -40,20 +40,27 @@ def _time_us(fn, iters: int) -> float:
 
 def attention_tiles(args) -> None:
     dev, T, nH, nKV, d, P = "cuda", args.rows, args.heads, args.kv_heads, args.head_dim, args.page_size
+    past = args.past
+    L = past + T
     q = torch.randn(T, nH, d, device=dev, dtype=torch.bfloat16)
-    nb = -(-T // P)
+    nb = -(-L // P)
     kc = torch.randn(nb, nKV, P, d, device=dev, dtype=torch.bfloat16)
     vc = torch.randn(nb, nKV, d, P, device=dev, dtype=torch.bfloat16)
     table = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
-    kernels = [("tiles", ops.attention_tiles, ops.attention_tile_rows(d, qt), qt) for qt in ([args.query_tiles] if args.query_tiles else list(ops.TILE_QTS))]
-    for name, fn, tile_rows, qt in kernels:
-        tiles = list(range(0, T, tile_rows))
+    row_req, positions = i32([0] * T), torch.arange(past, L, dtype=torch.int32, device=dev)
+    row_list = torch.arange(T, dtype=torch.int32, device=dev)
+    flops = 4.0 * nH * d * (T * past + T * (T + 1) / 2)
+    for qt in ([args.query_tiles] if args.query_tiles else list(ops.TILE_QTS)):
+        tiles = list(range(0, T, ops.attention_tile_rows(d, qt)))
         out = torch.empty(T, nH * d, device=dev, dtype=torch.bfloat16)
-        call = (q, kc, vc, out, i32([0] * len(tiles)), i32(tiles), i32([0]), i32([T]), i32([T]), table, None, 1 / math.sqrt(d), qt)
-        t = _time_us(lambda i: fn(*call), args.iters)
-        flops = 4.0 * nH * d * T * (T + 1) / 2
-        print(f"attention-tiles rows={T} {name}, query_tiles={qt}: {t:9.1f} us  {flops / t / 1e6:7.1f} TFLOP/s (causal half only)", flush=True)
+        for chunk in ([int(c) for c in args.tile_chunk.split(",")] if args.tile_chunk else [0]):
+            splits = -(-L // chunk) if chunk else 1
+            call = (q, kc, vc, out, i32([0] * len(tiles)), i32(tiles), i32([0]), i32([T]), i32([L]), table, None, 1 / math.sqrt(d), qt,
+                    chunk, splits, row_list if splits > 1 else None, row_req, positions)
+            t = _time_us(lambda i: ops.attention_tiles(*call), args.iters)
+            print(f"attention-tiles rows={T} past={past} query_tiles={qt} key splits={splits}: {t:9.1f} us  {flops / t / 1e6:7.1f} TFLOP/s "
+                  f"(visible keys only)", flush=True)
 
 
 def attention_rows(args) -> None:
@@ -149,6 +156,8 @@ def main(argv=None) -> int:
         if name == "attention-tiles":
             p.add_argument("--rows", type=int, default=2048, help="rows of one request in one step, no past")
             p.add_argument("--query-tiles", type=int, default=0, help="1 or 2 query tiles per wave (0: both)")
+            p.add_argument("--past", type=int, default=0, help="keys the request already holds (a later portion of a prompt)")
+            p.add_argument("--tile-chunk", default="", help="keys per split, comma separated (multiples of 64; empty or 0: no splits)")
         if name == "attention-rows":
             p.add_argument("--batch", type=int, default=8)
             p.add_argument("--context", type=int, default=3072)

@@ -586,7 +586,9 @@ def test_prompt_portions_with_a_long_past_split_their_keys(sharp_folders, monkey
     """Portions of a prompt late in a long context: few tiles, many keys, which the tile kernel cuts into splits.
     The thresholds are lowered so that the tiny models' 250 and 380 tokens qualify."""
     from inferflux_amd.kernels import attention
-    monkeypatch.setattr(attention, "TILE_SPLIT_MIN_KEYS", 64)
+    for name, value in (("TILE_SPLIT_MIN_KEYS", 64), ("TILE_SPLIT_MIN_LONGEST", 128), ("TILE_SPLIT_FEW_MIN_LONGEST", 128),
+                        ("TILE_SPLIT_FEW_MIN_KEYS", 64), ("TILE_QT2_MIN_KEYS", 300)):
+        monkeypatch.setattr(attention, name, value)
     calls = []
     real = attention.ops.attention_tiles
     monkeypatch.setattr(attention.ops, "attention_tiles", lambda *a, **k: (calls.append(a[14] if len(a) > 14 else 1), real(*a, **k))[1])
