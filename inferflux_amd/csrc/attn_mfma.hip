@@ -236,6 +236,10 @@ struct TileArgs {
   int chunk, max_splits;
   float* part_o;          // [T, nH, max_splits, D]
   float* part_ml;         // [T, nH, max_splits, 2]
+  // [8 * per_xcd] or nullptr: the work item of each place in the launch (-1: none), place x * per_xcd + i being
+  // the i-th workgroup that XCD x is given.  The caller orders the items so that the workgroups that come to
+  // share a compute unit have about the same number of key tiles between them on every unit.
+  const int* order;
 };
 
 constexpr int N_PIECES = TK * (D / 8);                // 16-byte pieces of a K tile, and as many of a V^T tile
@@ -463,8 +467,10 @@ void attn_tiles_kernel(TileArgs a) {
   // workgroups that read one kv head's keys and values share an L2 instead of filling all eight with
   // everything; within a run the tiles with the most keys (the latest rows) come first.
   const int ratio = a.nH / a.nKV;
-  const int work = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
-  if (blockIdx.x / 8 >= a.per_xcd || work >= a.n_tiles * a.nH * a.max_splits) return;   // the whole workgroup leaves together
+  const int place = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
+  if (blockIdx.x / 8 >= a.per_xcd) return;                                              // the whole workgroup leaves together
+  const int work = a.order ? a.order[place] : place;
+  if (work < 0 || work >= a.n_tiles * a.nH * a.max_splits) return;
   const int item = work / a.max_splits, split = work % a.max_splits;
   const int per_kv = ratio * a.n_tiles;
   const int kvh = item / per_kv, rem = item % per_kv;
@@ -558,7 +564,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
                               const int* q_len, const int* kv_len, const int* block_table, int max_blocks,
                               int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
                               float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
-                              const int* positions, void* stream) {
+                              const int* positions, const int* order, int order_per_xcd, void* stream) {
   IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_tiles: page_size %d must be a multiple of 16", page_size);
@@ -573,10 +579,12 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   if (n_tiles == 0) return 0;
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
-             n_tiles, 0, chunk, max_splits, part_o, part_ml};
+             n_tiles, 0, chunk, max_splits, part_o, part_ml, order};
   const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
-  a.per_xcd = (int)((items + 7) / 8);
+  IFX_REQUIRE(!order || (order_per_xcd > 0 && 8LL * order_per_xcd >= items && order_per_xcd <= items),
+              "attn_tiles: an order of 8 x %d places cannot hold %lld work items", order_per_xcd, items);
+  a.per_xcd = order ? order_per_xcd : (int)((items + 7) / 8);
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(attn_tiles_kernel, dim3(8 * a.per_xcd), dim3(256), 0, s, a);
   if (max_splits > 1) {

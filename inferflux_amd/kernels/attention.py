@@ -18,7 +18,7 @@ from . import ops
 
 TILE_MIN = 16       # fewer rows than this are cheaper one by one
 TILE_QT2_MIN_WORKGROUPS = 512   # two workgroups of the tile kernel for each of the 256 compute units
-TILE_QT2_MIN_KEYS = 2048        # ... or keys enough that reading them from LDS half as often decides (see choose_tiling)
+TILE_QT2_MIN_KEYS = 1536        # ... or rows that see this many keys on average, so that reading them from LDS half as often decides
 TILE_SPLIT_BELOW = 384          # fewer workgroups than this: the tile kernel splits the keys
 TILE_SPLIT_TARGET = 448         # ... aiming at this many workgroups,
 TILE_SPLIT_MIN_KEYS = 512       # with at least this many keys to a split
@@ -28,27 +28,33 @@ TILE_SPLIT_FEW = 128            # at most this many workgroups: splits pay from
 TILE_SPLIT_FEW_MIN_LONGEST = 1024   # this many keys on, and may be as short as
 TILE_SPLIT_FEW_MIN_KEYS = 256       # this while the walk is short
 TILE_MAX_SPLITS = 16
+TILE_ORDER_MIN_ITEMS = 64       # launches of more workgroups than this get them in tile_order
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 128  # and until a row has at most this many splits (one row over 131,072 keys: 91 us against 133 at 64)
 
 
-def choose_tiling(tiled_rows, longest: int, n_heads: int, rows_of):
+def choose_tiling(tiled_rows, tiled_keys, n_heads: int, rows_of):
     """(query tiles per wave, key splits, keys per split) for a launch of the tile kernel: ``tiled_rows`` the row
-    counts of the requests it covers, ``longest`` the most keys any of them sees, ``rows_of(qt)`` a tile's rows.
+    counts of the requests it covers, ``tiled_keys`` how many keys each of them holds after the step,
+    ``rows_of(qt)`` a tile's rows.
 
-    Measured at head size 128 (28, 16 and 40 query heads; portions of 256-2,048 rows after pasts of 0-7,680 keys):
-    two query tiles per wave are level with one at 2,048 rows without a past and 20-30 % faster behind a past
-    (2,048 rows after 2,048 / 4,096 / 6,144 keys: 185 / 271 / 354 us against 236 / 379 / 494), as long as the rows
-    fill the taller tiles; about 448 workgroups are the best number to cut the keys for (1,024 rows after 7,168
-    keys: 292 us whole, 199 in two splits, 208 in four), and a cut pays only when the walk it shortens is long
-    (512 rows after 512 keys: 34 us whole, 40 in two splits)."""
+    Measured at head size 128 (28, 16 and 40 query heads; portions of 256-8,192 rows after pasts of 0-7,680 keys,
+    workgroups in ``tile_order``): two query tiles per wave win when they still give two workgroups to each compute
+    unit (4,096 rows: 178 us against 236) or when a tile walks many keys on average (2,048 rows after 2,048 keys:
+    158 us against 218; 1,024 after 1,024: 74 against 80), as long as the rows fill the taller tiles, and lose
+    on a short causal prompt (2,048 rows: 81 us against 75).  About 448 workgroups are the best number to cut the
+    keys for (1,024 rows after 7,168 keys: 292 us whole, 199 in two splits, 208 in four), and a cut pays only when
+    the walk it shortens is long (512 rows after 512 keys: 34 us whole, 40 in two splits)."""
     total = int(sum(tiled_rows))
+    longest = int(max(tiled_keys))
+    # keys a row sees, averaged over the launch's rows: a request's rows see from (keys - rows) to keys of them
+    seen = sum(int(n) * (int(k) - int(n) / 2.0) for n, k in zip(tiled_rows, tiled_keys)) / max(total, 1)
     n_big = sum(-(-int(n) // rows_of(2)) for n in tiled_rows)
     qt = 1
     if n_big * n_heads >= TILE_QT2_MIN_WORKGROUPS:
         qt = 2
-    elif longest >= TILE_QT2_MIN_KEYS and n_big * rows_of(2) * 2 <= total * 3:
+    elif seen >= TILE_QT2_MIN_KEYS and n_big * rows_of(2) * 2 <= total * 3:
         qt = 2
     groups = sum(-(-int(n) // rows_of(qt)) for n in tiled_rows) * n_heads
     splits, chunk = 1, 0
@@ -64,7 +70,56 @@ def choose_tiling(tiled_rows, longest: int, n_heads: int, rows_of):
     return qt, splits, chunk
 
 
-def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk=0):
+N_XCD, CUS_PER_XCD = 8, 32     # the launch deals workgroups to the XCDs in turn, and an XCD deals its share to its compute units in turn
+
+
+def tile_order(first_pos, last_pos, n_heads: int, window: Optional[int], splits: int, chunk: int, period: int = CUS_PER_XCD) -> np.ndarray:
+    """Which work item each workgroup of a tile launch takes: int32 [8 * n], place x * n + i being the i-th workgroup
+    of XCD x (-1: none).  ``first_pos`` / ``last_pos``: the positions of every tile's first and last row.
+
+    A work item is (head, tile, split), numbered head * tiles * splits + (tiles - 1 - tile) * splits + split, and
+    walks a number of 64-key tiles that is known here.  Workgroups on one compute unit share its time, so a unit
+    that is given three long walks finishes long after one with three short ones: a causal prompt of 2,048 rows
+    took 100 us in the order longest first, head by head, where the walks of the unit that came first summed to
+    96 key tiles and the average was 58.  Here the items stay in head order (an XCD's workgroups read few kv heads,
+    which its L2 then holds), are cut into eight runs of equal walks, not equal counts, and go to the workgroups
+    of a run in boustrophedon order of their length with a compute unit's turn as the period, so that the i-th,
+    (2 * period - 1 - i)-th, (2 * period + i)-th ... longest meet on one unit."""
+    first_pos, last_pos = np.asarray(first_pos, np.int64), np.asarray(last_pos, np.int64)
+    n_tiles = first_pos.shape[0]
+    lo = np.maximum(first_pos - window + 1, 0) if window else np.zeros(n_tiles, np.int64)
+    if splits > 1:
+        s = np.arange(splits, dtype=np.int64)[None, :]
+        lo_ts = np.maximum(lo[:, None], s * chunk)
+        hi_ts = np.minimum(last_pos[:, None], (s + 1) * chunk - 1)
+    else:
+        lo_ts, hi_ts = lo[:, None], last_pos[:, None]
+    walk = np.where(hi_ts >= lo_ts // 64 * 64, hi_ts // 64 - lo_ts // 64 + 1, 0)        # [tiles, splits] key tiles walked
+    cost = (walk[::-1] + 1).reshape(-1)                                                # + 1: a workgroup's start and end
+    cost = np.tile(cost, n_heads)                                                      # [items] in the kernel's numbering
+    n_items = cost.shape[0]
+    cum = np.cumsum(cost)
+    run = np.minimum((cum - cost) * N_XCD // cum[-1], N_XCD - 1)                       # the run an item's start falls into
+    counts = np.bincount(run, minlength=N_XCD)
+    per_xcd = int(counts.max())
+    order = np.full((N_XCD, per_xcd), -1, np.int32)
+    start = 0
+    for x in range(N_XCD):
+        n = int(counts[x])
+        if n == 0:
+            continue
+        items = np.arange(start, start + n)
+        by_len = items[np.argsort(-cost[start:start + n], kind="stable")]
+        rank = np.arange(n)
+        row, col = rank // period, rank % period
+        width = np.minimum(period, n - row * period)
+        place = row * period + np.where(row % 2 == 0, col, width - 1 - col)
+        order[x, place] = by_len
+        start += n
+    return order.reshape(-1)
+
+
+def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk=0, window=None):
     """What the kernels need beyond the step's own arrays, computed once per step (and per number of
     kv heads, which decides how many waves a launch has)."""
     q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
@@ -77,9 +132,15 @@ def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk
     rows = np.nonzero(row_mask)[0].astype(np.int32)
     out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1,
            "tile_splits": 1, "tile_chunk": 0, "tile_row_list": None}
+    out["tile_order"] = None
     if tile_req:
-        out["tile_req"] = ctx.upload(np.asarray(tile_req, np.int32))
-        out["tile_q0"] = ctx.upload(np.asarray(tile_q0, np.int32))
+        tile_req, tile_q0 = np.asarray(tile_req, np.int32), np.asarray(tile_q0, np.int32)
+        out["tile_req"] = ctx.upload(tile_req)
+        out["tile_q0"] = ctx.upload(tile_q0)
+        if len(tile_req) * n_heads * tile_splits > TILE_ORDER_MIN_ITEMS:
+            first = (kv_len[tile_req] - q_len[tile_req] + tile_q0).astype(np.int64)
+            last = np.minimum(first + tile_rows, kv_len[tile_req]) - 1
+            out["tile_order"] = ctx.upload(tile_order(first, last, n_heads, window, tile_splits, tile_chunk))
         # Few tiles with many keys each (portions of prompts with a long past) leave most of the chip idle
         # and each workgroup walking its keys alone: the keys are cut into splits that run side by side.
         if tile_splits > 1:
@@ -109,16 +170,15 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     tiled = ctx.h_q_len >= TILE_MIN
     qt, splits, chunk = 1, 1, 0
     if tiled.any():
-        qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], int(ctx.h_kv_len[tiled].max()), nH,
-                                          lambda t: ops.attention_tile_rows(d, t))
+        qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], ctx.h_kv_len[tiled], nH, lambda t: ops.attention_tile_rows(d, t))
     tile_rows = ops.attention_tile_rows(d, qt)
-    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk),
-                    lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk))
+    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk, window),
+                    lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk, window))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
                             table, window, scale, qt, w["tile_chunk"], w["tile_splits"], w["tile_row_list"], ctx.row_req,
-                            ctx.positions)
+                            ctx.positions, w["tile_order"])
     if w["n_rows"]:
         ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
                            window, scale, w["chunk"], w["max_splits"])

@@ -17,6 +17,7 @@ import argparse
 import math
 import sys
 
+import numpy as np
 import torch
 
 from . import ops
@@ -56,11 +57,18 @@ def attention_tiles(args) -> None:
         out = torch.empty(T, nH * d, device=dev, dtype=torch.bfloat16)
         for chunk in ([int(c) for c in args.tile_chunk.split(",")] if args.tile_chunk else [0]):
             splits = -(-L // chunk) if chunk else 1
-            call = (q, kc, vc, out, i32([0] * len(tiles)), i32(tiles), i32([0]), i32([T]), i32([L]), table, None, 1 / math.sqrt(d), qt,
-                    chunk, splits, row_list if splits > 1 else None, row_req, positions)
-            t = _time_us(lambda i: ops.attention_tiles(*call), args.iters)
-            print(f"attention-tiles rows={T} past={past} query_tiles={qt} key splits={splits}: {t:9.1f} us  {flops / t / 1e6:7.1f} TFLOP/s "
-                  f"(visible keys only)", flush=True)
+            for period in [int(c) for c in args.order_period.split(",")]:
+                order = None
+                if period:
+                    from .attention import tile_order
+                    first = past + np.asarray(tiles)
+                    order = torch.from_numpy(tile_order(first, np.minimum(first + ops.attention_tile_rows(d, qt), L) - 1, nH, None, splits,
+                                                        chunk, period)).to(dev)
+                call = (q, kc, vc, out, i32([0] * len(tiles)), i32(tiles), i32([0]), i32([T]), i32([L]), table, None, 1 / math.sqrt(d), qt,
+                        chunk, splits, row_list if splits > 1 else None, row_req, positions, order)
+                t = _time_us(lambda i: ops.attention_tiles(*call), args.iters)
+                print(f"attention-tiles rows={T} past={past} query_tiles={qt} key splits={splits} order period={period}: {t:9.1f} us  "
+                      f"{flops / t / 1e6:7.1f} TFLOP/s (visible keys only)", flush=True)
 
 
 def attention_rows(args) -> None:
@@ -157,6 +165,8 @@ def main(argv=None) -> int:
             p.add_argument("--rows", type=int, default=2048, help="rows of one request in one step, no past")
             p.add_argument("--query-tiles", type=int, default=0, help="1 or 2 query tiles per wave (0: both)")
             p.add_argument("--past", type=int, default=0, help="keys the request already holds (a later portion of a prompt)")
+            p.add_argument("--order-period", default="0,32", help="workgroups ordered by attention.tile_order with these periods, "
+                           "comma separated (0: in the order of the heads, longest first)")
             p.add_argument("--tile-chunk", default="", help="keys per split, comma separated (multiples of 64; empty or 0: no splits)")
         if name == "attention-rows":
             p.add_argument("--batch", type=int, default=8)

@@ -721,14 +721,18 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     tile_req: torch.Tensor, tile_q0: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                     kv_len: torch.Tensor, block_table: torch.Tensor, window: Optional[int], scale: float,
                     qt: int = 1, chunk: int = 0, max_splits: int = 1, rows: Optional[torch.Tensor] = None,
-                    row_req: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
+                    row_req: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+                    order: Optional[torch.Tensor] = None) -> None:
     """Attention of tiles of ``attention_tile_rows(d, qt)`` consecutive rows of one request each (tile t:
     request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d].
 
     With ``max_splits`` > 1 every tile's keys are cut into splits of ``chunk`` keys (a multiple of 64;
     ``max_splits`` * chunk must reach past the largest position) that run as workgroups of their own, and
     the rows named by ``rows`` (int32: every row of every tiled request) are merged at the end; this
-    needs the step's ``row_req`` and ``positions`` [T]."""
+    needs the step's ``row_req`` and ``positions`` [T].
+
+    ``order`` (int32 [8 * n], from ``attention.tile_order``) says which work item each workgroup of the launch
+    takes; every item must appear exactly once (-1: a workgroup without work).  The result does not depend on it."""
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt)
     if mod.fn("ifx_attn_tile_rows", ())() != attention_tile_rows(d, qt):
         raise KernelError("attention_tiles: the compiled module's tile rows differ from attention_tile_rows()")
@@ -753,11 +757,17 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _check(positions, "positions", (T,), torch.int32)
         part_o = torch.empty((T, nH, max_splits, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nH, max_splits, 2), dtype=torch.float32, device=q.device)
-    _call(mod, "ifx_attn_tiles", (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P),
+    per_xcd = 0
+    if order is not None:
+        _check(order, "order", (None,), torch.int32)
+        if order.shape[0] % 8:
+            raise KernelError("attention_tiles: the order has a place for each of 8 XCDs' workgroups")
+        per_xcd = order.shape[0] // 8
+    _call(mod, "ifx_attn_tiles", (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
           n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
           block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), int(chunk), int(max_splits),
-          _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _stream())
+          _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, _stream())
 
 
 # ----------------------------------------------------------------------------------------

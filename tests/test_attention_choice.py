@@ -2,7 +2,9 @@
 choice must satisfy for the kernel to be right."""
 import random
 
-from inferflux_amd.kernels.attention import TILE_MAX_SPLITS, choose_tiling
+import numpy as np
+
+from inferflux_amd.kernels.attention import TILE_MAX_SPLITS, choose_tiling, tile_order
 
 ROWS_OF = lambda qt: 64 * qt          # head size 128
 
@@ -16,7 +18,10 @@ def test_the_measured_cases_get_the_choice_that_was_fastest():
         ([1024], 4096, 28, (2, 2)),
         ([1024], 8192, 28, (2, 2)),
         ([512], 8192, 28, (2, 4)),
-        ([2048], 4096, 28, (2, 1)),     # 185 us against 236 with one tile per wave
+        ([2048], 2048, 28, (1, 1)),     # a short causal prompt: 75 us against 81 with two tiles per wave
+        ([2048], 2048, 16, (1, 1)),
+        ([4096], 4096, 28, (2, 1)),
+        ([2048], 4096, 28, (2, 1)),     # 158 us against 218 with one tile per wave
         ([2048], 8192, 28, (2, 1)),
         ([8192], 8192, 28, (2, 1)),
         ([2048], 2048, 40, (2, 1)),
@@ -24,12 +29,12 @@ def test_the_measured_cases_get_the_choice_that_was_fastest():
         ([100] * 16, 100, 28, (1, 1)),
     ]
     for rows, longest, heads, want in cases:
-        qt, splits, chunk = choose_tiling(rows, longest, heads, ROWS_OF)
+        qt, splits, chunk = choose_tiling(rows, [longest] * len(rows), heads, ROWS_OF)
         assert (qt, splits) == want, (rows, longest, heads, qt, splits, chunk)
 
 
 def test_a_short_portion_does_not_take_half_empty_tall_tiles():
-    qt, splits, chunk = choose_tiling([64], 8256, 28, ROWS_OF)
+    qt, splits, chunk = choose_tiling([64], [8256], 28, ROWS_OF)
     assert qt == 1 and splits > 8
 
 
@@ -39,9 +44,62 @@ def test_every_choice_covers_its_keys_in_splits_the_kernel_takes():
         rows = [rng.randint(16, rng.choice([40, 300, 3000])) for _ in range(rng.randint(1, 6))]
         longest = max(rows) + rng.choice([0, rng.randint(0, 500), rng.randint(0, 40000)])
         heads = rng.choice([1, 2, 5, 16, 28, 40, 64])
-        qt, splits, chunk = choose_tiling(rows, longest, heads, ROWS_OF)
+        qt, splits, chunk = choose_tiling(rows, [r + rng.randint(0, longest - r) for r in rows[:-1]] + [longest], heads, ROWS_OF)
         assert qt in (1, 2) and 1 <= splits <= TILE_MAX_SPLITS
         if splits > 1:
             assert chunk % 64 == 0 and splits * chunk >= longest > (splits - 1) * chunk
         else:
             assert chunk == 0
+
+
+def _walks(first, last, window, splits, chunk):
+    """Key tiles each (tile, split) walks, written out from the kernel's loop bounds."""
+    out = []
+    for f, l in zip(first, last):
+        row = []
+        for s in range(splits):
+            lo = max(f - window + 1, 0) if window else 0
+            hi = l
+            if splits > 1:
+                lo, hi = max(lo, s * chunk), min(hi, (s + 1) * chunk - 1)
+            j0, n = lo // 64 * 64, 0
+            while j0 <= hi:
+                n, j0 = n + 1, j0 + 64
+            row.append(n)
+        out.append(row)
+    return out
+
+
+def test_the_order_names_every_work_item_once_and_balances_the_units():
+    rng = random.Random(9)
+    for trial in range(200):
+        n_tiles, heads = rng.randint(1, 40), rng.choice([1, 4, 16, 28])
+        rows = rng.choice([64, 128])
+        start = rng.randint(0, 3000)
+        first = [start + rows * t for t in range(n_tiles)]
+        last = [f + rng.randint(1, rows) - 1 for f in first]
+        window = rng.choice([None, None, 100, 1000])
+        splits = rng.choice([1, 1, 2, 5])
+        chunk = -(-(last[-1] + 1) // splits + 63) // 64 * 64 if splits > 1 else 0
+        period = rng.choice([2, 3, 32])
+        order = tile_order(first, last, heads, window, splits, chunk, period)
+        n_items = n_tiles * heads * splits
+        assert order.dtype == np.int32 and order.shape[0] % 8 == 0 and order.shape[0] // 8 <= n_items
+        assert sorted(order[order >= 0].tolist()) == list(range(n_items))
+        assert set(order[order < 0].tolist()) <= {-1}
+    # a causal prompt of 2,048 rows in tiles of 64, 28 heads: the compute units' first three workgroups (unit = place
+    # modulo 32 within an XCD) walk 50-61 key tiles together on every unit, where longest first head by head gave 3 to 96
+    first = [64 * t for t in range(32)]
+    last = [f + 63 for f in first]
+    order = tile_order(first, last, 28, None, 1, 0).reshape(8, -1)
+    walks = _walks(first, last, None, 1, 0)
+    sums = []
+    for x in range(8):
+        unit = [0] * 32
+        for i, w in enumerate(order[x][:96]):
+            if w >= 0:
+                unit[i % 32] += walks[31 - w % 32][0]
+        sums += unit
+        # an XCD's workgroups read the keys of few kv heads (7 query heads each)
+        assert len({int(w) // 32 // 7 for w in order[x] if w >= 0}) <= 2
+    assert min(sums) >= 48 and max(sums) <= 62, (min(sums), max(sums))

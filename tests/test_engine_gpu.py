@@ -587,7 +587,7 @@ def test_prompt_portions_with_a_long_past_split_their_keys(sharp_folders, monkey
     The thresholds are lowered so that the tiny models' 250 and 380 tokens qualify."""
     from inferflux_amd.kernels import attention
     for name, value in (("TILE_SPLIT_MIN_KEYS", 64), ("TILE_SPLIT_MIN_LONGEST", 128), ("TILE_SPLIT_FEW_MIN_LONGEST", 128),
-                        ("TILE_SPLIT_FEW_MIN_KEYS", 64), ("TILE_QT2_MIN_KEYS", 300)):
+                        ("TILE_SPLIT_FEW_MIN_KEYS", 64), ("TILE_QT2_MIN_KEYS", 300), ("TILE_ORDER_MIN_ITEMS", 0)):
         monkeypatch.setattr(attention, name, value)
     calls = []
     real = attention.ops.attention_tiles

@@ -381,11 +381,29 @@ def test_attention_tiles(case, qt, split_chunk):
     if split_chunk:
         splits = dict(chunk=split_chunk, max_splits=-(-max(info["kv_lens"]) // split_chunk),
                       rows=torch.arange(T, dtype=torch.int32, device=DEV), row_req=row_req, positions=positions)
-    ops.attention_tiles(q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV),
-                        q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt, **splits)
+    call = (q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV),
+            q_len.to(DEV), dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt)
+    ops.attention_tiles(*call, **splits)
+    plain_order = out.clone()
     out = out.cpu().double()
     assert torch.isfinite(out).all()
     assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
+    # the same launch with its workgroups in the balanced order, and in a shuffled one with gaps: the same bits
+    import numpy as np
+    from inferflux_amd.kernels.attention import tile_order
+    first = np.asarray([info["kv_lens"][r] - info["q_lens"][r] + q0 for r, q0 in tiles])
+    last = np.asarray([min(f + ops.attention_tile_rows(d, qt), info["kv_lens"][r]) - 1 for f, (r, _) in zip(first, tiles)])
+    n_splits = splits.get("max_splits", 1)
+    balanced = tile_order(first, last, nH, window, n_splits, split_chunk, period=3)
+    n_items = len(tiles) * nH * n_splits
+    assert sorted(balanced[balanced >= 0].tolist()) == list(range(n_items))
+    rng = np.random.default_rng(3)
+    shuffled = np.full(8 * (n_items // 8 + 3), -1, np.int32)
+    shuffled[rng.permutation(shuffled.shape[0])[:n_items]] = rng.permutation(n_items)
+    for order in (balanced, shuffled):
+        again = torch.zeros(T, nH * d, dtype=BF16, device=DEV)
+        ops.attention_tiles(*call[:3], again, *call[4:], **splits, order=torch.from_numpy(order).to(DEV))
+        assert torch.equal(again, plain_order)
 
 
 def test_attention_tiles_refuses_splits_it_cannot_merge():
@@ -396,6 +414,10 @@ def test_attention_tiles_refuses_splits_it_cannot_merge():
         ops.attention_tiles(*args, chunk=100, max_splits=2, rows=dev(list(range(64))), row_req=row_req, positions=positions)
     with pytest.raises(ops.KernelError, match="rows to merge"):
         ops.attention_tiles(*args, chunk=128, max_splits=2)
+    with pytest.raises(ops.KernelError, match="cannot hold"):
+        ops.attention_tiles(*args, order=torch.full((40,), -1, dtype=torch.int32, device=DEV))   # 5 places per XCD for 4 items
+    with pytest.raises(ops.KernelError, match="each of 8"):
+        ops.attention_tiles(*args, order=torch.full((12,), -1, dtype=torch.int32, device=DEV))
 
 
 def test_mfma_attention_refuses_what_it_cannot_do():
