@@ -174,6 +174,43 @@ def main() -> int:
         attn = 4.0 * L * nH * d * tokens * (tokens + 1) / 2
         return tokens / best, best * 1e3, (linear + attn) / best / 1e12 / PEAK_TFLOPS[args.dtype], sum(times) / len(times) * 1e3
 
+    def phase_shares(batch, steps=4):
+        """Where the GPU's time goes, part by part: shares of the time between events recorded around each part in
+        steps that are run kernel by kernel (not as a graph): a prompt of ``PROMPT`` tokens, then decode steps at
+        ``batch`` with the contexts of the timed run.  Eager steps of few rows leave the GPU waiting for the host
+        now and then, which is booked to the part that was being launched; the graphs' own times are the
+        ``ms_per_step`` figures."""
+        from inferflux_amd.engine.tracing import PhaseTimer
+        runner = ModelRunner(model, num_pages=batch * (-(-(kv_start + steps) // PAGE) + 1), page_size=PAGE, max_requests=batch,
+                             phase_timing=True)
+        runner.timer.quiet = True
+        out = {}
+        for name, n_steps, tokens in ((f"prefill_{PROMPT}", 1, PROMPT), (f"decode_b{batch}", steps, 1)):
+            if name.startswith("prefill"):
+                runner.add_request("p")
+                runner.step([StepEntry("p", torch.randint(0, V, (PROMPT,), generator=gen).tolist(), [PROMPT - 1])])   # warms the library up
+                runner.free_request("p")
+                runner.add_request("p")
+                runner.timer = PhaseTimer(quiet=True)
+                runner.step([StepEntry("p", torch.randint(0, V, (PROMPT,), generator=gen).tolist(), [PROMPT - 1])])
+                runner.free_request("p")
+            else:
+                runner.timer = PhaseTimer(quiet=True)
+                for r in range(batch):
+                    runner.add_request(r)
+                    for a0 in range(0, kv_start, 8192):
+                        runner.step([StepEntry(r, torch.randint(0, V, (min(8192, kv_start - a0),), generator=gen).tolist(), [])])
+                runner.step([StepEntry(r, [1], [0]) for r in range(batch)])
+                runner.timer = PhaseTimer(quiet=True)
+                for _ in range(n_steps):
+                    runner.step([StepEntry(r, [1], [0]) for r in range(batch)])
+            total = sum(runner.timer.totals.values())
+            out[name] = {k: round(v, 4) for k, v in runner.timer.shares().items()}
+            out[name]["ms_eager"] = round(total / n_steps, 3)
+        del runner
+        torch.cuda.empty_cache()
+        return out
+
     def measured_ceilings():
         """What this card gives a kernel that only reads 2 GB (streaming loads), and the library's 8192^3 bfloat16
         product: the yardsticks beside the data sheet's 8 TB/s and 2.5 PFLOP/s."""
@@ -251,6 +288,7 @@ def main() -> int:
             out[f"ms_per_step_b{b}"] = round(bms, 4)
             out[f"roofline_b{b}"] = hbm_roofline(b, bms, bkv, ceil)
         out["points"] = points
+        out["phases"] = phase_shares(args.batch)
     print(json.dumps(out), flush=True)
     return 0
 

@@ -1,31 +1,37 @@
 """Per-phase timing of a forward pass, for finding where a step's time goes.
 
 Like the reference's PhaseTiming (runtime/backends/cuda/native/transformer_forward.cu:71-131,
-enabled there by INFERFLUX_CUDA_PHASE_TIMING=1): the stream is synchronised at every mark and the
-wall time since the previous mark is booked to a phase, so the GPU pipeline is serialised while
-it is on (the reference measured half the throughput, docs/benchmarks.md:193-199).  For
-debugging and profiling only; decode steps are not captured as graphs while it is on.  Each phase
-is also a range for the profiler's timeline (roctx through torch.cuda.nvtx, where available), in
-the place of the reference's NVTX_SCOPE.
+enabled there by INFERFLUX_CUDA_PHASE_TIMING=1), which synchronises the stream at every mark and
+measured half the throughput with it on (docs/benchmarks.md:193-199).  Here a mark records an event on
+the stream and the step is waited for once, at its end; the time between two events is booked to the
+phase that the later one names.  The GPU's work is not serialised against the host, so the figures are
+GPU time, including whatever the GPU waited for the host inside the phase (eager steps of few rows).
+Decode steps are not captured as graphs while it is on.  Each phase is also a range for the profiler's
+timeline (roctx through torch.cuda.nvtx, where available), in the place of the reference's NVTX_SCOPE.
+
+Blocks mark "norm", "mixer" and "ffn"; the attention mixer and the gated feed-forward mark their own
+stages before that ("mixer.qkv", "mixer.attention", "ffn.gate_up"; what is left for the block's mark
+is the output projection and the down projection).
 """
 from __future__ import annotations
 
 import sys
-import time
-from typing import Dict
+from typing import Dict, List, Tuple
 
 import torch
 
-PHASES = ("embed", "norm", "mixer", "ffn", "final_norm", "lm_head")
+PHASES = ("embed", "norm", "mixer.qkv", "mixer.attention", "mixer", "ffn.gate_up", "ffn", "final_norm", "lm_head")
 
 
 class PhaseTimer:
-    def __init__(self, report_every: int = 10, stream=None):
-        self.totals: Dict[str, float] = {p: 0.0 for p in PHASES}
-        self.step: Dict[str, float] = {}
+    def __init__(self, report_every: int = 10, quiet: bool = False):
+        self.totals: Dict[str, float] = {p: 0.0 for p in PHASES}     # ms, over all forwards
+        self.step: Dict[str, float] = {}                             # ms, the last forward
         self.forwards = 0
         self.report_every = report_every
-        self._last = 0.0
+        self.quiet = quiet
+        self._marks: List[Tuple[str, torch.cuda.Event]] = []
+        self._start = None
         try:
             torch.cuda.nvtx.range_push("inferflux_amd")
             torch.cuda.nvtx.range_pop()
@@ -34,10 +40,14 @@ class PhaseTimer:
             self._ranges = False
         self._open = False
 
+    def _event(self) -> torch.cuda.Event:
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        return e
+
     def begin(self) -> None:
-        torch.cuda.synchronize()
-        self.step = {}
-        self._last = time.perf_counter()
+        self._marks = []
+        self._start = self._event()
 
     def enter(self, name: str) -> None:
         """Open a profiler range for the phase that starts now."""
@@ -48,23 +58,32 @@ class PhaseTimer:
             self._open = True
 
     def mark(self, name: str) -> None:
-        """Book the time since the last mark to ``name``."""
-        torch.cuda.synchronize()
-        now = time.perf_counter()
-        ms = (now - self._last) * 1e3
-        self._last = now
-        self.step[name] = self.step.get(name, 0.0) + ms
-        self.totals[name] = self.totals.get(name, 0.0) + ms
+        """Book the GPU time since the last mark to ``name``."""
+        self._marks.append((name, self._event()))
 
     def end(self, n_layers: int, n_tokens: int) -> None:
         if self._ranges and self._open:
             torch.cuda.nvtx.range_pop()
             self._open = False
+        self.step = {}
+        if self._marks:
+            self._marks[-1][1].synchronize()
+            last = self._start
+            for name, ev in self._marks:
+                ms = last.elapsed_time(ev)
+                last = ev
+                self.step[name] = self.step.get(name, 0.0) + ms
+                self.totals[name] = self.totals.get(name, 0.0) + ms
         self.forwards += 1
-        if self.forwards <= 5 or self.forwards % self.report_every == 0:
+        if not self.quiet and (self.forwards <= 5 or self.forwards % self.report_every == 0):
             parts = " ".join(f"{k}={v:.2f}" for k, v in self.step.items())
             print(f"[phase_timing] #{self.forwards} L={n_layers} tokens={n_tokens} {parts} "
                   f"total={sum(self.step.values()):.2f} ms", file=sys.stderr, flush=True)
+
+    def shares(self) -> Dict[str, float]:
+        """Each phase's share of the time booked so far."""
+        total = sum(self.totals.values())
+        return {k: v / total for k, v in self.totals.items() if v > 0.0} if total > 0 else {}
 
 
 def kernel_trace_summary(csv_path: str, n_steps: int = 16, end_marker: str = "argmax_final") -> str:

@@ -98,19 +98,30 @@ class PagedAttention(Mixer):
                 self._w_q = self._prepare_qkv(w.rows[:width], self.n_heads)
             w, b = self._w_q, (b[:width] if b is not None else None)
         slots = ctx.write_slots(cache.group) if binding.writes_cache else None
+        t = ctx.timer
         if (style == ops.ROPE_SPLIT_HALF and rotary_dim == d and w.order is not None and h.dtype == torch.bfloat16
                 and h.shape[0] <= 16 and not self.position.needs_apply):
             # few tokens: the rotation and the cache write are the projection's epilogue
             q = ops.qkv_rope_append(h, w, b, slots, cos, sin, nH, nKV, d, cache.k if slots is not None else None,
                                     cache.v if slots is not None else None, cache.page_size)
-            return self._project_out(paged_attention(q, cache, ctx, self.window, self.scale), sink)
+            if t is not None:
+                t.mark("mixer.qkv")
+            a = paged_attention(q, cache, ctx, self.window, self.scale)
+            if t is not None:
+                t.mark("mixer.attention")
+            return self._project_out(a, sink)
         qkv = ops.linear(h, w, keep_slices=not self.position.needs_apply)     # the rotary kernel adds partial sums itself
         if self.position.needs_apply:
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
         q = ops.rope_append(qkv, b, slots, cos, sin, style, rotary_dim, nH, nKV, d,
                             cache.k if slots is not None else None, cache.v if slots is not None else None,
                             cache.page_size)
-        return self._project_out(paged_attention(q, cache, ctx, self.window, self.scale), sink)
+        if t is not None:
+            t.mark("mixer.qkv")
+        a = paged_attention(q, cache, ctx, self.window, self.scale)
+        if t is not None:
+            t.mark("mixer.attention")
+        return self._project_out(a, sink)
 
     def _encode_outside(self, qkv, bias, ctx, nKV):
         """For a position part that transforms q and k itself: add the bias, let the part encode,

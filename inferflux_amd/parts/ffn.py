@@ -59,6 +59,8 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx, sink=None):
         a = ops.linear_swiglu(h, self.w_gate_up)
+        if ctx.timer is not None:
+            ctx.timer.mark("ffn.gate_up")
         if sink is not None and ops.adds_into_stream(a.shape[0], self.w_down, sink.norm_weight):
             return ops.linear_into_stream(a, self.w_down, sink.stream, sink.norm_weight, sink.eps)
         return ops.linear(a, self.w_down, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself

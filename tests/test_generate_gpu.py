@@ -212,7 +212,9 @@ def test_phase_timing_and_cache_planning(model_folders, capfd):
     err = capfd.readouterr().err
     assert "[phase_timing] #1 L=4 tokens=20" in err and "mixer=" in err and "lm_head=" in err
     t = timed.runner.timer
-    assert t.forwards == 5 and all(t.totals[k] > 0 for k in ("embed", "norm", "mixer", "ffn", "final_norm", "lm_head"))
+    assert t.forwards == 5 and all(t.totals[k] > 0 for k in ("embed", "norm", "mixer.qkv", "mixer.attention", "mixer", "ffn.gate_up",
+                                                              "ffn", "final_norm", "lm_head"))
+    assert abs(sum(t.shares().values()) - 1.0) < 1e-6
 
 
 def test_logprobs_through_the_engine(model_folders):
