@@ -452,10 +452,12 @@ __device__ __forceinline__ void tile_math(const bf16_t* k_s, const bf16_t* v_s, 
 
 // The kernel waits on LDS and on the matrix pipe, so waves to switch to are worth more than the
 // registers they cost: 3 waves per SIMD with one query tile per wave (162 registers, no spill), 2 with two.
+#ifndef TILE_WAVES_PER_SIMD
 #if TILE_QT == 1
 #define TILE_WAVES_PER_SIMD 3
 #else
 #define TILE_WAVES_PER_SIMD 2
+#endif
 #endif
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TILE_WAVES_PER_SIMD, TILE_WAVES_PER_SIMD)))
 void attn_tiles_kernel(TileArgs a) {
