@@ -61,7 +61,8 @@ def load_spec_from_args(args):
                              kv_pages=args.kv_pages, page_size=args.page_size, max_batch_tokens=args.batch_size,
                              chunked_prefill_tokens=args.chunked_prefill_tokens,
                              decode_weight_copy=not args.no_decode_weight_copy,
-                             strict_weights=not args.allow_unused_tensors, phase_timing=args.phase_timing).checked()
+                             strict_weights=not args.allow_unused_tensors, phase_timing=args.phase_timing,
+                             library_gemm_tuning=args.gemm_tuning).checked()
     except LoadSpecError as e:
         raise SystemExit(f"inferctl: {e}")
 
@@ -164,7 +165,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     c.add_argument("--no-decode-weight-copy", action="store_true",
                    help="keep one copy of the weights only (saves their size in memory, decoding is slower)")
     c.add_argument("--phase-timing", action="store_true",
-                   help="print per-phase times of every forward pass (synchronises after each phase: slow)")
+                   help="print per-phase GPU times of every forward pass (decode steps then run kernel by kernel, not as graphs)")
+    c.add_argument("--gemm-tuning", action="store_true",
+                   help="let the library time its kernels for the matrix-product shapes of prompts (faster prompts once a shape "
+                        "is known; the first product of a shape takes up to 0.3 s longer)")
     c.set_defaults(fn=cmd_completion)
     r = sub.add_parser("random-weights", help="write a model folder with seeded random weights")
     r.add_argument("--config", required=True, help="a config.json")

@@ -82,6 +82,9 @@ def load_runner(folder, dtype: torch.dtype = torch.bfloat16, num_pages: Optional
     ``cache_tokens`` need, within the free device memory."""
     if isinstance(folder, ModelLoadSpec):
         spec = folder.checked()
+        if spec.library_gemm_tuning:
+            from ..kernels import ops
+            ops.enable_library_gemm_tuning()
         model = load_model(spec)
         num_pages = spec.kv_pages
         if num_pages is None:

@@ -38,7 +38,9 @@ class ModelLoadSpec:
     chunked_prefill_tokens: int = 512       # largest portion of a prompt in one step
     decode_weight_copy: bool = True         # keep the tiled second copy of bfloat16 projections for decoding
     strict_weights: bool = True             # tensors in the file that no part reads are an error (else a warning)
-    phase_timing: bool = False              # time every phase of every forward pass (slow)
+    phase_timing: bool = False              # time every phase of every forward pass
+    library_gemm_tuning: bool = False       # let the library time its kernels for every product shape of more than 64 rows it
+                                            # meets (prompts: about a quarter faster once a shape is known, up to 0.3 s the first time)
 
     def validate(self) -> str:
         """The first thing wrong with the spec as a sentence, or "" (the reference's convention)."""
