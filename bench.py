@@ -204,9 +204,23 @@ def main() -> int:
                 runner.timer = PhaseTimer(quiet=True)
                 for _ in range(n_steps):
                     runner.step([StepEntry(r, [1], [0]) for r in range(batch)])
-            total = sum(runner.timer.totals.values())
+            totals = dict(runner.timer.totals)
+            total = sum(totals.values())
             out[name] = {k: round(v, 4) for k, v in runner.timer.shares().items()}
             out[name]["ms_eager"] = round(total / n_steps, 3)
+            # what each stage moves or computes per step, over its time: GB/s of weights and cache for decoding (a stage is
+            # bound by reading them once), TFLOP/s for the prompt
+            if tokens == 1:
+                kv = kv_start + 1 + n_steps / 2
+                work = {"mixer.qkv": L * (nH + 2 * nKV) * d * (H + 1) * esz, "mixer.attention": L * batch * kv * 2 * nKV * d * esz,
+                        "mixer": L * nH * d * H * esz, "ffn.gate_up": L * 2 * I * H * esz, "ffn": L * I * H * esz, "lm_head": V * H * esz}
+                out[name + "_GBs"] = {k: round(b / (totals[k] / n_steps * 1e-3) / 1e9, 1) for k, b in work.items() if totals.get(k, 0) > 0}
+            else:
+                T = tokens
+                work = {"mixer.qkv": 2.0 * T * L * (nH + 2 * nKV) * d * H, "mixer.attention": 4.0 * L * nH * d * T * (T + 1) / 2,
+                        "mixer": 2.0 * T * L * nH * d * H, "ffn.gate_up": 2.0 * T * L * 2 * I * H, "ffn": 2.0 * T * L * I * H}
+                out[name + "_TFLOPs"] = {k: round(f / (totals[k] * 1e-3) / 1e12, 1) for k, f in work.items() if totals.get(k, 0) > 0}
+        out["how"] = "events around each part of steps run kernel by kernel (waits for the host included); a replayed step's own time is ms_per_step"
         del runner
         torch.cuda.empty_cache()
         return out
