@@ -116,34 +116,58 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   const TD* dl = delta ? delta + src * H : nullptr;
   float x[NV][4];
   float ss = 0.f;
+  // Every load that does not depend on another goes out before the first is used: the row and the delta (or
+  // its first slice) for all of the thread's elements, then the further slices four at a time for all elements.
+  // With the elements outermost a row of 8 slices cost a dozen trips to the L2 one after the other.
+  float w4[NV][4];                       // the norm's weight: asked for now, needed after the sum over the row
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     const int i = 4 * (threadIdx.x + 256 * v);
     if (i < H) {
       load4<float>(res + i, x[v]);
-      if (dl) {
-        float d4[4];
-        load4<TD>(dl + i, d4);
-        for (int s0 = 1; s0 < n_slices; s0 += 4) {   // partial sums, added in slice order; four loads go out together
-          float p4[4][4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            if (s0 + u < n_slices) load4<TD>(dl + (size_t)(s0 + u) * slice_stride + i, p4[u]);
-            else p4[u][0] = p4[u][1] = p4[u][2] = p4[u][3] = 0.f;
-          }
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) d4[e] += p4[u][e];
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[v][e] += d4[e];
-        if (write_back) store4<float>(res + i, x[v]);
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ss += x[v][e] * x[v][e];
+      load4<TW>(weight + i, w4[v]);
+    } else {
+      x[v][0] = x[v][1] = x[v][2] = x[v][3] = 0.f;
+      w4[v][0] = w4[v][1] = w4[v][2] = w4[v][3] = 0.f;
     }
   }
+  if (dl) {
+    float d4[NV][4];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int i = 4 * (threadIdx.x + 256 * v);
+      if (i < H) load4<TD>(dl + i, d4[v]);
+      else d4[v][0] = d4[v][1] = d4[v][2] = d4[v][3] = 0.f;
+    }
+    for (int s0 = 1; s0 < n_slices; s0 += 4) {   // partial sums, added in slice order
+      float p4[4][NV][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          const int i = 4 * (threadIdx.x + 256 * v);
+          if (s0 + u < n_slices && i < H) load4<TD>(dl + (size_t)(s0 + u) * slice_stride + i, p4[u][v]);
+          else p4[u][v][0] = p4[u][v][1] = p4[u][v][2] = p4[u][v][3] = 0.f;
+        }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) d4[v][e] += p4[u][v][e];
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int i = 4 * (threadIdx.x + 256 * v);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[v][e] += d4[v][e];
+      if (write_back && i < H) store4<float>(res + i, x[v]);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < NV; ++v)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += x[v][e] * x[v][e];
   ss = block_sum(ss, red);
   const float rms = rsqrtf(ss / (float)H + eps);
   TO* o = out + (size_t)r * H;
@@ -151,10 +175,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   for (int v = 0; v < NV; ++v) {
     const int i = 4 * (threadIdx.x + 256 * v);
     if (i < H) {
-      float w4[4], y[4];
-      load4<TW>(weight + i, w4);
+      float y[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) y[e] = x[v][e] * rms * w4[e];
+      for (int e = 0; e < 4; ++e) y[e] = x[v][e] * rms * w4[v][e];
       store4<TO>(o + i, y);
     }
   }
@@ -266,17 +289,22 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
   const float* part = (const float*)a.qkv + (size_t)t * row_width;
-  auto in = [&](int i) {
-    if (a.n_slices <= 1) return to_f(row[i]);
-    float x = part[i];
-    for (int s0 = 1; s0 < a.n_slices; s0 += 4) {   // four loads go out together
-      float p[4];
+  // Elements i0 and i1 of the row; partial sums are added in slice order, eight slices of both elements asked for
+  // together (one after the other every slice would cost a trip to the L2).
+  auto in2 = [&](int i0, int i1, float& x0, float& x1) {
+    if (a.n_slices <= 1) { x0 = to_f(row[i0]); x1 = to_f(row[i1]); return; }
+    for (int s0 = 0; s0 < a.n_slices; s0 += 8) {
+      float p0[8], p1[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) p[u] = s0 + u < a.n_slices ? part[(size_t)(s0 + u) * a.slice_stride + i] : 0.f;
+      for (int u = 0; u < 8; ++u) {
+        p0[u] = s0 + u < a.n_slices ? part[(size_t)(s0 + u) * a.slice_stride + i0] : 0.f;
+        p1[u] = s0 + u < a.n_slices ? part[(size_t)(s0 + u) * a.slice_stride + i1] : 0.f;
+      }
+      if (s0 == 0) { x0 = p0[0]; x1 = p1[0]; }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) x += p[u];
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u > 0) { x0 += p0[u]; x1 += p1[u]; }
     }
-    return x;
   };
   const int slot = a.slots ? a.slots[t] : -1;
   const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
@@ -295,7 +323,8 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
       } else {
         i0 = 2 * p; i1 = 2 * p + 1;  // beyond the rotated part pairs are consecutive in both styles
       }
-      float x0 = in(col + i0), x1 = in(col + i1);
+      float x0, x1;
+      in2(col + i0, col + i1, x0, x1);
       if (a.bias) {
         x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
         x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
@@ -313,10 +342,13 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
     if (slot < 0) return;
     const int kh = head - a.nH - a.nKV;
     T* vc = (T*)a.v_cache + ((size_t)page * a.nKV + kh) * d * a.page_size + off;
-    for (int e = threadIdx.x; e < d; e += blockDim.x) {
-      float x = in(col + e);
-      if (a.bias) x += load_dyn(a.bias, a.bias_dtype, col + e);
+    for (int e = threadIdx.x; e < d; e += 2 * blockDim.x) {     // two elements per thread and round: their loads go out together
+      const int e1 = min(e + (int)blockDim.x, d - 1);
+      float x, x1;
+      in2(col + e, col + e1, x, x1);
+      if (a.bias) { x += load_dyn(a.bias, a.bias_dtype, col + e); x1 += load_dyn(a.bias, a.bias_dtype, col + e1); }
       vc[(size_t)e * a.page_size] = from_f<T>(x);
+      if (e + (int)blockDim.x < d) vc[(size_t)e1 * a.page_size] = from_f<T>(x1);
     }
   }
 }
