@@ -365,3 +365,51 @@ def test_requests_added_and_aborted_between_steps_by_hand(early, model_folders):
     alone = Engine.load(folder, dtype="float32", kv_pages=40, max_batch_size=4)
     assert alone.generate([P["s"]], SamplingParams(temperature=0.9, top_p=0.95, seed=77, max_tokens=12, ignore_eos=True))[0].token_ids \
         == done["s"].token_ids
+
+
+@pytest.mark.parametrize("early", [True, False], ids=["early", "late"])
+@pytest.mark.parametrize("name,seed", [("C", 2), ("A", 3)])
+def test_random_arrivals_aborts_priorities_and_preemptions(name, seed, early, model_folders):
+    """Forty requests of random lengths, limits and priorities arrive at random steps and some are aborted at random,
+    through a cache too small for them (requests are preempted and recomputed).  Every finished request's tokens are
+    the plain model's, every aborted one's a beginning of them, the cache's books are right after every step and
+    every pool is whole at the end."""
+    import random
+    folder, V = model_folders[name], TINY[name]["vocab_size"]
+    cfg, W = pm.load_folder(folder, torch.float64)
+    rng = random.Random(seed * 7 + (1 if early else 0))
+    pages = rng.randint(14, 22)
+    eng = Engine.load(folder, dtype="float32", kv_pages=pages, max_batch_size=rng.randint(3, 6),
+                      chunked_prefill_tokens=rng.choice([8, 16, 24, 48]), max_batch_tokens=rng.choice([32, 64, 256]),
+                      start_steps_early=early)
+    reqs, done, aborted = {}, {}, {}
+    n_req, next_id, steps = 40, 0, 0
+    while next_id < n_req or eng.has_unfinished():
+        steps += 1
+        for _ in range(rng.choice([0, 0, 0, 1, 1, 2, 3])):
+            if next_id < n_req:
+                n_new = rng.randint(1, 30)
+                prompt = seeded_ids(seed * 1000 + next_id, rng.randint(1, min(110, pages * 16 - n_new - 1)), V)
+                eng.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True), f"r{next_id}",
+                                priority=rng.choice([0, 0, 0, 1, 2]))
+                reqs[f"r{next_id}"] = (prompt, n_new)
+                next_id += 1
+        live = [r for r in reqs if r not in done and r not in aborted]
+        if live and rng.random() < 0.08:
+            rid = rng.choice(live)
+            out = eng.abort(rid)
+            if out is not None:
+                aborted[rid] = out
+        for o in eng.step():
+            done[o.request_id] = o
+        eng.runner.manager.check()
+        assert steps < 5000, "the engine makes no progress"
+    assert eng.runner.manager.free_pages() == [pages] * len(eng.runner.manager.groups) and not eng.runner.manager.live()
+    assert set(done) | set(aborted) == set(reqs) and not set(done) & set(aborted)
+    assert eng.stats.preemptions > 0 and aborted and len(done) > 10          # the run did meet what it is about
+    for rid, (prompt, n_new) in reqs.items():
+        want = pm.greedy_generate(cfg, W, prompt, n_new)
+        if rid in done:
+            assert done[rid].finish_reason == "length" and done[rid].token_ids == want, rid
+        else:
+            assert aborted[rid].finish_reason == "abort" and aborted[rid].token_ids == want[:len(aborted[rid].token_ids)], rid
