@@ -84,9 +84,13 @@ struct RowArgs {
 
 // out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s.
 // One wave per (row, head): lane s first weighs split s, then every lane sums its elements over
-// the splits in ascending order.
+// the splits in ascending order.  The partial results of the first MERGE_EARLY splits are asked for together
+// with the maxima and sums, before their weights are known (a kernel this short is a chain of trips to the L2:
+// maxima, then weights, then the partial results cost three; so it is one for rows of up to 32 splits).
+constexpr int MERGE_EARLY = 32;
 __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
   __shared__ float w_s[WAVE];
+  constexpr int C = (D + WAVE - 1) / WAVE;
   const int ri = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int row = a.rows ? a.rows[ri] : ri;
   const int pos = a.positions[row];
@@ -95,23 +99,33 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
   const size_t pi = a.part_by_row ? row : ri;
   const float* po = a.part_o + (pi * a.nH + head) * a.max_splits * D;
   const float* pml = a.part_ml + (pi * a.nH + head) * a.max_splits * 2;
-  float acc[(D + WAVE - 1) / WAVE];
+  float acc[C];
 #pragma unroll
-  for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = 0.f;
+  for (int c = 0; c < C; ++c) acc[c] = 0.f;
   float L = 0.f;
   // Lane s of a round holds split sb + s; rows with more than 64 splits take further rounds.  The first
   // round's maxima and sums are kept from the pass that finds the maximum (the usual case is one round).
-  float M = -INFINITY, m_first = -INFINITY, l_first = 0.f;
-  for (int sb = s0; sb <= s1; sb += WAVE) {
+  const int n_first = min(WAVE, s1 - s0 + 1);
+  const float2 ml_first = lane < n_first ? *(const float2*)(pml + 2 * (s0 + lane)) : float2{-INFINITY, 0.f};
+  // A split that saw no key has weight 0 and its partial result may hold anything: what was read of it is
+  // dropped by a select below, never multiplied.
+  float early[MERGE_EARLY][C];
+#pragma unroll
+  for (int u = 0; u < MERGE_EARLY; ++u)
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int e = lane + c * WAVE;
+      early[u][c] = (u < n_first && e < D) ? po[(size_t)(s0 + u) * D + e] : 0.f;
+    }
+  float M = ml_first.x;
+  for (int sb = s0 + WAVE; sb <= s1; sb += WAVE) {
     const int s = sb + lane;
-    const float2 ml = s <= s1 ? *(const float2*)(pml + 2 * s) : float2{-INFINITY, 0.f};
-    if (sb == s0) { m_first = ml.x; l_first = ml.y; }
-    M = fmaxf(M, ml.x);
+    M = fmaxf(M, s <= s1 ? pml[2 * s] : -INFINITY);
   }
   M = wave_max(M);
   for (int sb = s0; sb <= s1; sb += WAVE) {
     const int s = sb + lane;
-    float ms = m_first, ls = l_first;
+    float ms = ml_first.x, ls = ml_first.y;
     if (sb != s0) {
       const float2 ml = s <= s1 ? *(const float2*)(pml + 2 * s) : float2{-INFINITY, 0.f};
       ms = ml.x; ls = ml.y;
@@ -122,16 +136,24 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
     w_s[lane] = w;
     __syncthreads();
     const int n = min(WAVE, s1 - sb + 1);
-    // sixteen splits at a time, so that their loads are in flight together (a step of a loop that waits
-    // for its own loads costs a trip to the L2 each); an empty split (weight 0) is never read, its
-    // scratch may hold anything
-    for (int i = 0; i < n; i += 16) {
-      float wi[16], val[16][(D + WAVE - 1) / WAVE];
+    int i = 0;
+    if (sb == s0) {
+#pragma unroll
+      for (int u = 0; u < MERGE_EARLY; ++u) {
+        const float wu = u < n ? w_s[u] : 0.f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) acc[c] = fmaf(wu, wu != 0.f ? early[u][c] : 0.f, acc[c]);
+      }
+      i = MERGE_EARLY;
+    }
+    // the rest sixteen splits at a time, so that their loads are in flight together
+    for (; i < n; i += 16) {
+      float wi[16], val[16][C];
 #pragma unroll
       for (int u = 0; u < 16; ++u) {
         wi[u] = i + u < n ? w_s[i + u] : 0.f;
 #pragma unroll
-        for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
+        for (int c = 0; c < C; ++c) {
           const int e = lane + c * WAVE;
           val[u][c] = (wi[u] != 0.f && e < D) ? po[(size_t)(sb + i + u) * D + e] : 0.f;
         }
@@ -139,15 +161,14 @@ __global__ __launch_bounds__(WAVE) void attn_rows_merge_kernel(RowArgs a) {
 #pragma unroll
       for (int u = 0; u < 16; ++u)
 #pragma unroll
-        for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) acc[c] = fmaf(wi[u], val[u][c], acc[c]);
+        for (int c = 0; c < C; ++c) acc[c] = fmaf(wi[u], val[u][c], acc[c]);
     }
   }
   L = wave_sum(L);
   const float inv = L > 0.f ? 1.f / L : 0.f;
 #pragma unroll
-  for (int c = 0; c < (D + WAVE - 1) / WAVE; ++c) {
+  for (int c = 0; c < C; ++c) {
     const int e = lane + c * WAVE;
     if (e < D) a.out[((size_t)row * a.nH + head) * D + e] = (bf16_t)(acc[c] * inv);
   }
 }
-
