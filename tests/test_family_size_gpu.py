@@ -71,8 +71,8 @@ def test_bfloat16_engine_follows_the_float32_engine_at_7b_layer_sizes(runners):
 
 # ---- one layer at each family shape against the plain model ----------------------------------------------------
 # The layer shapes of Qwen2.5-7B, -3B and -14B (query : kv heads 7:1, 8:1, 5:1 at head size 128; feed-forward
-# widths 18,944 / 11,008 / 13,824; the 152,064- and 151,936-row vocabularies), one layer each and a tied head to
-# keep the folders small.  The oracle is the plain implementation in float32 on the CPU, which reads the folder
+# widths 18,944 / 11,008 / 13,824; the 152,064- and 151,936-row vocabularies) and of the small members -0.5B (head
+# size 64, width 896 = 7 x 128) and -1.5B (6:1), one layer each and a tied head to keep the folders small.  The oracle is the plain implementation in float32 on the CPU, which reads the folder
 # with the safetensors package: gate/up of 37,888 x 3,584, down with K = 18,944 and the head meet something that
 # is not the engine here.
 FAMILY = {
@@ -82,13 +82,19 @@ FAMILY = {
                rms_norm_eps=1e-6),
     "14B": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=13824, vocab_size=152064,
                 rms_norm_eps=1e-5),
+    # the small members: head size 64 on a width of 7 x 128, and 6 query heads to a kv head
+    "0.5B": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864, vocab_size=151936,
+                 rms_norm_eps=1e-6, head_dim=64),
+    "1.5B": dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960, vocab_size=151936,
+                 rms_norm_eps=1e-6),
 }
 N_TOKENS = 130
 # Largest difference to the plain model's (float64) logits over the largest logit.  Measured: float32 7.0e-6 / 4.7e-6 /
 # 1.04e-5 at the 7B / 3B / 14B shapes, the same under every cutting (sums of up to 18,944 products in float32);
-# bfloat16 1.72e-2 / 1.38e-2 / 2.08e-2 whole and by single rows, 1.32e-2 / 1.09e-2 / 1.54e-2 in portions of 17.
+# bfloat16 1.72e-2 / 1.38e-2 / 2.08e-2 whole and by single rows, 1.32e-2 / 1.09e-2 / 1.54e-2 in portions of 17; at the 0.5B and
+# 1.5B shapes float32 2.5e-6 / 3.8e-6 and bfloat16 8.9e-3 / 1.32e-2.
 # The bounds are those figures and half as much again (float32: the tiny configurations' 2e-5).
-FAMILY_TOL = {"float32": 2e-5, "bfloat16": {"7B": 2.6e-2, "3B": 2.1e-2, "14B": 3.1e-2}}
+FAMILY_TOL = {"float32": 2e-5, "bfloat16": {"7B": 2.6e-2, "3B": 2.1e-2, "14B": 3.1e-2, "0.5B": 1.35e-2, "1.5B": 2.0e-2}}
 
 
 def _write_family_folder(folder, name):
@@ -98,12 +104,12 @@ def _write_family_folder(folder, name):
     import json
     import os
     from safetensors.torch import save_file
-    shape = FAMILY[name]
-    cfg = dict(model_type="qwen2", architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, head_dim=128,
+    shape = dict({"head_dim": 128}, **FAMILY[name])
+    cfg = dict(model_type="qwen2", architectures=["Qwen2ForCausalLM"], num_hidden_layers=1,
                max_position_embeddings=4096, rope_theta=1000000.0, tie_word_embeddings=True, attention_bias=True,
                hidden_act="silu", torch_dtype="bfloat16", **shape)
     H, nH, nKV, I, V, d = (shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"],
-                           shape["intermediate_size"], shape["vocab_size"], 128)
+                           shape["intermediate_size"], shape["vocab_size"], shape["head_dim"])
     g = torch.Generator(device="cuda").manual_seed(1000 + H)
 
     def normal(*size, std=0.02):
