@@ -1,7 +1,8 @@
-"""The kernels at the sizes of the model family (Qwen2.5-7B layer shape: hidden 3584, 28 query heads
-on 4 kv heads of 128, feed-forward 18944, vocabulary 152064; two layers to keep it short): the
-bfloat16 engine against the float32 engine on the same weights, under several cuttings.  The
-float32 engine is the reference here; the tiny configurations tie it to the plain implementation."""
+"""The kernels at the sizes of the model family.  First two layers of the Qwen2.5-7B shape (hidden 3584, 28 query
+heads on 4 kv heads of 128, feed-forward 18944, vocabulary 152064): the bfloat16 engine against the float32 engine
+on the same weights under several cuttings, and the float32 engine bit-equal to itself.  Then one layer at each of
+the 7B, 3B, 14B, 0.5B and 1.5B shapes, written as a folder by the test itself, against the plain model in float64
+on the CPU, in both precisions and three cuttings."""
 import pytest
 import torch
 
