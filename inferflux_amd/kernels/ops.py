@@ -248,8 +248,9 @@ def enable_library_gemm_tuning(max_ms_per_shape: int = 300, filename: Optional[s
     tunable.set_max_tuning_duration(int(max_ms_per_shape))
     if not filename:
         import os
-        import tempfile
-        filename = os.path.join(tempfile.gettempdir(), f"inferflux_amd-{os.getuid()}-tunableop.csv")
+        from .library import _fallback_dir
+        # this user's private folder under the temporary directory (refused if somebody else made it or may write it)
+        filename = os.path.join(_fallback_dir(create=True), "tunableop.csv")
     tunable.set_filename(filename)     # choices are kept there and reused by later runs
 
 
