@@ -34,10 +34,40 @@ ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits 
 ROW_MAX_SPLITS = 128  # and until a row has at most this many splits (one row over 131,072 keys: 91 us against 133 at 64)
 
 
-def choose_tiling(tiled_rows, tiled_keys, n_heads: int, rows_of):
-    """(query tiles per wave, key splits, keys per split) for a launch of the tile kernel: ``tiled_rows`` the row
-    counts of the requests it covers, ``tiled_keys`` how many keys each of them holds after the step,
-    ``rows_of(qt)`` a tile's rows.
+DIRECT_MIN_WORK = 1 << 18       # rows x keys seen per row from which the tall tiles of head size 128 win
+DIRECT_SPLIT_FEW = 64           # at most this many workgroups: splits from 2,048 keys on,
+DIRECT_SPLIT_BELOW = 128        # at most this many: from 3,072 keys on; more workgroups are never split
+DIRECT_SPLIT_MIN_KEYS = 512
+
+
+def _choose_direct(tiled_rows, tiled_keys, n_heads: int, rows_of, total: int, longest: int, seen: float):
+    """``choose_tiling`` for head size 128, where the tall tiles are the kernel that loads straight into LDS.
+    Measured (28, 16 and 40 query heads, workgroups in ``tile_order``; us with tiles of 64 / of 128 rows, each with
+    its best number of splits): 512 rows 20 / 24, 1,024 rows 37 / 30, 2,048 rows 77 / 58, 8,192 rows 865 / 533;
+    512 rows after 512 keys 34 / 27, after 3,584 keys 96 / 69 (85 whole), 1,024 after 3,072 141 / 93 (117 in two
+    splits), 128 after 3,968 41 / 34 (83 whole), 2,048 after 6,144 436 / 226.  The tall tiles win wherever there
+    is work enough, and their keys want cutting only for few workgroups with long walks."""
+    n_big = sum(-(-int(n) // rows_of(2)) for n in tiled_rows)
+    if total * seen < DIRECT_MIN_WORK or n_big * rows_of(2) > 2 * total:
+        return None
+    groups = n_big * n_heads
+    splits, chunk = 1, 0
+    if (groups <= DIRECT_SPLIT_FEW and longest >= 2048) or (groups <= DIRECT_SPLIT_BELOW and longest >= 3072):
+        want = min(max(1, (2 * TILE_SPLIT_TARGET + groups) // (2 * groups)), longest // DIRECT_SPLIT_MIN_KEYS, TILE_MAX_SPLITS)
+        if want > 1:
+            chunk = (-(-longest // want) + 63) // 64 * 64
+            splits = -(-longest // chunk)
+            if splits <= 1:
+                splits, chunk = 1, 0
+    return 2, splits, chunk
+
+
+def choose_tiling(tiled_rows, tiled_keys, n_heads: int, rows_of, tall_direct: bool = False):
+    """(tiling: 1 = tiles of 64 rows, 2 = of 128; key splits; keys per split) for a launch of the tile kernel:
+    ``tiled_rows`` the row counts of the requests it covers, ``tiled_keys`` how many keys each of them holds after
+    the step, ``rows_of(qt)`` a tile's rows, ``tall_direct`` whether the tall tiles are the kernel of head size 128
+    (``_choose_direct`` then decides whether to take them).  What follows is measured on the other kernel, whose
+    tall tiles are two query tiles per wave.
 
     Measured at head size 128 (28, 16 and 40 query heads; portions of 256-8,192 rows after pasts of 0-7,680 keys,
     workgroups in ``tile_order``): two query tiles per wave win when they still give two workgroups to each compute
@@ -52,7 +82,11 @@ def choose_tiling(tiled_rows, tiled_keys, n_heads: int, rows_of):
     seen = sum(int(n) * (int(k) - int(n) / 2.0) for n, k in zip(tiled_rows, tiled_keys)) / max(total, 1)
     n_big = sum(-(-int(n) // rows_of(2)) for n in tiled_rows)
     qt = 1
-    if n_big * n_heads >= TILE_QT2_MIN_WORKGROUPS:
+    if tall_direct:
+        direct = _choose_direct(tiled_rows, tiled_keys, n_heads, rows_of, total, longest, seen)
+        if direct is not None:
+            return direct
+    elif n_big * n_heads >= TILE_QT2_MIN_WORKGROUPS:
         qt = 2
     elif seen >= TILE_QT2_MIN_KEYS and n_big * rows_of(2) * 2 <= total * 3:
         qt = 2
@@ -170,7 +204,8 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     tiled = ctx.h_q_len >= TILE_MIN
     qt, splits, chunk = 1, 1, 0
     if tiled.any():
-        qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], ctx.h_kv_len[tiled], nH, lambda t: ops.attention_tile_rows(d, t))
+        qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], ctx.h_kv_len[tiled], nH, lambda t: ops.attention_tile_rows(d, t),
+                                          tall_direct=d == ops.DIRECT_TILE_HEAD_DIM)
     tile_rows = ops.attention_tile_rows(d, qt)
     w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk, window),
                     lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk, window))

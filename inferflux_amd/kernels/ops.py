@@ -29,10 +29,12 @@ ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
 # first runs; these sizes are compiled ahead by build_all().
 MFMA_HEAD_DIMS_PREBUILT = (16, 32, 64, 128)
 MFMA_MAX_HEAD_DIM = 128
-# Query tiles of 16 rows per wave in the tile kernel: 2 (128 rows per workgroup) reuses each key and
-# value operand twice and is faster once there are enough workgroups to fill the chip; 1 (64 rows)
-# gives twice as many workgroups for short portions.
+# The tile kernel's two tilings: 1 = tiles of 64 rows (four waves of 16), which give twice as many workgroups for
+# short portions; 2 = tiles of 128 rows, in which every key and value fetched serves twice as many rows.  At head
+# size 128 the tall tiles are the kernel of attn_prefill.hip (eight waves of 16 rows, tiles loaded straight into
+# LDS), at the other head sizes attn_mfma.hip's with two query tiles per wave.
 TILE_QTS = (1, 2)
+DIRECT_TILE_HEAD_DIM = 128
 
 
 class KernelError(RuntimeError):
@@ -50,7 +52,14 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("ceilings", ())            # measurement only: what the memory gives a kernel that just reads
     for d in MFMA_HEAD_DIMS_PREBUILT:
         for qt in TILE_QTS:
-            yield ("attn_mfma", (("HEAD_DIM", d), ("TILE_QT", qt)))
+            yield _tile_module(d, qt)[:2]
+
+
+def _tile_module(head_dim: int, qt: int):
+    """(module, variant, entry point, the function that says its tile rows) of the tile kernel for a tiling."""
+    if qt == 2 and head_dim == DIRECT_TILE_HEAD_DIM:
+        return "attn_prefill", (("HEAD_DIM", head_dim),), "ifx_attn_prefill", "ifx_attn_prefill_tile_rows"
+    return "attn_mfma", (("HEAD_DIM", head_dim), ("TILE_QT", qt)), "ifx_attn_tiles", "ifx_attn_tile_rows"
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -685,7 +694,8 @@ def _attn_common(q, k_cache, v_cache, qt=1):
     if not mfma_attention_supported(q.dtype, d, page_size):
         raise KernelError(f"matrix-core attention needs bfloat16, head_dim a multiple of 16 up to {MFMA_MAX_HEAD_DIM} and "
                           f"page_size a power of two from 16; got head_dim {d}, page_size {page_size}")
-    return T, nH, d, nKV, page_size, load_module("attn_mfma", (("HEAD_DIM", d), ("TILE_QT", qt)))
+    name, variant, _, _ = _tile_module(d, qt)
+    return T, nH, d, nKV, page_size, load_module(name, variant)
 
 
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -712,9 +722,8 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
-    """Rows per tile of the tile kernel with ``qt`` query tiles per wave: four waves of ``qt`` tiles of 16 rows
-    (the compiled module says the same, ``ifx_attn_tile_rows``; asking it would compile a variant that a
-    short step never runs)."""
+    """Rows per tile of the tile kernel in tiling ``qt`` (see TILE_QTS; the compiled module says the same; asking it
+    would compile a variant that a short step never runs)."""
     return 64 * qt
 
 
@@ -735,7 +744,8 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     ``order`` (int32 [8 * n], from ``attention.tile_order``) says which work item each workgroup of the launch
     takes; every item must appear exactly once (-1: a workgroup without work).  The result does not depend on it."""
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt)
-    if mod.fn("ifx_attn_tile_rows", ())() != attention_tile_rows(d, qt):
+    _, _, entry, rows_fn = _tile_module(d, qt)
+    if mod.fn(rows_fn, ())() != attention_tile_rows(d, qt):
         raise KernelError("attention_tiles: the compiled module's tile rows differ from attention_tile_rows()")
     _check(out, "out", (T, nH * d), torch.bfloat16)
     n_tiles = tile_req.shape[0]
@@ -764,7 +774,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if order.shape[0] % 8:
             raise KernelError("attention_tiles: the order has a place for each of 8 XCDs' workgroups")
         per_xcd = order.shape[0] // 8
-    _call(mod, "ifx_attn_tiles", (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, P),
+    _call(mod, entry, (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
           n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
           block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), int(chunk), int(max_splits),

@@ -9,7 +9,37 @@ from inferflux_amd.kernels.attention import TILE_MAX_SPLITS, choose_tiling, tile
 ROWS_OF = lambda qt: 64 * qt          # head size 128
 
 
-def test_the_measured_cases_get_the_choice_that_was_fastest():
+def test_head_size_128_gets_the_choices_that_were_fastest():
+    """Tiles of 64 rows / of 128 rows (the kernel that loads straight into LDS), in us, each with its best splits."""
+    cases = [  # rows of the portion, keys it sees, query heads -> (tiling, key splits)
+        ([512], 512, 28, (1, 1)),        # 20 / 24
+        ([1024], 1024, 28, (2, 1)),      # 37 / 30
+        ([2048], 2048, 28, (2, 1)),      # 77 / 58
+        ([8192], 8192, 28, (2, 1)),      # 865 / 533
+        ([512], 1024, 28, (2, 1)),       # 34 / 27
+        ([512], 2048, 28, (2, 1)),       # 62 / 47 (55 in four splits)
+        ([512], 2048, 16, (2, 4)),       # 47 / 41 in four splits (47 whole)
+        ([512], 4096, 28, (2, 4)),       # 96 / 69 (85 whole)
+        ([256], 4096, 28, (2, 8)),       # 59 / 45 (84 whole)
+        ([1024], 4096, 28, (2, 1)),      # 141 / 93 (117 in two splits)
+        ([1024], 8192, 28, (2, 1)),      # 258 / 176 (174 in four splits)
+        ([512], 8192, 28, (2, 4)),       # 151 / 99 (164 whole)
+        ([128], 4096, 28, (2, 8)),       # 41 / 34 (83 whole)
+        ([128], 8192, 28, (2, 16)),      # 56 / 40
+        ([2048], 8192, 28, (2, 1)),      # 436 / 226
+        ([2048], 4096, 16, (2, 1)),      # 131 / 93
+        ([2048], 8192, 40, (2, 1)),      # 586 / 372
+        ([130], 130, 28, (1, 1)),
+        ([70] * 16, 70, 28, (1, 1)),     # sixteen short prompts: tall tiles would be half empty
+    ]
+    for rows, longest, heads, want in cases:
+        qt, splits, chunk = choose_tiling(rows, [longest] * len(rows), heads, ROWS_OF, tall_direct=True)
+        assert (qt, splits) == want, (rows, longest, heads, qt, splits, chunk)
+    qt, splits, _ = choose_tiling([64], [4096], 28, ROWS_OF, tall_direct=True)        # a half-empty tall tile: 26 us, this 30
+    assert qt == 1 and splits >= 8
+
+
+def test_other_head_sizes_get_the_choices_measured_with_two_query_tiles_per_wave():
     cases = [  # rows of the portion, keys it sees, query heads -> (query tiles per wave, key splits)
         ([512], 1024, 28, (1, 1)),      # 34 us whole against 40 in two splits
         ([512], 1024, 16, (1, 4)),      # half as many workgroups: 29 us in four splits against 33
@@ -44,7 +74,8 @@ def test_every_choice_covers_its_keys_in_splits_the_kernel_takes():
         rows = [rng.randint(16, rng.choice([40, 300, 3000])) for _ in range(rng.randint(1, 6))]
         longest = max(rows) + rng.choice([0, rng.randint(0, 500), rng.randint(0, 40000)])
         heads = rng.choice([1, 2, 5, 16, 28, 40, 64])
-        qt, splits, chunk = choose_tiling(rows, [r + rng.randint(0, longest - r) for r in rows[:-1]] + [longest], heads, ROWS_OF)
+        qt, splits, chunk = choose_tiling(rows, [r + rng.randint(0, longest - r) for r in rows[:-1]] + [longest], heads, ROWS_OF,
+                                          tall_direct=rng.random() < 0.5)
         assert qt in (1, 2) and 1 <= splits <= TILE_MAX_SPLITS
         if splits > 1:
             assert chunk % 64 == 0 and splits * chunk >= longest > (splits - 1) * chunk

@@ -179,8 +179,8 @@ def test_one_layer_of_each_family_shape_against_the_plain_model(name, tmp_path):
 
 def test_portions_behind_long_pasts_at_the_7b_layer_shape(monkeypatch):
     """A sequence of 3,000 tokens through one layer of the 7B shape in portions whose pasts grow to 2,364 keys: the
-    tile kernel then runs with one and with two query tiles per wave, its keys in two to five splits of several
-    lengths, its workgroups in the balanced order.  Every cutting stays as close to the float32 engine (run whole)
+    tile kernels then run with tiles of 64 and of 128 rows, their keys whole and in splits of several lengths, their
+    workgroups in the balanced order.  Every cutting stays as close to the float32 engine (run whole)
     as the uncut bfloat16 run does."""
     from inferflux_amd.config import config_from_dict
     from inferflux_amd.engine.context import StepEntry
@@ -190,7 +190,7 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(monkeypatch):
     cfg = config_from_dict(dict(SHAPE, num_hidden_layers=1, tie_word_embeddings=True, max_position_embeddings=8192))
     N, last = 3000, 24
     ids = seeded_ids(5, N, SHAPE["vocab_size"])
-    cuttings = ([N], [700, 1100, 64, 500, 636], [1024, 1024, 952], [256] * 11 + [184])
+    cuttings = ([N], [700, 1100, 64, 500, 636], [1024, 1024, 952], [256] * 11 + [184], [2560, 128, 312])
     wanted = sorted({sum(c[:i + 1]) - 1 - k for c in cuttings for i in range(len(c)) for k in range(min(last, c[i]))})
     tilings = set()
     real = attention.choose_tiling
@@ -214,4 +214,4 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(monkeypatch):
         e = rel_err(run(torch.bfloat16, cuts), ref)
         print(f"7B layer, 3,000 tokens in {len(cuts)} portions: {e:.2e}", flush=True)
         assert e < FAMILY_TOL["bfloat16"]["7B"], (cuts, e)        # measured 1.4e-2 to 1.7e-2, whole and cut alike
-    assert {t[0] for t in tilings} == {1, 2} and len({t[1] for t in tilings}) >= 4, tilings
+    assert {t[0] for t in tilings} == {1, 2} and len({t[1] for t in tilings}) >= 3, tilings

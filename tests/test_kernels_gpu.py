@@ -333,6 +333,11 @@ MFMA_CASES = [c for c in ATTN_CASES if c[4] % 16 == 0 and c[4] <= 128] + [
     ([1, 1], [5000, 300], 2, 1, 128, 64, 1000, None),              # a window inside a long context, pages of 64
     ([40, 3], [30, 170], 6, 3, 96, 16, None, 20),                  # head sizes between the prebuilt ones
     ([90], [75], 5, 1, 80, 32, 50, None),
+    # head size 128, where tiles of 128 rows are the kernel that loads straight into LDS: requests that end inside a
+    # tile, pages of 32, a window across tiles, a long past with a planted key, seven query heads to a kv head
+    ([300, 130], [500, 0], 8, 2, 128, 32, None, 100),
+    ([129], [260], 4, 4, 128, 16, 200, None),
+    ([260, 17], [3000, 40], 14, 2, 128, 16, None, 1500),
 ]
 
 
