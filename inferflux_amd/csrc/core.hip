@@ -107,6 +107,52 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const floa
 template <typename TD, typename TO, typename TW, int NV>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                                               const TW* __restrict__ weight, TO* __restrict__ out,
+                                                              const int* __restrict__ rows, int H, float eps, int write_back) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* res = residual + src * H;
+  const TD* dl = delta ? delta + src * H : nullptr;
+  float x[NV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int i = 4 * (threadIdx.x + 256 * v);
+    if (i < H) {
+      load4<float>(res + i, x[v]);
+      if (dl) {
+        float d4[4];
+        load4<TD>(dl + i, d4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[v][e] += d4[e];
+        if (write_back) store4<float>(res + i, x[v]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += x[v][e] * x[v][e];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rms = rsqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)r * H;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int i = 4 * (threadIdx.x + 256 * v);
+    if (i < H) {
+      float w4[4], y[4];
+      load4<TW>(weight + i, w4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = x[v][e] * rms * w4[e];
+      store4<TO>(o + i, y);
+    }
+  }
+}
+
+
+// The same with the delta given as float partial sums (n_slices of them, slice_stride elements apart, added in slice
+// order): the few rows of a decode step, where the kernel's time is its chain of trips to the L2.
+template <typename TD, typename TO, typename TW, int NV>
+__global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                                              const TW* __restrict__ weight, TO* __restrict__ out,
                                                               const int* __restrict__ rows, int H, float eps, int write_back,
                                                               int n_slices, size_t slice_stride) {
   __shared__ float red[16];
@@ -119,17 +165,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   // Every load that does not depend on another goes out before the first is used: the row and the delta (or
   // its first slice) for all of the thread's elements, then the further slices four at a time for all elements.
   // With the elements outermost a row of 8 slices cost a dozen trips to the L2 one after the other.
-  float w4[NV][4];                       // the norm's weight: asked for now, needed after the sum over the row
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     const int i = 4 * (threadIdx.x + 256 * v);
-    if (i < H) {
-      load4<float>(res + i, x[v]);
-      load4<TW>(weight + i, w4[v]);
-    } else {
-      x[v][0] = x[v][1] = x[v][2] = x[v][3] = 0.f;
-      w4[v][0] = w4[v][1] = w4[v][2] = w4[v][3] = 0.f;
-    }
+    if (i < H) load4<float>(res + i, x[v]);
+    else x[v][0] = x[v][1] = x[v][2] = x[v][3] = 0.f;
   }
   if (dl) {
     float d4[NV][4];
@@ -175,9 +215,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   for (int v = 0; v < NV; ++v) {
     const int i = 4 * (threadIdx.x + 256 * v);
     if (i < H) {
-      float y[4];
+      float w4[4], y[4];
+      load4<TW>(weight + i, w4);      // (asked for only now: held across the sum, it costs registers that many-row launches miss)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) y[e] = x[v][e] * rms * w4[v][e];
+      for (int e = 0; e < 4; ++e) y[e] = x[v][e] * rms * w4[e];
       store4<TO>(o + i, y);
     }
   }
@@ -186,15 +227,19 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 template <typename TD, typename TO, typename TW>
 static void launch_rmsnorm_vec(float* residual, const void* delta, const void* weight, void* out, const int* rows,
                                int n_rows, int H, float eps, int write_back, int n_slices, size_t slice_stride, hipStream_t s) {
-  if (H <= 4 * 256 * 2)
-    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 2>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
-                       (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);
-  else if (H <= 4 * 256 * 4)
-    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 4>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
-                       (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);
-  else
-    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, 8>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta,
-                       (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);
+#define GO(NV_)                                                                                                              \
+  do {                                                                                                                       \
+    if (n_slices > 1)                                                                                                        \
+      hipLaunchKernelGGL((add_rmsnorm_slices_kernel<TD, TO, TW, NV_>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta, \
+                         (const TW*)weight, (TO*)out, rows, H, eps, write_back, n_slices, slice_stride);                      \
+    else                                                                                                                     \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TO, TW, NV_>), dim3(n_rows), dim3(256), 0, s, residual, (const TD*)delta, \
+                         (const TW*)weight, (TO*)out, rows, H, eps, write_back);                                              \
+  } while (0)
+  if (H <= 4 * 256 * 2) GO(2);
+  else if (H <= 4 * 256 * 4) GO(4);
+  else GO(8);
+#undef GO
 }
 
 // n_slices > 1: ``delta`` (float32) holds that many partial sums, slice_stride elements apart, added in order.
