@@ -165,24 +165,30 @@ def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk
     row_mask = ~tiled[ctx.h_row_req] if ctx.n_tokens else np.zeros(0, bool)
     rows = np.nonzero(row_mask)[0].astype(np.int32)
     out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1,
-           "tile_splits": 1, "tile_chunk": 0, "tile_row_list": None}
-    out["tile_order"] = None
+           "tile_splits": 1, "tile_chunk": 0, "tile_row_list": None, "tile_order": None}
+    lists = {}                       # everything that goes to the device, in one copy (each copy is a wait for the host)
     if tile_req:
         tile_req, tile_q0 = np.asarray(tile_req, np.int32), np.asarray(tile_q0, np.int32)
-        out["tile_req"] = ctx.upload(tile_req)
-        out["tile_q0"] = ctx.upload(tile_q0)
+        lists["tile_req"], lists["tile_q0"] = tile_req, tile_q0
         if len(tile_req) * n_heads * tile_splits > TILE_ORDER_MIN_ITEMS:
             first = (kv_len[tile_req] - q_len[tile_req] + tile_q0).astype(np.int64)
             last = np.minimum(first + tile_rows, kv_len[tile_req]) - 1
-            out["tile_order"] = ctx.upload(tile_order(first, last, n_heads, window, tile_splits, tile_chunk))
+            lists["tile_order"] = tile_order(first, last, n_heads, window, tile_splits, tile_chunk)
         # Few tiles with many keys each (portions of prompts with a long past) leave most of the chip idle
         # and each workgroup walking its keys alone: the keys are cut into splits that run side by side.
         if tile_splits > 1:
             out["tile_splits"], out["tile_chunk"] = tile_splits, tile_chunk
-            out["tile_row_list"] = ctx.upload(np.nonzero(~row_mask)[0].astype(np.int32))
+            lists["tile_row_list"] = np.nonzero(~row_mask)[0].astype(np.int32)
+    if rows.size and rows.size != ctx.n_tokens:
+        lists["rows"] = rows
+    if lists:
+        sizes = [(k, v.shape[0]) for k, v in lists.items()]
+        packed = ctx.upload(np.concatenate([np.concatenate([v, np.zeros(-v.shape[0] % 4, np.int32)]) for v in lists.values()]))
+        at = 0
+        for k, n in sizes:
+            out[k] = packed[at:at + n]
+            at += n + -n % 4          # every list starts at a multiple of 16 bytes
     if rows.size:
-        if rows.size != ctx.n_tokens:
-            out["rows"] = ctx.upload(rows)
         max_kv = ctx.kv_bound     # not the lengths themselves: see StepContext.kv_bound
         chunk = ROW_CHUNK
         n_kv_heads = ctx_kv_heads
