@@ -97,7 +97,7 @@ __device__ __forceinline__ void direct_load(unsigned long long base, int bytes, 
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                :
                : "s"(lds_addr), "v"(voffset), "s"(rsrc)
-               : "memory");
+               : "memory", "m0");
 }
 
 // Wait until at most N of this wave's vector memory loads are still in flight, then meet the other waves.
