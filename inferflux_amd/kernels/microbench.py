@@ -27,8 +27,16 @@ GEMM_SHAPES = {"qkv": (4608, 3584), "o": (3584, 3584), "gate_up": (37888, 3584),
 
 
 def _time_us(fn, iters: int) -> float:
-    for i in range(3):
-        fn(i)
+    """Average time of a call, after about 50 ms of the same calls (the card's clocks take that long to settle: a
+    kernel of 0.5 ms timed after three warm-up calls reads 10-20 % slow)."""
+    import time
+    t0 = time.perf_counter()
+    n = 0
+    while n < 3 or (time.perf_counter() - t0 < 0.05 and n < 2000):
+        fn(n)
+        n += 1
+        if n % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
