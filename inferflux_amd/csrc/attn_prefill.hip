@@ -286,9 +286,12 @@ void attn_prefill_kernel(TileArgs a) {
   const unsigned long long k_head = (unsigned long long)(a.k_cache + (size_t)kvh * P * D);
   const unsigned long long v_head = (unsigned long long)(a.v_cache + (size_t)kvh * D * P);
   const unsigned long long page_bytes = (unsigned long long)a.nKV * P * D * 2;
-  const int run_at = (16 * my_run) & (P - 1);      // (tiles start at multiples of 64 keys)
-  // Ask for this wave's part of K tile ``kt`` (page ``kpage``) into K slot kt % NS and of V tile ``vt`` into V slot vt % NS.
-  auto issue = [&](int k_slot, int kpage, int v_slot, int vpage) {
+  // where this wave's run of key tile t starts inside its page (tiles start at multiples of 64 keys: with pages of
+  // up to 64 tokens that is the same for every tile, with larger pages it is not)
+  auto run_at_of = [&](int t) { return (j_first + TK * t + 16 * my_run) & (P - 1); };
+  // Ask for this wave's part of key tile t (its run's page ``kpage`` = ``vpage``) into K slot ``k_slot`` and V slot ``v_slot``.
+  auto issue = [&](int t, int k_slot, int kpage, int v_slot, int vpage) {
+    const int run_at = run_at_of(t);
     const unsigned long long kb = k_head + (unsigned long long)max(kpage, 0) * page_bytes + (unsigned)(run_at * D * 2);
     const unsigned long long vb = v_head + (unsigned long long)max(vpage, 0) * page_bytes + (unsigned)(run_at * 2);
     const int kbytes = kpage >= 0 ? 16 * D * 2 : 0, vbytes = vpage >= 0 ? ((D - 1) * P + 16) * 2 : 0;
@@ -308,12 +311,12 @@ void attn_prefill_kernel(TileArgs a) {
   // whole, and everyone is done with tile s - 1), asks for tile s + 1 into the stage that tile s - 1 has left, and
   // computes tile s while those loads are on their way.  Loads are asked for in every step, also for tiles that do
   // not exist (no page: they deliver zeros).  The other workgroup on the compute unit fills the waits.
-  issue(0, page_of(0), 0, page_of(0));
+  issue(0, 0, page_of(0), 0, page_of(0));
   int next_page = page_of(1);
   for (int s = 0; s < n_tiles_k; ++s) {
     wait_loads_and_barrier<0>();
     const int slot = s & 1;
-    issue(slot ^ 1, next_page, slot ^ 1, next_page);
+    issue(s + 1, slot ^ 1, next_page, slot ^ 1, next_page);
     next_page = page_of(s + 2);
     const int j0 = j_first + TK * s;
     if (wave_q >= qlen || j0 > wave_hi || j0 + TK <= wave_lo) continue;   // (a wave without rows only fetches) uniform over the wave; the barrier is at the loop's top

@@ -338,6 +338,9 @@ MFMA_CASES = [c for c in ATTN_CASES if c[4] % 16 == 0 and c[4] <= 128] + [
     ([300, 130], [500, 0], 8, 2, 128, 32, None, 100),
     ([129], [260], 4, 4, 128, 16, 200, None),
     ([260, 17], [3000, 40], 14, 2, 128, 16, None, 1500),
+    # pages larger than a tile of 64 keys: where a tile's keys start inside their page changes from tile to tile
+    ([200, 40], [300, 1000], 4, 2, 128, 128, None, 50),
+    ([150], [700], 6, 2, 128, 256, 500, None),
 ]
 
 
@@ -409,6 +412,53 @@ def test_attention_tiles(case, qt, split_chunk):
         again = torch.zeros(T, nH * d, dtype=BF16, device=DEV)
         ops.attention_tiles(*call[:3], again, *call[4:], **splits, order=torch.from_numpy(order).to(DEV))
         assert torch.equal(again, plain_order)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_attention_tiles_random_cases(seed):
+    """The tile kernels at shapes drawn at random (the first 24: tiles of 128 rows at head size 128, the kernel that
+    loads its tiles straight into LDS; the others: either tiling at head sizes 16-128): several requests of 16-400
+    rows behind pasts of 0-1,500 keys, pages of 16-256, with and without a window, one to eight query heads to a kv
+    head, whole and in key splits, in the engine's workgroup order; against float64."""
+    import random
+    import numpy as np
+    from inferflux_amd.kernels.attention import tile_order
+    rng = random.Random(100 + seed)
+    d, P = 128, rng.choice([16, 16, 32, 64, 128, 256])
+    qt = 2
+    if seed >= 24:
+        d, qt = rng.choice([16, 32, 64, 128]), rng.choice([1, 2])
+    nKV = rng.choice([1, 2, 4])
+    nH = nKV * rng.choice([1, 2, 5, 7, 8])
+    n_req = rng.randint(1, 3)
+    lens_q = [rng.randint(16, rng.choice([40, 150, 400])) for _ in range(n_req)]
+    lens_past = [rng.choice([0, rng.randint(1, 300), rng.randint(300, 1500)]) for _ in range(n_req)]
+    window = rng.choice([None, None, rng.randint(20, 700)])
+    sharp = rng.choice([None, 3, -200])
+    (q, kc, vc, row_req, positions, table), want, info = paged_case(300 + seed, lens_q, lens_past, nH, nKV, d, P, BF16, window, sharp=sharp)
+    T = q.shape[0]
+    q_len = torch.tensor(info["q_lens"], dtype=torch.int32)
+    q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
+    rows = ops.attention_tile_rows(d, qt)
+    tiles = [(r, q0) for r, n in enumerate(info["q_lens"]) for q0 in range(0, n, rows)]
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    first = np.asarray([info["kv_lens"][r] - info["q_lens"][r] + q0 for r, q0 in tiles])
+    last = np.asarray([min(f + rows, info["kv_lens"][r]) - 1 for f, (r, _) in zip(first, tiles)])
+    for chunk in (0, rng.choice([64, 128, 320, 512])):
+        splits = {}
+        n_splits = 1
+        if chunk:
+            n_splits = -(-max(info["kv_lens"]) // chunk)
+            splits = dict(chunk=chunk, max_splits=n_splits, rows=torch.arange(T, dtype=torch.int32, device=DEV), row_req=row_req,
+                          positions=positions)
+        order = torch.from_numpy(tile_order(first, last, nH, window, n_splits, chunk)).to(DEV)
+        out = torch.zeros(T, nH * d, dtype=BF16, device=DEV)
+        ops.attention_tiles(q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV), q_len.to(DEV),
+                            dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt, order=order, **splits)
+        out = out.cpu().double()
+        assert torch.isfinite(out).all()
+        assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), (seed, chunk, d, qt, lens_q, lens_past, nH, nKV, P, window,
+                                                                 float((out - want).abs().max()))
 
 
 def test_attention_tiles_refuses_splits_it_cannot_merge():
