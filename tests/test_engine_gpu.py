@@ -560,9 +560,9 @@ def test_toy_position_encoding_and_routed_feed_forward(tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("page_size", [32, 64, 128])
 def test_other_page_sizes(page_size, dtype, sharp_folders):
-    """Pages of 32 and 64 tokens (trace_run's rounding unit): mixed steps over a pool that is used again."""
+    """Pages of 32, 64 (trace_run's rounding unit) and 128 tokens: mixed steps over a pool that is used again."""
     import traces
     folder = sharp_folders["C", dtype]
     seqs = {f"r{i}": seeded_ids(500 + i, n, 777) for i, n in enumerate([70, 130, 45, 200, 64])}

@@ -177,11 +177,12 @@ def test_one_layer_of_each_family_shape_against_the_plain_model(name, tmp_path):
         torch.cuda.empty_cache()
 
 
-def test_portions_behind_long_pasts_at_the_7b_layer_shape(monkeypatch):
+@pytest.mark.parametrize("page_size", [16, 128])
+def test_portions_behind_long_pasts_at_the_7b_layer_shape(page_size, monkeypatch):
     """A sequence of 3,000 tokens through one layer of the 7B shape in portions whose pasts grow to 2,364 keys: the
     tile kernels then run with tiles of 64 and of 128 rows, their keys whole and in splits of several lengths, their
     workgroups in the balanced order.  Every cutting stays as close to the float32 engine (run whole)
-    as the uncut bfloat16 run does."""
+    as the uncut bfloat16 run does.  Pages of 16 tokens and of 128 (larger than a tile of 64 keys)."""
     from inferflux_amd.config import config_from_dict
     from inferflux_amd.engine.context import StepEntry
     from inferflux_amd.engine.model import Model
@@ -197,7 +198,8 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(monkeypatch):
     monkeypatch.setattr(attention, "choose_tiling", lambda *a, **k: (tilings.add(real(*a, **k)), real(*a, **k))[1])
 
     def run(dtype, cuts):
-        runner = ModelRunner(Model(cfg).init_random(21, dtype, torch.device("cuda", 0)), num_pages=N // 16 + 2, max_requests=2)
+        runner = ModelRunner(Model(cfg).init_random(21, dtype, torch.device("cuda", 0)), num_pages=N // page_size + 2,
+                             page_size=page_size, max_requests=2)
         runner.add_request("a")
         rows, pos = {}, 0
         for n in cuts:
@@ -206,7 +208,7 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(monkeypatch):
             rows.update({pos + w: logits[i] for i, w in enumerate(want)})
             pos += n
         runner.free_request("a")
-        assert runner.manager.free_pages() == [N // 16 + 2]
+        assert runner.manager.free_pages() == [N // page_size + 2]
         return torch.stack([rows[p] for p in wanted])
 
     ref = run(torch.float32, [N])

@@ -363,6 +363,37 @@ def test_attention_rows(case, chunk):
     assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_attention_rows_random_cases(seed):
+    """The row kernel and its merge at shapes drawn at random: one to five requests of 1-15 rows behind pasts of
+    0-2,500 keys, head sizes 16-128, pages of 16-256, with and without a window, 1-20 query heads to a kv head,
+    splits of 32-1,024 keys, all rows or a subset; against float64."""
+    import random
+    rng = random.Random(500 + seed)
+    d = rng.choice([16, 32, 64, 128])
+    P = rng.choice([16, 16, 32, 64, 128, 256])
+    nKV = rng.choice([1, 2, 3])
+    nH = nKV * rng.choice([1, 2, 5, 7, 8, 20])
+    n_req = rng.randint(1, 5)
+    lens_q = [rng.randint(1, 15) for _ in range(n_req)]
+    lens_past = [rng.choice([0, rng.randint(1, 200), rng.randint(200, 2500)]) for _ in range(n_req)]
+    window = rng.choice([None, None, rng.randint(5, 900)])
+    chunk = rng.choice([32, 64, 128, 256, 1024])
+    (q, kc, vc, row_req, positions, table), want, _ = paged_case(600 + seed, lens_q, lens_past, nH, nKV, d, P, BF16, window,
+                                                                 sharp=rng.choice([None, 2, -50]))
+    T = q.shape[0]
+    rows = None
+    if rng.random() < 0.4 and T > 1:
+        rows = torch.tensor(sorted(rng.sample(range(T), rng.randint(1, T - 1))), dtype=torch.int32, device=DEV)
+    out = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), rows=rows, chunk=chunk).cpu().double()
+    sel = list(range(T)) if rows is None else rows.cpu().tolist()
+    assert torch.isfinite(out).all()
+    assert torch.allclose(out[sel], want[sel], rtol=1e-2, atol=1e-2), (seed, d, P, nH, nKV, lens_q, lens_past, window, chunk,
+                                                                      float((out[sel] - want[sel]).abs().max()))
+    rest = [i for i in range(T) if i not in sel]
+    assert torch.all(out[rest] == 0)
+
+
 def test_attention_rows_subset_leaves_other_rows_alone():
     (q, kc, vc, row_req, positions, table), want, _ = paged_case(8, [5, 1, 3], [10, 99, 40], 6, 2, 32, 16, BF16)
     rows = torch.tensor([5, 0, 8], dtype=torch.int32, device=DEV)
