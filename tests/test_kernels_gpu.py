@@ -116,12 +116,13 @@ def test_rope_append(dtype, style, rot, bias):
 
 @pytest.mark.parametrize("d,nH,nKV", [(16, 3, 1), (32, 4, 2), (128, 7, 1)])
 @pytest.mark.parametrize("bias", [True, False])
-def test_rope_append_in_pieces(d, nH, nKV, bias):
+@pytest.mark.parametrize("P", [16, 32, 128])
+def test_rope_append_in_pieces(d, nH, nKV, bias, P):
     """bfloat16, split-half over the whole head, head size a multiple of 16: the kernel's 16-byte path.  Slots:
     an aligned run of 16 (written as pieces of the transposed page), a run that starts at an odd offset, scattered
     ones, one token without a slot."""
     g = gen(31)
-    T, P, pages, theta = 133, 16, 16, 1e4
+    T, pages, theta = 133, 256 // P, 1e4
     width = (nH + 2 * nKV) * d
     qkv = torch.randn(T, width, generator=g).to(BF16)
     b = (0.5 * torch.randn(width, generator=g)).to(BF16) if bias else None
@@ -627,11 +628,12 @@ def test_tiled_copy_in_another_row_tile_order():
 @pytest.mark.parametrize("M", [1, 5, 16])
 @pytest.mark.parametrize("d,nH,nKV,K", [(32, 3, 1, 72), (128, 7, 1, 264), (64, 4, 2, 128)])
 @pytest.mark.parametrize("bias", [True, False])
-def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, nKV, K, bias):
+@pytest.mark.parametrize("P_", [16, 64, 128])
+def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, nKV, K, bias, P_):
     """The fused kernel against the product followed by the rotary + append kernel (itself checked against the
     plain formulas above): same q, same cache, nothing else touched; and queries only."""
     g = gen(21)
-    P_, pages, theta = 16, 5, 1e4
+    pages, theta = 5, 1e4
     heads = nH + 2 * nKV
     w = (torch.randn(heads * d, K, generator=g) / math.sqrt(K)).to(BF16).to(DEV)
     b = (0.5 * torch.randn(heads * d, generator=g)).to(BF16).to(DEV) if bias else None
