@@ -11,7 +11,7 @@ slot, zero-filled, and clears a slot when it is reused
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 

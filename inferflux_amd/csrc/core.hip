@@ -563,24 +563,3 @@ extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, in
   IFX_LAUNCH_CHECK();
 }
 
-// ---------------------------------------------------------------------------------------
-// out = float(in) or bf16(in), elementwise: the only cast the engine needs outside a kernel's
-// own epilogue (a bf16 activation in front of a matrix that the file stores in 32-bit).
-template <typename TI, typename TO>
-__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
-  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx < n) out[idx] = from_f<TO>(to_f(in[idx]));
-}
-
-extern "C" int ifx_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n, void* stream) {
-  IFX_REQUIRE(n >= 0, "cast: bad size");
-  if (n == 0) return 0;
-  const unsigned blocks = (unsigned)((n + 255) / 256);
-  hipStream_t s = (hipStream_t)stream;
-  if (in_dtype == DT_F32 && out_dtype == DT_BF16)
-    hipLaunchKernelGGL((cast_kernel<float, bf16_t>), dim3(blocks), dim3(256), 0, s, (const float*)in, (bf16_t*)out, (size_t)n);
-  else if (in_dtype == DT_BF16 && out_dtype == DT_F32)
-    hipLaunchKernelGGL((cast_kernel<bf16_t, float>), dim3(blocks), dim3(256), 0, s, (const bf16_t*)in, (float*)out, (size_t)n);
-  else IFX_FAIL("cast: unsupported %d -> %d", in_dtype, out_dtype);
-  IFX_LAUNCH_CHECK();
-}

@@ -13,8 +13,6 @@ import dataclasses
 import time
 from typing import Callable, Dict, Hashable, List, Optional, Sequence
 
-import torch
-
 from .. import log
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler, SamplingState

@@ -14,7 +14,7 @@ raises before it touches the cache.
 from __future__ import annotations
 
 import os
-from typing import Hashable, List, Optional, Sequence
+from typing import Hashable, Optional, Sequence
 
 import torch
 

@@ -34,7 +34,7 @@ from __future__ import annotations
 import collections
 import dataclasses
 import time
-from typing import Callable, Deque, Dict, Hashable, List, Optional, Sequence
+from typing import Callable, Deque, Hashable, List, Optional, Sequence
 
 from ..cache.manager import CacheManager, OutOfPages
 

@@ -216,16 +216,6 @@ def swiglu(gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     return out
 
 
-def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    if x.dtype == dtype:
-        return x
-    _check(x, "x")
-    out = torch.empty(x.shape, dtype=dtype, device=x.device)
-    _call(load_module("core"), "ifx_cast", (P, I, P, I, LL, P),
-          x.data_ptr(), _dt(x), out.data_ptr(), _DT[dtype], x.numel(), _stream())
-    return out
-
-
 # ----------------------------------------------------------------------------------------
 def gemm_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:

@@ -39,7 +39,7 @@ optional for every part; one that declares nothing is run as above.
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Callable, Dict, Mapping, Optional
+from typing import Callable, Dict, Mapping, Optional
 
 import torch
 
