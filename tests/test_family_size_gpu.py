@@ -1,7 +1,7 @@
 """The kernels at the sizes of the model family.  First two layers of the Qwen2.5-7B shape (hidden 3584, 28 query
 heads on 4 kv heads of 128, feed-forward 18944, vocabulary 152064): the bfloat16 engine against the float32 engine
 on the same weights under several cuttings, and the float32 engine bit-equal to itself.  Then one layer at each of
-the 7B, 3B, 14B, 0.5B and 1.5B shapes, written as a folder by the test itself, against the plain model in float64
+the 7B, 3B, 14B, 0.5B, 1.5B, 32B and 72B shapes, written as a folder by the test itself, against the plain model in float64
 on the CPU, in both precisions and three cuttings."""
 import pytest
 import torch
@@ -88,14 +88,21 @@ FAMILY = {
                  rms_norm_eps=1e-6, head_dim=64),
     "1.5B": dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960, vocab_size=151936,
                  rms_norm_eps=1e-6),
+    # the large members: feed-forward widths of 27,648 and 29,568 (= 2^7 x 231), a width of 8,192, 64 query heads
+    "32B": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=27648, vocab_size=152064,
+                rms_norm_eps=1e-5),
+    "72B": dict(hidden_size=8192, num_attention_heads=64, num_key_value_heads=8, intermediate_size=29568, vocab_size=152064,
+                rms_norm_eps=1e-5),
 }
 N_TOKENS = 130
 # Largest difference to the plain model's (float64) logits over the largest logit.  Measured: float32 7.0e-6 / 4.7e-6 /
 # 1.04e-5 at the 7B / 3B / 14B shapes, the same under every cutting (sums of up to 18,944 products in float32);
 # bfloat16 1.72e-2 / 1.38e-2 / 2.08e-2 whole and by single rows, 1.32e-2 / 1.09e-2 / 1.54e-2 in portions of 17; at the 0.5B and
-# 1.5B shapes float32 2.5e-6 / 3.8e-6 and bfloat16 8.9e-3 / 1.32e-2.
+# 1.5B shapes float32 2.5e-6 / 3.8e-6 and bfloat16 8.9e-3 / 1.32e-2; at the 32B and 72B shapes float32 1.21e-5 / 1.38e-5
+# and bfloat16 2.06e-2 / 2.32e-2.
 # The bounds are those figures and half as much again (float32: the tiny configurations' 2e-5).
-FAMILY_TOL = {"float32": 2e-5, "bfloat16": {"7B": 2.6e-2, "3B": 2.1e-2, "14B": 3.1e-2, "0.5B": 1.35e-2, "1.5B": 2.0e-2}}
+FAMILY_TOL = {"float32": 2e-5, "bfloat16": {"7B": 2.6e-2, "3B": 2.1e-2, "14B": 3.1e-2, "0.5B": 1.35e-2, "1.5B": 2.0e-2,
+                                             "32B": 3.1e-2, "72B": 3.5e-2}}
 
 
 def _write_family_folder(folder, name):
