@@ -35,6 +35,12 @@ SHAPE_05B = dict(SHAPE_7B, vocab_size=151936, hidden_size=896, num_hidden_layers
                  num_key_value_heads=2, head_dim=64, intermediate_size=4864, tie_word_embeddings=True)
 SHAPE_15B = dict(SHAPE_7B, vocab_size=151936, hidden_size=1536, num_hidden_layers=28, num_attention_heads=12,
                  num_key_value_heads=2, intermediate_size=8960, tie_word_embeddings=True)
+# the family's large members (the 72B shape's weights and their copy for small batches do not fit one card together:
+# run it with --layers or --no-decode-weight-copy)
+SHAPE_32B = dict(SHAPE_7B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=40, num_key_value_heads=8,
+                 intermediate_size=27648, rms_norm_eps=1e-5)
+SHAPE_72B = dict(SHAPE_7B, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8,
+                 intermediate_size=29568, rms_norm_eps=1e-5)
 WORKLOADS = {
     "mixed3b": dict(shape=SHAPE_3B, name="Qwen2.5-3B shape", requests=64, prompt=(128, 2048), new=256, chunk=512),
     "long14b": dict(shape=SHAPE_14B, name="Qwen2.5-14B shape", requests=32, prompt=(8192, 8192), new=512, chunk=2048),
@@ -67,7 +73,7 @@ def main() -> int:
                     help="measure what the card gives (a 2 GB streaming read, an 8192^3 bf16 library product) once and "
                          "report every share against it beside the data sheet's peak")
     ap.add_argument("--context", type=int, default=DECODE_KV_START, help="tokens each request holds when the timed decode steps start")
-    ap.add_argument("--shape", choices=["7b", "3b", "14b", "1.5b", "0.5b"], default="7b", help="layer sizes of the decode / prefill measurement (the headline is 7b)")
+    ap.add_argument("--shape", choices=["7b", "3b", "14b", "1.5b", "0.5b", "32b", "72b"], default="7b", help="layer sizes of the decode / prefill measurement (the headline is 7b)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT, help="--workload prefill: tokens of the prompt")
     ap.add_argument("--prefill-chunk", type=int, default=0, help="--workload prefill: the prompt in portions of this many tokens, one step each (0: whole)")
     args = ap.parse_args()
@@ -97,7 +103,8 @@ def main() -> int:
     ops.decode_weight_copy = not args.no_decode_weight_copy
     if args.workload in WORKLOADS:
         return run_workload(args, WORKLOADS[args.workload])
-    shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B, "1.5b": SHAPE_15B, "0.5b": SHAPE_05B}[args.shape])
+    shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B, "1.5b": SHAPE_15B, "0.5b": SHAPE_05B, "32b": SHAPE_32B,
+                  "72b": SHAPE_72B}[args.shape])
     shape_name = f"Qwen2.5-{args.shape.upper()} shape"
     layers_full = shape["num_hidden_layers"]
     if args.layers:
