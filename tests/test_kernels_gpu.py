@@ -809,6 +809,37 @@ def test_linear_picks_by_weight_type_and_rows():
         assert mixed.dtype == BF16 and torch.allclose(mixed.cpu().double(), x.bfloat16().double() @ w.double().t(), rtol=1e-2, atol=0.1)
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_linear_random_shapes(seed):
+    """``linear`` and ``linear_swiglu`` at shapes drawn at random: 1-90 rows (the streaming kernels up to 64, the
+    library beyond), 1-6,000 weight rows, K a multiple of 8 up to 4,800, with and without the streamed copy in whatever
+    tile height ``prepare_linear`` picks for the weight, partial sums kept or added, bf16 or float out; against
+    float64."""
+    import random
+    rng = random.Random(500 + seed)
+    M = rng.choice([1, rng.randint(2, 16), rng.randint(17, 64), rng.randint(65, 90)])
+    N = rng.choice([rng.randint(1, 40), rng.randint(41, 700), rng.randint(701, 6000)])
+    K = 8 * rng.choice([rng.randint(1, 16), rng.randint(17, 150), rng.randint(151, 600)])
+    out_dtype = rng.choice([BF16, F32])
+    g = gen(600 + seed)
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = (torch.randn(N, K, generator=g) * 0.3).to(BF16)
+    want = x.double() @ w.double().t()
+    t = dict(rtol=1e-4, atol=3e-3 * max(1.0, K / 1000)) if out_dtype == F32 else dict(rtol=1e-2, atol=0.1 * max(1.0, (K / 1000) ** 0.5))
+    weight = ops.prepare_linear(w.to(DEV)) if rng.random() < 0.75 else w.to(DEV)
+    got = ops.linear(x.to(DEV), weight, out_dtype, keep_slices=rng.random() < 0.5)
+    if isinstance(got, ops.SliceSums):
+        got = got.sum()
+    got = got.cpu().double()
+    assert got.shape == (M, N) and torch.allclose(got, want, **t), (M, N, K, out_dtype, float((got - want).abs().max()))
+    if N % 2 == 0:
+        act = ops.linear_swiglu(x.to(DEV), weight).cpu().double()
+        gt, up = want[:, 0::2], want[:, 1::2]
+        ref = gt / (1 + torch.exp(-gt)) * up
+        assert act.shape == (M, N // 2) and torch.allclose(act, ref, rtol=2e-2, atol=2e-2 * max(1.0, float(ref.abs().max()) / 8)), \
+            (M, N, K, float((act - ref).abs().max()))
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 40, 100])
 def test_linear_swiglu_pairs(M):
     g = gen(14)
@@ -877,6 +908,39 @@ def test_row_factors_are_applied_by_the_product_that_reads_the_rows(M, copy):
     gt, up = (rows @ w2[0::2].double().t()) * factor, (rows @ w2[1::2].double().t()) * factor
     act = ops.linear_swiglu(scaled, lw2).cpu().double()
     assert torch.allclose(act, gt / (1 + torch.exp(-gt)) * up, **tol(BF16))
+
+
+@pytest.mark.parametrize("seed", range(25))
+def test_stream_add_and_row_factors_random_shapes(seed):
+    """A product added into the stream with the next norm prepared, then the products that take the rows with their
+    factors, at widths, row counts and tile heights drawn at random; against float64."""
+    import random
+    rng = random.Random(700 + seed)
+    M = rng.randint(1, 16)
+    H = 8 * rng.choice([rng.randint(1, 12), rng.randint(13, 120), rng.randint(121, 450)])
+    K = 8 * rng.choice([rng.randint(1, 20), rng.randint(21, 300)])
+    I = 2 * rng.choice([rng.randint(1, 30), rng.randint(31, 1200)])
+    copy = rng.choice([False, True, 14, 10, 8])
+    eps = rng.choice([1e-6, 1e-3])
+    x, w, stream, nw, lw = _stream_case(M, H, K, 800 + seed, copy)
+    s = stream.to(DEV)
+    scaled = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), eps)
+    want = stream.double() + x.double() @ w.double().t()
+    assert torch.allclose(s.cpu().double(), want, rtol=1e-5, atol=1e-4 * max(1.0, K / 500)), (M, H, K, copy)
+    rows = scaled.rows.cpu().double()
+    factor = torch.rsqrt((s.cpu().double() ** 2).mean(-1, keepdim=True) + eps)
+    assert torch.allclose(rows * factor, pm.rms_norm(s.cpu().double(), nw.double(), eps), **tol(BF16)), (M, H, K, copy)
+    g = gen(900 + seed)
+    w2 = (torch.randn(I, H, generator=g) * 0.2).to(BF16)
+    lw2 = ops.LinearWeight(w2.to(DEV), ops.tile_weights(w2.to(DEV), tile_rows=lw.tile_rows) if copy else None, None, lw.tile_rows)
+    ref = (rows @ w2.double().t()) * factor
+    big = max(1.0, float(ref.abs().max()))
+    got = ops.linear(scaled, lw2, torch.float32).cpu().double()
+    assert torch.allclose(got, ref, rtol=1e-4, atol=1e-4 * big), (M, H, K, I, copy, float((got - ref).abs().max()))
+    gt, up = ref[:, 0::2], ref[:, 1::2]
+    act = ops.linear_swiglu(scaled, lw2).cpu().double()
+    want_act = gt / (1 + torch.exp(-gt)) * up
+    assert torch.allclose(act, want_act, rtol=8e-3, atol=1e-3 * max(1.0, float(want_act.abs().max()))), (M, H, K, I, copy)
 
 
 def test_row_factors_in_the_fused_qkv_product():
