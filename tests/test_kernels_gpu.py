@@ -61,6 +61,42 @@ def test_add_rmsnorm(dtype, H, wdtype):
     assert torch.allclose(out3.cpu().double(), want[rows.long()], **tol(dtype))
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_add_rmsnorm_random_shapes(seed):
+    """Residual add and norm at widths of 1-9,000 (the vector form takes multiples of 8, the plain form the others),
+    1-300 rows, a delta that is bf16, float, partial sums of 2-9 slices, or absent, and a gathered subset of rows;
+    against float64."""
+    import random
+    rng = random.Random(1100 + seed)
+    T = rng.choice([1, rng.randint(2, 20), rng.randint(21, 300)])
+    H = rng.choice([rng.randint(1, 64), 8 * rng.randint(8, 600), rng.randint(65, 9000), 8 * rng.randint(601, 1100)])
+    out_dtype, wdtype = rng.choice([F32, BF16]), rng.choice([F32, BF16])
+    kind = rng.choice(["bf16", "f32", "slices", "slices", "none"])
+    eps = rng.choice([1e-6, 1e-5, 1e-2])
+    g = gen(1200 + seed)
+    res = torch.randn(T, H, generator=g) * 3
+    w = (1 + 0.3 * torch.randn(H, generator=g)).to(wdtype)
+    delta, want_res = None, res.double()
+    if kind == "slices":
+        parts = torch.randn(rng.randint(2, 9), T, H, generator=g)
+        delta = ops.SliceSums(parts.to(DEV), out_dtype)
+        want_res = res.double() + parts.double().sum(0)
+    elif kind != "none":
+        d = torch.randn(T, H, generator=g).to(BF16 if kind == "bf16" else F32)
+        delta, want_res = d.to(DEV), res.double() + d.double()
+    want = pm.rms_norm(want_res, w.double(), eps)
+    r = res.to(DEV)
+    out = ops.add_rmsnorm(r, delta, w.to(DEV), eps, out_dtype)
+    case = (T, H, kind, out_dtype, wdtype)
+    assert torch.allclose(r.cpu().double(), want_res, rtol=1e-6, atol=1e-5), case          # the stream took the delta
+    assert torch.allclose(out.cpu().double(), want, **tol(out_dtype)), case
+    rows = torch.tensor([rng.randrange(T) for _ in range(rng.randint(1, 5))], dtype=torch.int32)
+    r2 = res.to(DEV)
+    out2 = ops.add_rmsnorm(r2, delta, w.to(DEV), eps, out_dtype, rows.to(DEV))             # gathered rows: stream untouched
+    assert torch.equal(r2.cpu(), res), case
+    assert torch.allclose(out2.cpu().double(), want[rows.long()], **tol(out_dtype)), case
+
+
 def test_rmsnorm_eps_is_inside_the_root():
     x = torch.full((1, 64), 1e-4)
     w = torch.ones(64)
