@@ -344,6 +344,36 @@ def test_sample_matches_the_plain_rule(V):
         assert lo - 1e-4 <= float(u[r]) <= hi + 1e-4, (r, got[r], lo, float(u[r]), hi)
 
 
+@pytest.mark.parametrize("seed", range(20))
+def test_sample_random_vocabularies_and_filters(seed):
+    """The draw against the plain rule at vocabularies of 2-200,000 (no multiple of anything), 1-40 rows, and
+    temperatures, top-k, top-p and min-p drawn at random, several filters at once; the greedy rows beside them."""
+    import random
+    rng = random.Random(1300 + seed)
+    V = rng.choice([rng.randint(2, 70), rng.randint(71, 5000), rng.randint(5001, 200000)])
+    R = rng.randint(1, 40)
+    g = gen(1400 + seed)
+    logits = rng.choice([1.0, 3.0, 8.0]) * torch.randn(R, V, generator=g)
+    temps = torch.tensor([rng.choice([0.0, 0.3, 0.7, 1.0, 1.5, 2.5]) for _ in range(R)])
+    top_k = torch.tensor([rng.choice([0, 0, 1, 2, 5, 40, 1000]) for _ in range(R)], dtype=torch.int32)
+    top_p = torch.tensor([rng.choice([1.0, 1.0, 0.999, 0.9, 0.5, 0.1]) for _ in range(R)])
+    min_p = torch.tensor([rng.choice([0.0, 0.0, 0.01, 0.1, 0.5]) for _ in range(R)])
+    u = torch.rand(R, generator=g)
+    got = ops.sample(logits.to(DEV), temps.to(DEV), top_k.to(DEV), top_p.to(DEV), min_p.to(DEV), u.to(DEV)).cpu().tolist()
+    assert ops.argmax(logits.to(DEV)).cpu().tolist() == logits.argmax(-1).tolist()
+    for r in range(R):
+        case = (seed, V, r, float(temps[r]), int(top_k[r]), float(top_p[r]), float(min_p[r]))
+        assert 0 <= got[r] < V, case
+        if float(temps[r]) == 0.0 or int(top_k[r]) == 1:
+            assert got[r] == int(logits[r].argmax()), case
+            continue
+        w = pm.filtered_probs(logits[r], float(temps[r]), int(top_k[r]), float(top_p[r]), float(min_p[r]))
+        assert w[got[r]] > 0, (case, "a filtered-out token was drawn")
+        cum = torch.cumsum(w, 0) / w.sum()
+        lo = float(cum[got[r] - 1]) if got[r] > 0 else 0.0
+        assert lo - 1e-4 <= float(u[r]) <= float(cum[got[r]]) + 1e-4, (case, got[r], lo, float(u[r]), float(cum[got[r]]))
+
+
 def test_sample_histogram_follows_the_probabilities():
     g = gen(10)
     V, N = 50, 4000
