@@ -184,6 +184,69 @@ def test_rope_append_in_pieces(d, nH, nKV, bias, P):
     assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P, -1)[~written] == 0)
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_rope_append_random_shapes(seed):
+    """Bias, rotation and cache write at shapes drawn at random: head sizes of 2-256 (the 16-byte path takes bfloat16
+    heads of a multiple of 16 rotated whole; the plain path the rest), 1-40 query heads on 1-8 kv heads, either rotation
+    style over the whole head or a part of it, pages of 16-128, q/k/v given whole or as partial sums, slots scattered
+    with some rows unwritten; against float64."""
+    import random
+    rng = random.Random(1500 + seed)
+    dtype = rng.choice([F32, BF16, BF16])
+    d = rng.choice([16 * rng.randint(1, 16), 16 * rng.randint(1, 8), 2 * rng.randint(1, 40)])
+    nKV = rng.choice([1, 2, 3, 4, 8])
+    nH = nKV * rng.choice([1, 2, 5, 7])
+    style = rng.choice(["split_half", "split_half", "consecutive"])
+    rd = rng.choice([d, d, 2 * rng.randint(1, d // 2)])
+    bias = rng.random() < 0.6
+    P = rng.choice([16, 32, 64, 128])
+    T = rng.choice([1, rng.randint(2, 16), rng.randint(17, 150)])
+    pages, theta = -(-(T + 40) // P) + 1, rng.choice([1e4, 1e6])
+    g = gen(1600 + seed)
+    width = (nH + 2 * nKV) * d
+    qkv = torch.randn(T, width, generator=g).to(dtype)
+    b = (0.5 * torch.randn(width, generator=g)).to(dtype) if bias else None
+    positions = torch.randint(0, 40000, (T,), generator=g).to(torch.int32)
+    slots = torch.randperm(pages * P, generator=g)[:T].to(torch.int32)
+    if T > 3:
+        slots[rng.randrange(T)] = -1
+    run = min(T, 16)
+    if rng.random() < 0.5 and pages * P >= 32:                 # an aligned run of 16 slots: written as pieces of the page
+        slots[:run] = torch.arange(16, 16 + run, dtype=torch.int32)
+        taken = set(slots[:run].tolist())
+        rest = [x for x in torch.randperm(pages * P, generator=g).tolist() if x not in taken][: T - run]
+        slots[run:] = torch.tensor(rest, dtype=torch.int32)
+    kc = torch.zeros(pages, nKV, P, d, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, nKV, d, P, dtype=dtype, device=DEV)
+    inv_freq = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64), 2.0 * torch.arange(rd // 2, dtype=torch.float64) / rd)).float()
+    code = {"split_half": ops.ROPE_SPLIT_HALF, "consecutive": ops.ROPE_CONSECUTIVE}[style]
+    cs, sn = ops.rope_table(positions.to(DEV), inv_freq.to(DEV))
+    given = qkv.to(DEV)
+    want_in = qkv.double()
+    if rng.random() < 0.4:                                     # partial sums of a product cut along K
+        parts = torch.randn(rng.randint(2, 8), T, width, generator=g)
+        given, want_in = ops.SliceSums(parts.to(DEV), dtype), parts.double().sum(0)
+    q = ops.rope_append(given, b.to(DEV) if bias else None, slots.to(DEV), cs, sn, code, rd, nH, nKV, d, kc, vc, P)
+    x = want_in + (b.double() if bias else 0)
+    xq, xk, xv = x[:, : nH * d].view(T, nH, d), x[:, nH * d: (nH + nKV) * d].view(T, nKV, d), x[:, (nH + nKV) * d:].view(T, nKV, d)
+
+    def rope(t):
+        fn = pm.rope_split_half if style == "split_half" else pm.rope_consecutive
+        return torch.cat([fn(t[..., :rd], positions.tolist(), theta), t[..., rd:]], dim=-1)
+
+    case = (seed, dtype, d, nH, nKV, style, rd, bias, P, T, isinstance(given, ops.SliceSums))
+    # angles are formed in float (position * rounded frequency, positions up to 40,000): allow that on top of the rounding
+    t = dict(rtol=tol(dtype)["rtol"], atol=tol(dtype)["atol"] + 2e-2)
+    assert torch.allclose(q.cpu().double(), rope(xq), **t), case
+    live = slots >= 0
+    k_got, v_got = cache_rows(kc.cpu(), vc.cpu(), slots[live], P)
+    assert torch.allclose(k_got.double(), rope(xk)[live], **t), case
+    assert torch.allclose(v_got.double(), xv[live], **tol(dtype)), case
+    written = torch.zeros(pages * P, dtype=torch.bool); written[slots[live].long()] = True
+    assert torch.all(kc.cpu().permute(0, 2, 1, 3).reshape(pages * P, -1)[~written] == 0), case   # nothing else touched
+    assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P, -1)[~written] == 0), case
+
+
 def test_rope_queries_only():
     g = gen(4)
     T, nH, d = 4, 3, 16
