@@ -360,6 +360,55 @@ def test_attention_plain(dtype, case):
     assert torch.allclose(out, want, **t), float((out - want).abs().max())
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_attention_plain_random_cases(seed):
+    """The plain attention kernel (the 32-bit path's, and the reference beside the matrix-core ones) at shapes drawn at
+    random: head sizes of 1-256, pages of any size from 1 (no power of two), 1-3 requests of 1-60 rows behind pasts of
+    0-400 keys, with and without a window and a planted far key; float32 and bfloat16, against float64."""
+    import random
+    rng = random.Random(1700 + seed)
+    dtype = rng.choice([F32, F32, BF16])
+    d = rng.choice([rng.randint(1, 24), 8 * rng.randint(1, 32), rng.randint(25, 256)])
+    P = rng.choice([1, 3, 16, 24, 50, 64])
+    nKV = rng.choice([1, 2, 3])
+    nH = nKV * rng.choice([1, 2, 4, 7])
+    n_req = rng.randint(1, 3)
+    lens_q = [rng.randint(1, rng.choice([2, 20, 60])) for _ in range(n_req)]
+    lens_past = [rng.choice([0, rng.randint(1, 60), rng.randint(61, 400)]) for _ in range(n_req)]
+    window = rng.choice([None, None, rng.randint(1, 200)])
+    sharp = rng.choice([None, 0, 2, -3])
+    (q, kc, vc, row_req, positions, table), want, _ = paged_case(1800 + seed, lens_q, lens_past, nH, nKV, d, P, dtype, window, sharp=sharp)
+    out = ops.attention_plain(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d))
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == F32 else dict(rtol=1e-2, atol=1e-2)
+    assert torch.allclose(out.cpu().double(), want, **t), (seed, dtype, d, P, nH, nKV, lens_q, lens_past, window, sharp,
+                                                            float((out.cpu().double() - want).abs().max()))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_gemm_f32_random_shapes(seed):
+    """The 32-bit product at shapes drawn at random (1-300 rows, 1-3,000 weight rows, any K up to 5,000), float32 or
+    bfloat16 activations, with and without a bias; against float64, and the same row gives the same bits whatever else
+    is in the batch."""
+    import random
+    rng = random.Random(1900 + seed)
+    M = rng.choice([1, rng.randint(2, 20), rng.randint(21, 300)])
+    N = rng.choice([rng.randint(1, 40), rng.randint(41, 3000)])
+    K = rng.choice([rng.randint(1, 70), rng.randint(71, 5000)])
+    adtype = rng.choice([F32, BF16])
+    g = gen(2000 + seed)
+    x = torch.randn(M, K, generator=g).to(adtype)
+    w = torch.randn(N, K, generator=g) * 0.2
+    b = torch.randn(N, generator=g) if rng.random() < 0.5 else None
+    want = x.double() @ w.double().t() + (b.double() if b is not None else 0)
+    got = ops.gemm_f32(x.to(DEV), w.to(DEV), b.to(DEV) if b is not None else None)
+    assert got.dtype == adtype or got.dtype == F32
+    t = dict(rtol=1e-4, atol=2e-5 * max(1.0, K ** 0.5)) if got.dtype == F32 else dict(rtol=1e-2, atol=0.05 * max(1.0, (K / 500) ** 0.5))
+    assert torch.allclose(got.cpu().double(), want, **t), (M, N, K, adtype, float((got.cpu().double() - want).abs().max()))
+    r = rng.randrange(M)
+    alone = ops.gemm_f32(x[r:r + 1].to(DEV), w.to(DEV), b.to(DEV) if b is not None else None)
+    assert torch.equal(alone[0], got[r]), (M, N, K, r)
+
+
 # ---- sampling -------------------------------------------------------------------------------
 def test_argmax_lowest_index_wins_ties():
     l = torch.zeros(3, 1500)
