@@ -847,6 +847,49 @@ def test_qkv_projection_with_rotation_and_cache_write_as_its_epilogue(M, d, nH, 
     assert torch.allclose(qq.float(), q.float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_qkv_random_shapes(seed):
+    """The q/k/v product with bias, rotation and cache write as its epilogue, at shapes drawn at random (1-16 rows,
+    head sizes of 32-256 in steps of 32, 1-40 query heads, K a multiple of 8 up to 4,000, pages of 16-128); against
+    the plain formulas in float64."""
+    import random
+    rng = random.Random(2100 + seed)
+    M = rng.randint(1, 16)
+    d = 32 * rng.choice([1, 2, 2, 3, 4, 4, 8])
+    nKV = rng.choice([1, 2, 4, 8])
+    nH = nKV * rng.choice([1, 2, 5, 7])
+    K = 8 * rng.choice([rng.randint(1, 30), rng.randint(31, 500)])
+    P_ = rng.choice([16, 32, 64, 128])
+    bias = rng.random() < 0.6
+    pages, theta = 3, rng.choice([1e4, 1e6])
+    g = gen(2200 + seed)
+    heads = nH + 2 * nKV
+    w = (torch.randn(heads * d, K, generator=g) / math.sqrt(K)).to(BF16)
+    b = (0.5 * torch.randn(heads * d, generator=g)).to(BF16) if bias else None
+    x = torch.randn(M, K, generator=g).to(BF16)
+    positions = torch.randint(0, 3000, (M,), generator=g).to(torch.int32)
+    slots = torch.randperm(pages * P_, generator=g)[:M].to(torch.int32)
+    if M > 2:
+        slots[rng.randrange(M)] = -1
+    inv_freq = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64), 2.0 * torch.arange(d // 2, dtype=torch.float64) / d)).float()
+    cs, sn = ops.rope_table(positions.to(DEV), inv_freq.to(DEV))
+    lw = ops.prepare_linear(w.to(DEV), torch.tensor(ops.pair_tile_order(heads, d), dtype=torch.int32, device=DEV))
+    kc, vc = torch.zeros(pages, nKV, P_, d, dtype=BF16, device=DEV), torch.zeros(pages, nKV, d, P_, dtype=BF16, device=DEV)
+    q = ops.qkv_rope_append(x.to(DEV), lw, b.to(DEV) if bias else None, slots.to(DEV), cs, sn, nH, nKV, d, kc, vc, P_)
+    qkv = x.double() @ w.double().t() + (b.double() if bias else 0)
+    xq, xk, xv = qkv[:, : nH * d].view(M, nH, d), qkv[:, nH * d: (nH + nKV) * d].view(M, nKV, d), qkv[:, (nH + nKV) * d:].view(M, nKV, d)
+    case = (seed, M, d, nH, nKV, K, P_, bias)
+    t = dict(rtol=1e-2, atol=1e-2)
+    assert torch.allclose(q.cpu().double(), pm.rope_split_half(xq, positions.tolist(), theta), **t), case
+    live = slots >= 0
+    k_got, v_got = cache_rows(kc.cpu(), vc.cpu(), slots[live], P_)
+    assert torch.allclose(k_got.double(), pm.rope_split_half(xk, positions.tolist(), theta)[live], **t), case
+    assert torch.allclose(v_got.double(), xv[live], **t), case
+    written = torch.zeros(pages * P_, dtype=torch.bool); written[slots[live].long()] = True
+    assert torch.all(kc.cpu().permute(0, 2, 1, 3).reshape(pages * P_, -1)[~written] == 0), case   # nothing else touched
+    assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P_, -1)[~written] == 0), case
+
+
 @pytest.mark.parametrize("M", [9, 17, 32, 33, 50, 64])
 @pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136)])
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
