@@ -643,6 +643,59 @@ def test_sizes_that_are_multiples_of_little(name, dtype, tmp_path):
     assert rel_err(torch.cat(got), want) < REL_TOL[dtype]
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Configurations drawn at random (1-3 layers, head sizes of 8-128, 1-3 kv heads with 1-4 query heads each, a
+    width that need not be heads x head size, odd vocabularies, with and without bias, tied head, a window on the
+    upper layers; pages of 16 or 32), each run as a mix of up to four live requests in a pool so small that pages are
+    used again.  float32 against the plain model at the tight bound, and bfloat16 beside float32 at bfloat16's."""
+    import random
+    import traces
+    from conftest import QK_GAIN, sharpen
+    from inferflux_amd.config import config_from_dict
+    from inferflux_amd.weights import write_random_model
+    rng = random.Random(4000 + seed)
+    d = rng.choice([8, 16, 24, 32, 48, 64, 128])
+    nKV = rng.randint(1, 3)
+    nH = nKV * rng.randint(1, 4)
+    window = rng.random() < 0.4
+    layers = rng.randint(1, 3)
+    cfg = dict(model_type="qwen2", architectures=["Qwen2ForCausalLM"], vocab_size=rng.randint(40, 2500),
+               hidden_size=8 * rng.randint(3, 30), num_hidden_layers=layers, num_attention_heads=nH, num_key_value_heads=nKV,
+               head_dim=d, intermediate_size=8 * rng.randint(3, 60), max_position_embeddings=512,
+               rope_theta=rng.choice([1e4, 5e5, 1e6]), rms_norm_eps=rng.choice([1e-6, 1e-5, 3e-6]),
+               tie_word_embeddings=rng.random() < 0.5, attention_bias=rng.random() < 0.6, use_sliding_window=window,
+               sliding_window=rng.randint(5, 60), max_window_layers=rng.randint(0, layers - 1) if window else layers,
+               hidden_act="silu", torch_dtype="bfloat16")
+    page_size = rng.choice([16, 16, 32])
+    raw = str(tmp_path / "raw")
+    write_random_model(raw, config_from_dict(cfg), seed=seed, dtype=torch.bfloat16)
+    seqs = {f"r{i}": seeded_ids(seed * 10 + i, rng.randint(3, 150), cfg["vocab_size"]) for i in range(6)}
+    steps, expected = traces.mixed(seqs, seed=seed)
+    pages = traces.peak_tokens(steps, round_to=page_size) // page_size
+    for dtype in ("float32", "bfloat16"):
+        folder = str(tmp_path / dtype)
+        sharpen(raw, folder, 50 + seed, QK_GAIN[dtype] * min(1.0, (64 / cfg["hidden_size"]) ** 0.5))   # (scores grow with the width)
+        n_pages = pages + (1 if window else 0)
+        runner = load_runner(folder, DT[dtype], num_pages=n_pages, page_size=page_size, max_requests=4)
+        got, want = [], []
+        for st in steps:
+            for e in st["entries"]:
+                if not runner.has_request(e["id"]):
+                    runner.add_request(e["id"])
+            logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+            if st["step"] in expected:
+                got.append(logits.float().cpu())
+                want += [plain_logits(folder, seqs[rid])[p] for rid, p in expected[st["step"]]]
+            for rid in st["end"]:
+                runner.free_request(rid)
+        e = rel_err(torch.cat(got), torch.stack(want))
+        print(f"random configuration {seed} {dtype}: {e:.2e}", flush=True)
+        assert e < REL_TOL[dtype], (seed, dtype, e, cfg, page_size)
+        runner.manager.check()
+        assert runner.manager.free_pages() == [n_pages] * len(runner.manager.groups), (seed, dtype)
+
+
 def test_a_toy_embedding_that_reads_positions_and_a_toy_mixer_with_narrow_values(tmp_path):
     """Two parts from outside the package that need more of the step than the built-in ones: an embedding that adds
     a learned table of absolute positions (it is given the step's context, not just the token ids), and an
