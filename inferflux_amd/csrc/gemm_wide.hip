@@ -1,7 +1,7 @@
-// Weight-streaming matrix product for 17-64 rows:  out[M,N] = x[M,K] * W[N,K]^T from the tiled copy of W
+// Weight-streaming matrix product for 17-128 rows:  out[M,N] = x[M,K] * W[N,K]^T from the tiled copy of W
 // (layout: gemm_bf16.hip), bf16 in, float accumulate on the matrix cores (16x16x32), out bf16 or float.
 //
-// At these sizes the product is still bound by reading W once, but every tile of W now meets two to four
+// At these sizes the product is still bound by reading W once, but every tile of W now meets two to eight
 // tiles of x, and a wave that fetched those from the L2 itself would move more bytes of x than of W.  A
 // workgroup of 8-16 waves therefore owns one tile of 16 weight rows per wave and one slice of K, and the
 // rows of x for the next 128 k-values are copied to LDS once per workgroup (two buffers, one barrier per
@@ -19,6 +19,12 @@
 // j = 4 kt + g of rows 16 mt + col: sixteen consecutive slots per group of 16 lanes, no bank conflict; the
 // shift by j keeps the stores of 16 consecutive pieces of one row apart as well.
 //
+// More than 64 rows (five to eight tiles of x, 170 registers a wave) run as workgroups of exactly 8 waves.  That is
+// worth it where the weight has few rows and K is cut into slices (down, o, q/k/v of the 7B shape at 65-128 rows:
+// 37-50, 15-21 and 16-22 us against the library's 58-66, 30-34 and 30-37); a tall weight such as gate/up would need
+// more than one workgroup of 8 waves per compute unit and is left to the library there (115 against 64 us at 128
+// rows).  The caller decides (ops._small_m_kernel).
+//
 // With more than one slice of K the slices write float partial sums and a second kernel adds them in slice
 // order; the result never depends on timing.
 //
@@ -32,6 +38,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 constexpr int DEPTH = 3;                                           // rounds of W and x on their way
 constexpr int MIN_WAVES = 8, MAX_WAVES = 16;
+constexpr int MAX_ROWS = 128, MANY_ROWS = 64;                     // beyond MANY_ROWS a workgroup has exactly MIN_WAVES waves
 constexpr int WK = 128, WK_TILES = WK / 32, WK_PIECES = WK / 8;   // k-values, k-tiles and 16-byte pieces of a round
 
 __device__ __forceinline__ bf16x8 zero8() {
@@ -44,7 +51,7 @@ __device__ __forceinline__ bf16x8 zero8() {
 // EPI 0: out[m, n] = sum.  EPI 1: the rows of W alternate gate, up, ...: out[m, n / 2] = silu(gate) * up.
 // ``order``: tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
 template <int MT, typename TO, int EPI>
-__global__ __launch_bounds__(MAX_WAVES * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
+__global__ __launch_bounds__((16 * MT > MANY_ROWS ? MIN_WAVES : MAX_WAVES) * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
                                                                      TO* __restrict__ out, float* __restrict__ part, int M,
                                                                      int N, int K, int k_tiles, int rounds_per_slice,
                                                                      const int* __restrict__ order, int tile_rows) {
@@ -170,13 +177,14 @@ extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S
 
 // Waves per workgroup and slices of K for a shape.  ``waves`` / ``slices`` 0: chosen here (about one workgroup
 // for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
-// several workgroups to a unit; then slices of at least four rounds, at most eight); the gate/up epilogue takes
-// one slice.  Returns waves * 256 + slices.
-extern "C" int ifx_wide_gemm_plan(int N, int K, int waves, int slices, int epi, int tile_rows) {
+// several workgroups to a unit; 8 waves for more than 64 rows; then slices of at least four rounds, at most eight);
+// the gate/up epilogue takes one slice.  Returns waves * 256 + slices.
+extern "C" int ifx_wide_gemm_plan(int rows, int N, int K, int waves, int slices, int epi, int tile_rows) {
   if (tile_rows < 8 || tile_rows > 16) tile_rows = 16;
   const int n_tiles = (N + tile_rows - 1) / tile_rows, n_rounds = (K + WK - 1) / WK;
   if (waves <= 0) waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
   waves = waves < MIN_WAVES ? MIN_WAVES : (waves > MAX_WAVES ? MAX_WAVES : waves);
+  if (rows > MANY_ROWS) waves = MIN_WAVES;
   const int groups = (n_tiles + waves - 1) / waves;
   if (epi != 0) slices = 1;
   if (slices <= 0) {
@@ -213,7 +221,7 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
   IFX_LAUNCH_CHECK();
 }
 
-// x [M <= 64, K] times the tiled copy Wt of W [N, K], transposed.  ``waves``, ``slices``: as ifx_wide_gemm_plan
+// x [M <= 128, K] times the tiled copy Wt of W [N, K], transposed.  ``waves``, ``slices``: as ifx_wide_gemm_plan
 // returned them; ``part``: slices * M * N floats when there is more than one slice.
 // epi 1: gate/up rows interleaved in W, out = silu(gate) * up, [M, N / 2] (one slice, no tile order).
 // order: the row-tile order the copy was written with (or null); tile_rows: the rows to a tile it was written with.
@@ -224,7 +232,7 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
   IFX_REQUIRE(out || slices > 1, "wide_gemm: no output");
   IFX_REQUIRE(tile_rows >= 8 && tile_rows <= 16 && tile_rows % 2 == 0 && (tile_rows == 16 || !order),
               "wide_gemm: %d rows to a tile (8 to 16, even; a tile order goes with 16)", tile_rows);
-  IFX_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "wide_gemm: M=%d must be at most 64 (N=%d K=%d)", M, N, K);
+  IFX_REQUIRE(M >= 0 && M <= MAX_ROWS && N > 0 && K > 0, "wide_gemm: M=%d must be at most %d (N=%d K=%d)", M, MAX_ROWS, N, K);
   IFX_REQUIRE(K % 8 == 0, "wide_gemm: K=%d must be a multiple of 8", K);
   IFX_REQUIRE(out_dtype == DT_BF16 || out_dtype == DT_F32, "wide_gemm: unknown out dtype %d", out_dtype);
   IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0 && !order && slices == 1), "wide_gemm: epilogue %d with N=%d, %d slices%s", epi, N,
@@ -232,6 +240,7 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
   const int n_rounds = (K + WK - 1) / WK;
   IFX_REQUIRE(waves >= MIN_WAVES && waves <= MAX_WAVES && slices >= 1 && slices <= n_rounds, "wide_gemm: %d waves (%d-%d), %d slices of %d rounds",
               waves, MIN_WAVES, MAX_WAVES, slices, n_rounds);
+  IFX_REQUIRE(M <= MANY_ROWS || waves == MIN_WAVES, "wide_gemm: %d rows take workgroups of %d waves, not %d", M, MIN_WAVES, waves);
   IFX_REQUIRE(slices == 1 || part, "wide_gemm: %d slices of K need a scratch buffer", slices);
   if (M == 0) return 0;
   const int rps = (n_rounds + slices - 1) / slices;
@@ -241,6 +250,10 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
     case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
     case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
     case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    default: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 4: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 5: return launch_wide<5>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 6: return launch_wide<6>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 7: return launch_wide<7>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    default: return launch_wide<8>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
   }
 }

@@ -234,6 +234,8 @@ def gemm_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
 
 
 SKINNY_MAX_M = 64
+WIDE_MAX_M = 128           # rows the product that shares x through LDS takes at most ...
+WIDE_MANY_ROWS_MAX_N = 16384   # ... beyond 64 of them only for weights of up to this many rows (see _small_m_kernel)
 
 
 def enable_library_gemm_tuning(max_ms_per_shape: int = 300, filename: Optional[str] = None) -> None:
@@ -522,23 +524,24 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
 
 def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
               slices: int = 0, swiglu_pairs: bool = False, keep_slices: bool = False):
-    """bfloat16 x [M <= 64, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
-    of a workgroup: the product for 17-64 rows.  ``waves`` (8-16 per workgroup, one tile of 16 weight rows each)
-    and ``slices`` of K (added in a fixed order): 0 lets the kernel choose.  With ``keep_slices`` a product of
+    """bfloat16 x [M <= 128, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
+    of a workgroup: the product for 17-64 rows, and for 65-128 rows of weights with few rows.  ``waves`` (8-16 per
+    workgroup, 8 beyond 64 rows; one tile of weight rows each) and ``slices`` of K (added in a fixed order): 0 lets the
+    kernel choose.  With ``keep_slices`` a product of
     several slices comes back as ``SliceSums``."""
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     N = weight.rows.shape[0]
     if weight.tiled is None or weight.rows.shape[1] != K or weight.rows.dtype != torch.bfloat16:
         raise KernelError(f"wide_gemm: needs the tiled copy of a bfloat16 [N, {K}] weight")
-    if M > SKINNY_MAX_M or K % 8:
-        raise KernelError(f"wide_gemm: M={M} must be <= {SKINNY_MAX_M} and K={K} a multiple of 8")
+    if M > WIDE_MAX_M or K % 8:
+        raise KernelError(f"wide_gemm: M={M} must be <= {WIDE_MAX_M} and K={K} a multiple of 8")
     if swiglu_pairs and (N % 2 or weight.order is not None):
         raise KernelError("wide_gemm: gate/up pairs need an even number of weight rows in their natural order")
     mod = load_module("gemm_wide")
     if _tiled_size(N, K, weight.tile_rows) != weight.tiled.numel():
         raise KernelError(f"wide_gemm: the copy is not that of a [{N}, {K}] weight in tiles of {weight.tile_rows} rows")
-    plan = mod.fn("ifx_wide_gemm_plan", (I, I, I, I, I, I))(N, K, waves, slices, 1 if swiglu_pairs else 0, weight.tile_rows)
+    plan = mod.fn("ifx_wide_gemm_plan", (I, I, I, I, I, I, I))(M, N, K, waves, slices, 1 if swiglu_pairs else 0, weight.tile_rows)
     n_waves, n_slices = plan // 256, plan % 256
     part = torch.empty((n_slices, M, N), dtype=torch.float32, device=x.device) if n_slices > 1 else None
     keep = keep_slices and n_slices > 1
@@ -613,12 +616,15 @@ def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional
     Measured on the 7B shapes: up to 16 rows the product that splits K over the waves of a workgroup (with x
     staged in LDS for very tall weights such as the head's when there is no tiled copy); from 17 to 64 rows
     the product that shares x through LDS, which needs the tiled copy (without it, the first kernel up to 32
-    rows on narrow weights); beyond that the library's tiles reuse the rows better."""
+    rows on narrow weights); from 65 to 128 rows the same product for weights of few rows, whose K it cuts into
+    slices to fill the chip where the library has too few output tiles to (down, o and q/k/v of the 7B shape:
+    37-50, 15-21 and 16-22 us against 58-66, 30-34 and 30-37); beyond that, and for tall weights such as gate/up
+    and the head, the library's tiles reuse the rows better."""
     if K % 8:
         return None
     if M <= 16:
         return "staged" if N >= 65536 and not has_tiled else "skinny"
-    if M <= SKINNY_MAX_M and has_tiled:
+    if has_tiled and (M <= SKINNY_MAX_M or (M <= WIDE_MAX_M and N <= WIDE_MANY_ROWS_MAX_N)):
         return "wide"
     if M <= 32 and N <= 4096:
         return "skinny"

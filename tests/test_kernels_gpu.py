@@ -890,7 +890,7 @@ def test_fused_qkv_random_shapes(seed):
     assert torch.all(vc.cpu().permute(0, 3, 1, 2).reshape(pages * P_, -1)[~written] == 0), case
 
 
-@pytest.mark.parametrize("M", [9, 17, 32, 33, 50, 64])
+@pytest.mark.parametrize("M", [9, 17, 32, 33, 50, 64, 65, 81, 100, 128])
 @pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136)])
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
 @pytest.mark.parametrize("tile_rows", [16, 14, 10])
@@ -908,10 +908,10 @@ def test_wide_gemm(M, N, K, out_dtype, tile_rows):
         assert torch.equal(ops.linear(x.to(DEV), lw, out_dtype).cpu().double(), got)   # what linear picks at these rows
 
 
-@pytest.mark.parametrize("waves,slices", [(8, 1), (8, 3), (11, 2), (16, 1), (16, 8)])
-def test_wide_gemm_every_launch_shape_gives_the_same_product(waves, slices):
+@pytest.mark.parametrize("waves,slices,M", [(8, 1, 41), (8, 3, 41), (11, 2, 41), (16, 1, 41), (16, 8, 41), (8, 1, 113), (8, 4, 113), (8, 9, 70)])
+def test_wide_gemm_every_launch_shape_gives_the_same_product(waves, slices, M):
     g = gen(41)
-    M, N, K = 41, 333, 1096                    # 9 rounds of 128 k-values, the last one short; 21 row tiles, the last one short
+    N, K = 333, 1096                           # 9 rounds of 128 k-values, the last one short; 21 row tiles, the last one short
     x = torch.randn(M, K, generator=g).to(BF16)
     w = torch.randn(N, K, generator=g).to(BF16)
     lw = ops.prepare_linear(w.to(DEV))
@@ -939,7 +939,9 @@ def test_wide_gemm_gate_up_pairs_and_tile_order():
     with pytest.raises(ops.KernelError, match="wide_gemm"):
         ops.wide_gemm(x.to(DEV), lq, BF16, swiglu_pairs=True)                          # pairs in a permuted copy
     with pytest.raises(ops.KernelError, match="wide_gemm"):
-        ops.wide_gemm(torch.zeros(65, K, dtype=BF16, device=DEV), lq)
+        ops.wide_gemm(torch.zeros(129, K, dtype=BF16, device=DEV), lq)
+    x65 = torch.randn(65, K, generator=g).to(BF16).to(DEV)
+    assert torch.equal(ops.wide_gemm(x65, lq, F32, waves=16), ops.wide_gemm(x65, lq, F32))   # beyond 64 rows: taken as 8 waves
     assert torch.equal(ops.wide_gemm(x.to(DEV), lq, F32, waves=3).cpu().double(), out)    # fewer than 8 waves: taken as 8
 
 
@@ -1001,8 +1003,10 @@ def test_linear_weight_uses_the_copy_for_few_rows_and_the_rows_beyond():
     x = torch.randn(5, 136, generator=g).to(BF16).to(DEV)
     want = x.double().cpu() @ w.double().cpu().t()
     assert torch.allclose(ops.linear(x, lw, out_dtype=F32).cpu().double(), want, rtol=1e-4, atol=2e-3)
-    big = torch.randn(100, 136, generator=g).to(BF16).to(DEV)
+    big = torch.randn(200, 136, generator=g).to(BF16).to(DEV)
     assert torch.all(ops.linear(big, lw) == 0)
+    mid = torch.randn(100, 136, generator=g).to(BF16).to(DEV)          # 65-128 rows of a weight with few rows: the copy again
+    assert torch.allclose(ops.linear(mid, lw, out_dtype=F32).cpu().double(), mid.double().cpu() @ w.double().cpu().t(), rtol=1e-4, atol=2e-3)
     pairs = ops.prepare_linear(w)
     got = ops.linear_swiglu(x, pairs).cpu().double()
     gt, up = want[:, 0::2], want[:, 1::2]
@@ -1032,13 +1036,13 @@ def test_linear_picks_by_weight_type_and_rows():
 
 @pytest.mark.parametrize("seed", range(40))
 def test_linear_random_shapes(seed):
-    """``linear`` and ``linear_swiglu`` at shapes drawn at random: 1-90 rows (the streaming kernels up to 64, the
-    library beyond), 1-6,000 weight rows, K a multiple of 8 up to 4,800, with and without the streamed copy in whatever
+    """``linear`` and ``linear_swiglu`` at shapes drawn at random: 1-150 rows (the streaming kernels up to 64 and, for
+    the weight's copy, 128; the library beyond), 1-6,000 weight rows, K a multiple of 8 up to 4,800, with and without the streamed copy in whatever
     tile height ``prepare_linear`` picks for the weight, partial sums kept or added, bf16 or float out; against
     float64."""
     import random
     rng = random.Random(500 + seed)
-    M = rng.choice([1, rng.randint(2, 16), rng.randint(17, 64), rng.randint(65, 90)])
+    M = rng.choice([1, rng.randint(2, 16), rng.randint(17, 64), rng.randint(65, 128), rng.randint(129, 150)])
     N = rng.choice([rng.randint(1, 40), rng.randint(41, 700), rng.randint(701, 6000)])
     K = 8 * rng.choice([rng.randint(1, 16), rng.randint(17, 150), rng.randint(151, 600)])
     out_dtype = rng.choice([BF16, F32])
