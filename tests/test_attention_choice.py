@@ -134,3 +134,17 @@ def test_the_order_names_every_work_item_once_and_balances_the_units():
         # an XCD's workgroups read the keys of few kv heads (7 query heads each)
         assert len({int(w) // 32 // 7 for w in order[x] if w >= 0}) <= 2
     assert min(sums) >= 48 and max(sums) <= 62, (min(sums), max(sums))
+
+
+def test_library_products_are_cut_only_where_slices_fill_the_chip_and_stay_long():
+    from inferflux_amd.kernels.ops import library_k_slices as f
+    assert [f(M, 3584, 18944) for M in (129, 512, 1024, 2048, 4096)] == [8, 8, 4, 2, 1]     # down of the 7B shape
+    assert all(f(M, 3584, 3584) == 1 and f(M, 4608, 3584) == 1 for M in (129, 512, 2048))  # o, q/k/v: K too short to cut
+    assert f(512, 37888, 3584) == 1 and f(512, 152064, 3584) == 1                           # tall weights fill the chip as they are
+    assert f(512, 2048, 11008) == 4 and f(512, 8192, 29568) == 4                            # down of the 3B and 72B shapes
+    assert f(512, 3584, 18944 + 8) == 1                                                     # slices must be multiples of 8 k-values
+    for M in (130, 777, 3000):
+        for N in (64, 1000, 5120):
+            for K in (2048, 4096, 10000, 65536):
+                S = f(M, N, K)
+                assert S in (1, 2, 4, 8) and K % S == 0 and (S == 1 or (K // S >= 2048 and (K // S) % 8 == 0))

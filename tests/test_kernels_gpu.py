@@ -1020,6 +1020,30 @@ def test_linear_weight_uses_the_copy_for_few_rows_and_the_rows_beyond():
     assert ops.prepare_linear(w.float()).tiled is None  # a 32-bit weight has no copy
 
 
+@pytest.mark.parametrize("M,N,K", [(130, 200, 4096), (512, 136, 16384), (300, 520, 8192 + 4096), (1000, 64, 4096)])
+def test_linear_cuts_deep_narrow_products_of_many_rows_into_slices(M, N, K):
+    """Many rows times a weight with few rows and a long K: the library runs it as a batch of K slices with float32
+    partial sums, which the caller's norm kernel adds; the sum is the product, and without ``keep_slices`` nothing is cut."""
+    g = gen(51)
+    x = torch.randn(M, K, generator=g).to(BF16)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(BF16)
+    want = x.double() @ w.double().t()
+    S = ops.library_k_slices(M, N, K)
+    assert S > 1
+    got = ops.linear(x.to(DEV), w.to(DEV), keep_slices=True)
+    assert isinstance(got, ops.SliceSums) and got.parts.shape == (S, M, N) and got.parts.dtype == F32
+    assert torch.allclose(got.parts.cpu().double().sum(0), want, rtol=1e-4, atol=2e-3 * (K / 4096) ** 0.5)
+    assert torch.allclose(got.sum().cpu().double(), want, rtol=1e-2, atol=0.1)
+    plain = ops.linear(x.to(DEV), w.to(DEV))
+    assert isinstance(plain, torch.Tensor) and torch.allclose(plain.cpu().double(), want, rtol=1e-2, atol=0.1)
+    res = torch.randn(M, N, generator=g)
+    nw = (1 + 0.3 * torch.randn(N, generator=g)).to(BF16)
+    r = res.to(DEV)
+    out = ops.add_rmsnorm(r, got, nw.to(DEV), 1e-5, BF16)                       # the consumer: adds the slices in order
+    assert torch.allclose(r.cpu().double(), res.double() + want, rtol=1e-4, atol=2e-3 * (K / 4096) ** 0.5)
+    assert torch.allclose(out.cpu().double(), pm.rms_norm(res.double() + want, nw.double(), 1e-5), **tol(BF16))
+
+
 def test_linear_picks_by_weight_type_and_rows():
     g = gen(13)
     w = torch.randn(96, 72, generator=g)
