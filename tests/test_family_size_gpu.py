@@ -224,3 +224,50 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(page_size, monkeypatch
         print(f"7B layer, 3,000 tokens in {len(cuts)} portions: {e:.2e}", flush=True)
         assert e < FAMILY_TOL["bfloat16"]["7B"], (cuts, e)        # measured 1.4e-2 to 1.7e-2, whole and cut alike
     assert {t[0] for t in tilings} == {1, 2} and len({t[1] for t in tilings}) >= 3, tilings
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_mixed_requests_at_the_7b_layer_shape(seed):
+    """Five requests of 200-900 tokens through one layer of the 7B shape, up to four live at a time, in portions of 2-600
+    tokens beside single decoded tokens, in a pool so small that pages are used again: steps of 1-16, 17-64, 65-128
+    and more rows meet every product kernel (the streaming ones, the one that shares x through LDS up to 128 rows,
+    the library whole and in slices of K) and both attention kernels in one batch.  bfloat16 against the float32
+    engine running each request whole."""
+    import random
+    import traces
+    from inferflux_amd.config import config_from_dict
+    from inferflux_amd.engine.context import StepEntry
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    cfg = config_from_dict(dict(SHAPE, num_hidden_layers=1, tie_word_embeddings=True))
+    rng = random.Random(70 + seed)
+    seqs = {f"r{i}": seeded_ids(900 + 10 * seed + i, rng.randint(200, 900), SHAPE["vocab_size"]) for i in range(5)}
+    steps, expected = traces.mixed(seqs, seed=seed, chunk_sizes=(2, 9, 17, 40, 70, 100, 128, 129, 300, 600))
+    rows_per_step = sorted({sum(len(e["tokens"]) for e in st["entries"]) for st in steps})
+    assert rows_per_step[0] <= 16 and any(64 < n <= 128 for n in rows_per_step) and rows_per_step[-1] > 256, rows_per_step
+    ref_runner = ModelRunner(Model(cfg).init_random(21, torch.float32, torch.device("cuda", 0)), num_pages=60, max_requests=2)
+    ref = {}
+    for rid, ids in seqs.items():
+        ref_runner.add_request(rid)
+        ref[rid] = ref_runner.step([StepEntry(rid, ids, list(range(len(ids))))]).cpu()
+        ref_runner.free_request(rid)
+    del ref_runner
+    torch.cuda.empty_cache()
+    pages = traces.peak_tokens(steps, round_to=16) // 16
+    runner = ModelRunner(Model(cfg).init_random(21, torch.bfloat16, torch.device("cuda", 0)), num_pages=pages, max_requests=4)
+    got, want = [], []
+    for st in steps:
+        for e in st["entries"]:
+            if not runner.has_request(e["id"]):
+                runner.add_request(e["id"])
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+        if st["step"] in expected:
+            got.append(logits.float().cpu())
+            want += [ref[rid][p] for rid, p in expected[st["step"]]]
+        for rid in st["end"]:
+            runner.free_request(rid)
+    e = rel_err(torch.cat(got), torch.stack(want))
+    print(f"7B layer, mixed requests, seed {seed}: {e:.2e} over {len(want)} rows, steps of {rows_per_step[0]}-{rows_per_step[-1]} rows", flush=True)
+    assert e < FAMILY_TOL["bfloat16"]["7B"], e
+    runner.manager.check()
+    assert runner.manager.free_pages() == [pages]
