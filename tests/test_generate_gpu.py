@@ -18,7 +18,7 @@ if torch.cuda.is_available():
     from inferflux_amd import Engine, SamplingParams
     from inferflux_amd.sampling.params import philox_uniform
 
-# BASELINE workloads of the tiny configurations: prompts of 7/13/29 tokens with 16 greedy tokens
+# Generation workloads of the tiny configurations: prompts of 7/13/29 tokens with 16 greedy tokens
 # each (A); prompts of 1/17/64/100/250 with 24 tokens, prefill portions of 32, pages of 16 (B).
 WORKLOADS = {"A": ([7, 13, 29], 16, 512), "B": ([1, 17, 64, 100, 250], 24, 32), "C": ([40, 3, 90], 20, 16)}
 
