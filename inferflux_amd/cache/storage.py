@@ -58,6 +58,8 @@ class CacheStorage:
         # One page more than the manager hands out, at the end of every cache tensor: the scratch page, which rows
         # that stand for nobody (padding of a captured decode step's batch) write to and read back.
         self.scratch_pages = list(counts)
+        # ... and one state slot more than the manager hands out, for the same rows: what they leave there is read by nobody.
+        self.scratch_state_slot = max_requests
         self._caches: Dict[int, LayerCache] = {}
         self._states: Dict[int, torch.Tensor] = {}
         for i, e in enumerate(schedule):
@@ -71,7 +73,7 @@ class CacheStorage:
                 self._caches[i] = LayerCache(k, v, g, page_size)
             st = m.state_spec()
             if st is not None:
-                self._states[i] = torch.zeros((max_requests, *st.shape), dtype=_STATE_DTYPES[st.dtype], device=device)
+                self._states[i] = torch.zeros((max_requests + 1, *st.shape), dtype=_STATE_DTYPES[st.dtype], device=device)
         if self._states:
             self.manager.on_add = self.reset_state       # every admission path starts a request with zero state
         self._bindings: List[MixerBinding] = []

@@ -194,20 +194,149 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   }
 }
 
+// The same walk by a workgroup of ``a.waves`` waves per (row, kv head), for launches whose (row, kv head) pairs fill
+// the chip by themselves: the row's visible keys are dealt evenly to the waves in runs of 32, every wave walks its
+// share exactly as above, and the waves' (max, sum, unnormalised output) meet in LDS, are combined in wave order and
+// written to ``out``.  No partial results in memory and no second launch (64 rows x 4 kv heads over 3,100 keys:
+// 67 us against 88 in splits with the merge launch).
+//
+// Fewer pairs than compute units need a pair's keys on several units, hence a merge across workgroups.  Measured
+// for that, and not kept: the workgroup that finishes a row last merges it inside the launch (partial results,
+// a release fence at device scope, a counter per pair).  The fence (a write-back of the unit's L2) takes about
+// 45-60 ns per workgroup and the chip serves them one after the other: 8 rows over 3,100 keys in 224 workgroups
+// 36 us against 21 with the merge launch, 64 rows in 8,192 workgroups 518 us against 104; without the fence (wrong,
+// for timing) 21 and 154 us, the counters' atomics costing about 10 ns apiece on top.
+//
+// Dynamic LDS: waves x nc x (D + 4) floats of outputs and waves x nc x 2 of (max, sum); nc = heads per pass.
+constexpr int OPAD = D + 4;       // floats per output row in LDS (the padding spreads the 16 columns over the banks)
+
+template <bool STREAM>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_rows_whole_kernel(RowArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int kvh = blockIdx.x, ri = blockIdx.y;
+  const int tid = threadIdx.x, wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g4 = lane >> 4;
+  const int W = a.waves, n_threads = W * WAVE;
+  const int row = a.rows ? a.rows[ri] : ri;
+  const int pos = a.positions[row];
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  // this wave's keys: the visible ones from the first visible run of 32 on, in W equal shares of whole runs
+  const int first = lo / 32 * 32;
+  const int chunk = ((pos + 1 - first + W - 1) / W + 31) / 32 * 32;
+  const int ka = max(lo, first + wid * chunk), kb = min(pos + 1, first + (wid + 1) * chunk);
+  const int ratio = a.nH / a.nKV;
+  const int nc_max = min(16, ratio);
+  const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
+  float* o_s = lds;                                        // [W][nc_max][OPAD]
+  float* ml_s = lds + W * nc_max * OPAD;                   // [W][nc_max][2]
+  constexpr int D4 = D / 4;
+
+  for (int qt = 0; qt < ratio; qt += 16) {
+    const int nc = min(16, ratio - qt);
+    const int head = kvh * ratio + qt + col;
+    const bool head_ok = col < nc;
+    floatx4 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    if (ka < kb) {
+      bf16x8 qop[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int c = 32 * ks + 8 * g4;
+        qop[ks] = (head_ok && c < D) ? *(const bf16x8*)(a.q + ((size_t)row * a.nH + head) * D + c) : zero8();
+      }
+      RowBlock b0, b1;
+      int j0 = (ka / 32) * 32;
+      int page_base = 0, pages = -1;
+      bool have_pages = false;
+      auto table_for = [&](int j) {
+        if (have_pages && (j + 31) / a.P - page_base < WAVE) return;
+        have_pages = true;
+        page_base = j / a.P;
+        pages = page_base + lane < a.max_blocks ? table[page_base + lane] : -1;
+      };
+      table_for(j0);
+      load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0, ka, kb, col, g4);
+      for (; j0 < kb; j0 += 64) {
+        const bool more1 = j0 + 32 < kb, more2 = j0 + 64 < kb;
+        if (more1) {
+          table_for(j0 + 32);
+          load_row_block<STREAM>(b1, a, pages, page_base, kvh, j0 + 32, ka, kb, col, g4);
+        }
+        use_row_block(b0, a, qop, o, m, l, j0, ka, kb, g4);
+        if (more1) {
+          if (more2) {
+            table_for(j0 + 64);
+            load_row_block<STREAM>(b0, a, pages, page_base, kvh, j0 + 64, ka, kb, col, g4);
+          }
+          use_row_block(b1, a, qop, o, m, l, j0 + 32, ka, kb, g4);
+        }
+      }
+      l = col_sum(l);
+    }
+    // the waves' results meet in LDS (a wave without visible keys brings weight zero)
+    if (qt > 0) __syncthreads();                           // everyone is done with the last pass's LDS
+    if (head_ok) {
+      float* os = o_s + (wid * nc_max + col) * OPAD;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(floatx4*)(os + 16 * dt + 4 * g4) = o[dt];
+      if (g4 == 0) { ml_s[(wid * nc_max + col) * 2] = m; ml_s[(wid * nc_max + col) * 2 + 1] = l; }
+    }
+    __syncthreads();
+    for (int i = tid; i < nc * D4; i += n_threads) {
+      const int c = i / D4, e = 4 * (i % D4);
+      float M = -INFINITY;
+      for (int w = 0; w < W; ++w) M = fmaxf(M, ml_s[(w * nc_max + c) * 2]);
+      floatx4 acc{0.f, 0.f, 0.f, 0.f};
+      float L = 0.f;
+      for (int w = 0; w < W; ++w) {
+        const float mw = ml_s[(w * nc_max + c) * 2];
+        if (mw == -INFINITY) continue;
+        const float wgt = fast_exp2(mw - M);
+        L = fmaf(wgt, ml_s[(w * nc_max + c) * 2 + 1], L);
+        const floatx4 v = *(const floatx4*)(o_s + (w * nc_max + c) * OPAD + e);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = fmaf(wgt, v[r], acc[r]);
+      }
+      const float inv = L > 0.f ? 1.f / L : 0.f;
+      bf16x4 w4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(acc[r] * inv);
+      *(bf16x4*)(a.out + ((size_t)row * a.nH + kvh * ratio + qt + c) * D + e) = w4;
+    }
+  }
+}
+
+// ``waves`` 0: one wave per (row, kv head, split of ``chunk`` keys) and a second launch that merges the splits
+// (``max_splits`` * chunk must reach past every row's position; part_o / part_ml are the partial results).
+// ``waves`` 1-8: one workgroup of that many waves per (row, kv head), which shares the row's keys evenly and writes
+// the output itself; chunk, max_splits and the scratch are not used.
 extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_cache, void* out, const int* rows,
                              const int* row_req, const int* positions, const int* block_table, int max_blocks,
                              int n_rows, int nH, int nKV, int d, int page_size, int window, int chunk,
-                             int max_splits, float scale, float* part_o, float* part_ml, void* stream) {
+                             int max_splits, float scale, float* part_o, float* part_ml, int waves, void* stream) {
   IFX_REQUIRE(d == D, "attn_rows: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_rows >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_rows: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_rows: page_size %d must be a multiple of 16", page_size);
-  IFX_REQUIRE(chunk > 0 && chunk % 32 == 0 && max_splits > 0 && max_splits <= 65535, "attn_rows: bad chunk %d / splits %d", chunk, max_splits);
   IFX_REQUIRE(nKV <= 65535 && n_rows <= 65535, "attn_rows: too many kv heads or rows for one launch");
+  IFX_REQUIRE(waves >= 0 && waves <= 8, "attn_rows: %d waves per workgroup (0-8)", waves);
   if (n_rows == 0) return 0;
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-            scale * 1.4426950408889634f, 0};
+            scale * 1.4426950408889634f, 0, waves};
   hipStream_t s = (hipStream_t)stream;
+  if (waves > 0) {
+    const int nc = nH / nKV < 16 ? nH / nKV : 16;
+    const size_t lds = (size_t)waves * nc * (OPAD + 2) * sizeof(float);
+    IFX_REQUIRE(lds <= 65536, "attn_rows: %d waves of %d heads need %zu bytes of LDS", waves, nc, lds);
+    if (n_rows >= ROW_STREAM_MIN_ROWS)
+      hipLaunchKernelGGL(attn_rows_whole_kernel<true>, dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+    else
+      hipLaunchKernelGGL(attn_rows_whole_kernel<false>, dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
+    IFX_LAUNCH_CHECK();
+  }
+  IFX_REQUIRE(chunk > 0 && chunk % 32 == 0 && max_splits > 0 && max_splits <= 65535, "attn_rows: bad chunk %d / splits %d", chunk, max_splits);
+  IFX_REQUIRE(part_o && part_ml, "attn_rows: splits need scratch for their partial results");
   if (n_rows >= ROW_STREAM_MIN_ROWS) hipLaunchKernelGGL(attn_rows_kernel<true>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
   else hipLaunchKernelGGL(attn_rows_kernel<false>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
   hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, a);

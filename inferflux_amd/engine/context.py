@@ -30,11 +30,12 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
-def _pad_arrays(arrays, n_pad: int, scratch_pages: Sequence[int], page_size: int):
+def _pad_arrays(arrays, n_pad: int, scratch_pages: Sequence[int], page_size: int, scratch_state_slot: int = 0):
     """``arrays`` of a step (``CacheManager.step_arrays``) with ``n_pad`` rows that stand for nobody appended: each is
     a request of its own with one token at position 0 whose key and value go to the group's scratch page (a page
-    outside every pool, which nobody's block table names) and which reads that one key back.  Such rows keep a
-    step's layout the same while the number of real requests changes; what they compute is thrown away."""
+    outside every pool, which nobody's block table names) and which reads that one key back; a mixer with state of
+    its own is given ``scratch_state_slot`` for them (a slot no request ever holds).  Such rows keep a step's layout
+    the same while the number of real requests changes; what they compute is thrown away."""
     R, T = arrays["q_len"].shape[0], arrays["positions"].shape[0]
     i32 = lambda v: np.asarray(v, dtype=np.int32)
     out = dict(arrays)
@@ -42,7 +43,7 @@ def _pad_arrays(arrays, n_pad: int, scratch_pages: Sequence[int], page_size: int
     out["q_start"] = np.concatenate([arrays["q_start"], i32(np.arange(T, T + n_pad))])
     out["q_len"] = np.concatenate([arrays["q_len"], np.ones(n_pad, np.int32)])
     out["kv_len"] = np.concatenate([arrays["kv_len"], np.ones(n_pad, np.int32)])
-    out["state_slots"] = np.concatenate([arrays["state_slots"], np.zeros(n_pad, np.int32)])
+    out["state_slots"] = np.concatenate([arrays["state_slots"], np.full(n_pad, scratch_state_slot, np.int32)])
     out["row_req"] = np.concatenate([arrays["row_req"], i32(np.arange(R, R + n_pad))])
     out["positions"] = np.concatenate([arrays["positions"], np.zeros(n_pad, np.int32)])
     tables, slots = [], []
@@ -60,12 +61,13 @@ class StepContext:
     for many steps).  ``slab`` is a device buffer to fill instead of a new one, ``pinned`` the host
     buffer the copy goes through; ``layout_key`` tells whether two steps have the same layout.
     ``pad_requests`` appends that many rows that stand for nobody (see ``_pad_arrays``; ``scratch_pages``: per
-    cache group the page they write to); their logits come last and are the caller's to drop.  ``n_requests``
+    cache group the page they write to, ``scratch_state_slot``: the state slot they use); their logits come last and
+    are the caller's to drop.  ``n_requests``
     and ``n_tokens`` count them, ``n_real_requests`` and ``n_real_tokens`` do not."""
 
     def __init__(self, entries: Sequence[StepEntry], manager, act_dtype: torch.dtype, device,
                  width_multiple: int = 8, slab: torch.Tensor = None, pinned: torch.Tensor = None, upload: bool = True,
-                 pad_requests: int = 0, scratch_pages: Sequence[int] = ()):
+                 pad_requests: int = 0, scratch_pages: Sequence[int] = (), scratch_state_slot: int = 0):
         self.act_dtype, self.device = act_dtype, device
         self.timer = None              # a tracing.PhaseTimer while per-phase timing is on
         self.entries = list(entries)
@@ -76,7 +78,7 @@ class StepContext:
         if pad_requests > 0:
             if len(scratch_pages) != len(manager.groups):
                 raise ValueError("padding rows need a scratch page for every cache group")
-            arrays = _pad_arrays(arrays, pad_requests, scratch_pages, manager.page_size)
+            arrays = _pad_arrays(arrays, pad_requests, scratch_pages, manager.page_size, scratch_state_slot)
         R = self.n_requests = self.n_real_requests + max(pad_requests, 0)
         q_len, q_start, start = arrays["q_len"], arrays["q_start"], arrays["start"]
         T = self.n_tokens = int(arrays["positions"].shape[0])

@@ -136,12 +136,11 @@ class ModelRunner:
     def _decode_context(self, entries) -> StepContext:
         """The context of a step of single tokens in the layout its captured graph has: block tables as wide as the
         next multiple of GRAPH_WIDTH_MULTIPLE pages, the batch filled up to the next of GRAPH_BATCH_SIZES."""
-        n, pad = len(entries), 0
-        if not self.storage.has_state:          # (a row that stands for nobody would still need a state slot to scribble on)
-            size = next((b for b in self.GRAPH_BATCH_SIZES if b >= n), -(-n // 16) * 16)
-            pad = size - n
+        n = len(entries)
+        size = next((b for b in self.GRAPH_BATCH_SIZES if b >= n), -(-n // 16) * 16)
         return StepContext(entries, self.manager, self.dtype, self.device, width_multiple=self.GRAPH_WIDTH_MULTIPLE,
-                           upload=False, pad_requests=pad, scratch_pages=self.storage.scratch_pages)
+                           upload=False, pad_requests=size - n, scratch_pages=self.storage.scratch_pages,
+                           scratch_state_slot=self.storage.scratch_state_slot)
 
     @property
     def starts_steps_early(self) -> bool:

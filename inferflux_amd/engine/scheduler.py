@@ -23,11 +23,12 @@ Order of admission.  The reference sorts its queues by a score, priority + age_m
 arrival (scheduler/batch_selection_policy.cpp:10-20; scheduler/scheduler.cpp:2013-2031).  Here a
 request carries a ``priority`` (0 unless given) and the scheduler a ``score`` function of the
 waiting request; the waiting request with the highest score is admitted next, the earlier arrival
-among equals.  The default score is the priority alone, which is first come first served while
-nobody sets one; ``priority_age_score`` is the reference's.  The best-scoring request that does
-not fit blocks those behind it (no overtaking by smaller requests, hence no starvation).  When
-pages run out the victim is the running request of lowest priority, the most recently admitted
-among those.
+among equals.  The default score is the reference's (``priority_age_score``): every two seconds
+of waiting count as one step of priority, so a steady stream of more important arrivals cannot
+keep a waiting request out for ever, and while nobody sets a priority the order is first come
+first served; ``priority_score`` is the priority alone.  The best-scoring request that does
+not fit blocks those behind it (no overtaking by smaller requests).  When pages run out the
+victim is the running request of lowest priority, the most recently admitted among those.
 """
 from __future__ import annotations
 
@@ -100,13 +101,14 @@ class StepPlan:
 
 
 def priority_score(seq: "Sequence_", now: float) -> float:
-    """The default: the request's priority; equal priorities are served in arrival order."""
+    """The request's priority alone; equal priorities are served in arrival order.  Under it a stream of more
+    important arrivals keeps a less important request waiting for as long as it lasts."""
     return float(seq.priority)
 
 
 def priority_age_score(aging_divisor_ms: float = 2000.0) -> Callable[["Sequence_", float], float]:
-    """The reference's policy: every ``aging_divisor_ms`` of waiting adds one to the effective priority
-    (scheduler/batch_selection_policy.cpp:10-20)."""
+    """The default, and the reference's policy: every ``aging_divisor_ms`` of waiting adds one to the effective
+    priority (scheduler/batch_selection_policy.cpp:10-20)."""
     def score(seq: "Sequence_", now: float) -> float:
         return float(seq.priority) + (now - seq.arrival_time) * 1e3 / aging_divisor_ms
     return score
@@ -116,11 +118,11 @@ class Scheduler:
     def __init__(self, manager: CacheManager, config: SchedulerConfig, max_position: int,
                  score: Optional[Callable[["Sequence_", float], float]] = None,
                  clock: Callable[[], float] = time.monotonic):
-        """``score(request, now)``: the waiting request with the highest is admitted next (``priority_score`` unless
-        given); ``clock`` gives ``now`` and the requests' arrival times, in seconds."""
+        """``score(request, now)``: the waiting request with the highest is admitted next (``priority_age_score()``
+        unless given); ``clock`` gives ``now`` and the requests' arrival times, in seconds."""
         config.validate()
         self.manager, self.config, self.max_position = manager, config, max_position
-        self.score, self.clock = score or priority_score, clock
+        self.score, self.clock = score or priority_age_score(), clock
         self.waiting: Deque[Sequence_] = collections.deque()
         self.running: List[Sequence_] = []
         self._arrivals = 0

@@ -32,6 +32,8 @@ TILE_ORDER_MIN_ITEMS = 64       # launches of more workgroups than this get them
 ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
 ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
 ROW_MAX_SPLITS = 128  # and until a row has at most this many splits (one row over 131,072 keys: 91 us against 133 at 64)
+ROW_WHOLE_MIN_PAIRS = 192   # (row, kv head) pairs from which a workgroup takes a pair's keys whole
+ROW_WAVE_SLOTS = 2048       # waves the chip holds at the row kernel's two per SIMD
 
 
 DIRECT_MIN_WORK = 1 << 18       # rows x keys seen per row from which the tall tiles of head size 128 win
@@ -153,7 +155,7 @@ def tile_order(first_pos, last_pos, n_heads: int, window: Optional[int], splits:
     return order.reshape(-1)
 
 
-def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk=0, window=None):
+def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk=0, window=None, row_waves=8):
     """What the kernels need beyond the step's own arrays, computed once per step (and per number of
     kv heads, which decides how many waves a launch has)."""
     q_len, q_start, kv_len = ctx.h_q_len, ctx.h_q_start, ctx.h_kv_len
@@ -164,7 +166,7 @@ def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk
             tile_req.append(r); tile_q0.append(q0)
     row_mask = ~tiled[ctx.h_row_req] if ctx.n_tokens else np.zeros(0, bool)
     rows = np.nonzero(row_mask)[0].astype(np.int32)
-    out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1,
+    out = {"n_tiles": len(tile_req), "n_rows": int(rows.size), "rows": None, "chunk": ROW_CHUNK, "max_splits": 1, "waves": 0,
            "tile_splits": 1, "tile_chunk": 0, "tile_row_list": None, "tile_order": None}
     lists = {}                       # everything that goes to the device, in one copy (each copy is a wait for the host)
     if tile_req:
@@ -189,14 +191,33 @@ def _work_lists(ctx, ctx_kv_heads, tile_rows, n_heads, tile_splits=1, tile_chunk
             out[k] = packed[at:at + n]
             at += n + -n % 4          # every list starts at a multiple of 16 bytes
     if rows.size:
-        max_kv = ctx.kv_bound     # not the lengths themselves: see StepContext.kv_bound
-        chunk = ROW_CHUNK
-        n_kv_heads = ctx_kv_heads
-        while (-(-max_kv // chunk) > ROW_MAX_SPLITS
-               or int(rows.size) * n_kv_heads * -(-max_kv // (2 * chunk)) >= ROW_MIN_WAVES):
-            chunk *= 2
-        out["chunk"], out["max_splits"] = chunk, -(-max_kv // chunk)
+        out["chunk"], out["waves"], out["max_splits"] = row_launch_shape(int(rows.size), ctx_kv_heads, ctx.kv_bound, row_waves)
     return out
+
+
+def row_launch_shape(n_rows: int, n_kv_heads: int, max_kv: int, max_waves: int = 8):
+    """(keys per split, waves per workgroup, splits) of a launch of the row kernel over ``n_rows`` rows whose requests
+    hold at most ``max_kv`` keys (the bound of their block tables, not the lengths themselves: see
+    StepContext.kv_bound).  ``max_waves``: what fits the kernel's LDS (``ops.row_waves_fit``).
+
+    With (row, kv head) pairs enough to fill the chip by themselves, one workgroup takes a pair whole (keys per split
+    0): its waves, as many as give the chip about one round of 2,048, share the row's keys evenly, meet in LDS and
+    write the output, with no partial results in memory and no second launch.  Measured at 28 : 4 heads of 128 over
+    3,100 keys, us whole / in splits with the merge launch: 48 rows 61 / 69, 64 rows 68 / 88, 96 rows 116 / 133, 128
+    rows 129 / 178, 256 rows 250 / 361; 64 rows over 16,384 keys 328 / 358; 32 rows 57 / 48, so fewer pairs than 192
+    keep the splits: their keys have to be spread over more compute units than there are pairs, which only a second
+    launch can merge (one wave per split of ``chunk`` keys, waves per workgroup 0)."""
+    pairs = n_rows * n_kv_heads
+    if pairs >= ROW_WHOLE_MIN_PAIRS:
+        waves = 1
+        while waves * 2 <= min(max_waves, ROW_WAVE_SLOTS // pairs):
+            waves *= 2
+        return 0, waves, 1
+    chunk = ROW_CHUNK
+    while (-(-max_kv // chunk) > ROW_MAX_SPLITS
+           or pairs * -(-max_kv // (2 * chunk)) >= ROW_MIN_WAVES):
+        chunk *= 2
+    return chunk, 0, -(-max_kv // chunk)
 
 
 def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: float) -> torch.Tensor:
@@ -213,8 +234,8 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
         qt, splits, chunk = choose_tiling(ctx.h_q_len[tiled], ctx.h_kv_len[tiled], nH, lambda t: ops.attention_tile_rows(d, t),
                                           tall_direct=d == ops.DIRECT_TILE_HEAD_DIM)
     tile_rows = ops.attention_tile_rows(d, qt)
-    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk, window),
-                    lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk, window))
+    w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk, window, d),
+                    lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk, window, ops.row_waves_fit(nH, n_kv, d, ops.ROW_MAX_WAVES)))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
@@ -222,5 +243,5 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
                             ctx.positions, w["tile_order"])
     if w["n_rows"]:
         ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
-                           window, scale, w["chunk"], w["max_splits"])
+                           window, scale, w["chunk"], w["max_splits"], w["waves"])
     return out

@@ -132,9 +132,13 @@ def _lib_filename(name: str, variant: Variant) -> str:
 
 def find_library(name: str, variant: Variant = ()) -> Optional[str]:
     fn = _lib_filename(name, variant)
-    for d in (CSRC, _fallback_dir()):
-        if d is None:
-            continue
+    p = os.path.join(CSRC, fn)
+    if os.path.isfile(p):
+        return p
+    # Only a library that is not beside the sources is looked for in the per-user folder, so that a folder of that
+    # name which fails the ownership check (anybody can make one) cannot stop a tree that has everything built.
+    d = _fallback_dir()
+    if d is not None:
         p = os.path.join(d, fn)
         if os.path.isfile(p):
             return p

@@ -94,13 +94,20 @@ def attention_rows(args) -> None:
     out = torch.empty(B, nH * d, device=dev, dtype=torch.bfloat16)
     row_req = torch.arange(B, dtype=torch.int32, device=dev)
     pos = torch.full((B,), kv - 1, dtype=torch.int32, device=dev)
-    for chunk in ([args.chunk] if args.chunk else [128, 256, 512, 1024]):
-        splits = -(-kv // chunk)
+    bound = -(-kv // (64 * P)) * 64 * P if args.graph_width else kv   # a captured step's grid covers its block-table width
+    gb = B * kv * nKV * d * 2 * 2 / 1e9
+    for chunk in ([int(c) for c in args.chunk.split(",")] if args.chunk else [128, 256, 512, 1024]):
+        splits = -(-bound // chunk)
         t = _time_us(lambda i: ops.attention_rows(q, *caches[i % copies], out, None, B, row_req, pos, table, None,
                                                   1 / math.sqrt(d), chunk, splits), args.iters)
-        gb = B * kv * nKV * d * 2 * 2 / 1e9
-        print(f"attention-rows batch={B} context={kv} chunk={chunk} splits={splits}: {t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache "
-              f"(row kernel + merge)", flush=True)
+        print(f"attention-rows batch={B} context={kv} one wave per split of {chunk} keys ({splits} splits) + merge launch: "
+              f"{t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache", flush=True)
+    for waves in [int(w) for w in args.waves.split(",") if w]:
+        waves = ops.row_waves_fit(nH, nKV, d, waves)
+        t = _time_us(lambda i: ops.attention_rows(q, *caches[i % copies], out, None, B, row_req, pos, table, None,
+                                                  1 / math.sqrt(d), 0, 1, waves), args.iters)
+        print(f"attention-rows batch={B} context={kv} one workgroup of {waves} waves per (row, kv head): "
+              f"{t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache", flush=True)
 
 
 def gemm(args) -> None:
@@ -179,7 +186,10 @@ def main(argv=None) -> int:
         if name == "attention-rows":
             p.add_argument("--batch", type=int, default=8)
             p.add_argument("--context", type=int, default=3072)
-            p.add_argument("--chunk", type=int, default=0, help="keys per split (0: 128, 256, 512 and 1024)")
+            p.add_argument("--chunk", default="", help="keys per split, comma separated (empty: 128, 256, 512 and 1024)")
+            p.add_argument("--waves", default="4,8", help="also: one workgroup of this many waves per (row, kv head), comma separated")
+            p.add_argument("--graph-width", action="store_true", help="size the grid by the block-table width a captured step has "
+                           "(the next multiple of 64 pages), not by the context")
             p.add_argument("--rotate-gb", type=float, default=2.0,
                            help="memory the launches rotate through (a model's step touches tens of GB between two uses of a cache)")
             p.add_argument("--pages", choices=["shuffled", "in-order"], default="shuffled", help="how a request's pages lie in the pool")

@@ -719,12 +719,27 @@ def _attn_common(q, k_cache, v_cache, qt=1):
     return T, nH, d, nKV, page_size, load_module(name, variant)
 
 
+ROW_MAX_WAVES = 8
+
+
+def row_waves_fit(n_heads: int, n_kv_heads: int, head_dim: int, waves: int) -> int:
+    """The most waves per workgroup, up to ``waves``, whose results fit the row kernel's 64 KB of LDS."""
+    nc = min(16, n_heads // n_kv_heads)
+    while waves > 1 and waves * nc * (head_dim + 6) * 4 > 65536:
+        waves //= 2
+    return waves
+
+
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                    rows: Optional[torch.Tensor], n_rows: int, row_req: torch.Tensor, positions: torch.Tensor,
-                   block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int) -> None:
+                   block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int,
+                   waves: int = 0) -> None:
     """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].
-    Split s of a row covers key positions [s*chunk, (s+1)*chunk); ``max_splits`` * chunk must reach
-    past the largest position among the rows."""
+
+    ``waves`` 0: split s of a row covers key positions [s*chunk, (s+1)*chunk), one wave each, and a second launch
+    merges a row's splits; ``max_splits`` * chunk must reach past the largest position among the rows.
+    ``waves`` 1-8: one workgroup of that many waves per (row, kv head) shares the row's keys evenly and writes the
+    output itself (``chunk`` and ``max_splits`` are not used): for launches with pairs enough to fill the chip."""
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache)
     _check(out, "out", (T, nH * d), torch.bfloat16)
     _check(row_req, "row_req", (T,), torch.int32)
@@ -734,12 +749,17 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         _check(rows, "rows", (n_rows,), torch.int32)
     elif n_rows != T:
         raise KernelError("attention_rows: without a row list every row of the batch is handled")
-    part_o = torch.empty((n_rows, nH, max_splits, d), dtype=torch.float32, device=q.device)
-    part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
-    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, P),
+    if not 0 <= waves <= ROW_MAX_WAVES or row_waves_fit(nH, nKV, d, waves) != waves:
+        raise KernelError(f"attention_rows: {waves} waves per workgroup (0-{ROW_MAX_WAVES}, and their results within 64 KB of LDS: "
+                          f"up to {row_waves_fit(nH, nKV, d, ROW_MAX_WAVES)} at these head counts)")
+    part_o = part_ml = None
+    if waves == 0:
+        part_o = torch.empty((n_rows, nH, max_splits, d), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
+    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(rows), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_rows, nH, nKV, d, page_size,
-          int(window or 0), chunk, max_splits, float(scale), part_o.data_ptr(), part_ml.data_ptr(), _stream())
+          int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, _stream())
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:

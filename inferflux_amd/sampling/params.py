@@ -72,8 +72,23 @@ _W0, _W1 = np.uint32(0x9E3779B9), np.uint32(0xBB67AE85)
 _MASK = np.uint64(0xFFFFFFFF)
 
 
+def philox4x32_10(counter, key):
+    """The ten rounds of Philox4x32 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", 2011) on arrays:
+    ``counter`` four and ``key`` two arrays of 32-bit words (as uint64); returns the four output words."""
+    c = [np.asarray(w, dtype=np.uint64) & _MASK for w in counter]
+    k0, k1 = (np.asarray(key[0], dtype=np.uint64) & _MASK).astype(np.uint32), (np.asarray(key[1], dtype=np.uint64) & _MASK).astype(np.uint32)
+    with np.errstate(over="ignore"):
+        for _ in range(10):
+            p0, p1 = _M0 * c[0], _M1 * c[2]
+            c = [((p1 >> np.uint64(32)) ^ c[1] ^ k0.astype(np.uint64)) & _MASK, p1 & _MASK,
+                 ((p0 >> np.uint64(32)) ^ c[3] ^ k1.astype(np.uint64)) & _MASK, p0 & _MASK]
+            k0, k1 = k0 + _W0, k1 + _W1
+    return c
+
+
 def philox_uniform(seeds: np.ndarray, steps: np.ndarray) -> np.ndarray:
-    """One float32 in [0, 1) per (seed, step): Philox4x32-10 keyed by the seed, counter = step.
+    """One float32 in [0, 1) per (seed, step): Philox4x32-10 keyed by the seed, counter = step; the top 24 bits of
+    the first output word.
 
     A counter-based generator: the number depends on the pair alone, not on what was drawn before
     or on which other requests share the batch (the reference's invariant that batched sampling
@@ -81,12 +96,6 @@ def philox_uniform(seeds: np.ndarray, steps: np.ndarray) -> np.ndarray:
     """
     seeds = np.asarray(seeds, dtype=np.uint64)
     steps = np.asarray(steps, dtype=np.uint64)
-    c = [steps & _MASK, steps >> np.uint64(32), np.zeros_like(steps), np.zeros_like(steps)]
-    k0, k1 = (seeds & _MASK).astype(np.uint32), ((seeds >> np.uint64(32)) & _MASK).astype(np.uint32)
-    with np.errstate(over="ignore"):
-        for _ in range(10):
-            p0, p1 = _M0 * c[0], _M1 * c[2]
-            c = [((p1 >> np.uint64(32)) ^ c[1] ^ k0.astype(np.uint64)) & _MASK, p1 & _MASK,
-                 ((p0 >> np.uint64(32)) ^ c[3] ^ k1.astype(np.uint64)) & _MASK, p0 & _MASK]
-            k0, k1 = k0 + _W0, k1 + _W1
+    zero = np.zeros_like(steps)
+    c = philox4x32_10([steps & _MASK, steps >> np.uint64(32), zero, zero], [seeds & _MASK, seeds >> np.uint64(32)])
     return ((c[0] >> np.uint64(8)).astype(np.float64) * (1.0 / (1 << 24))).astype(np.float32)

@@ -162,6 +162,33 @@ def forward(cfg, W, ids, positions=None):
     return linear(h, head)
 
 
+def forward_rows_one_layer(cfg, W, ids, rows):
+    """Logits [len(rows), V] at the places ``rows`` of a whole sequence, for a model of ONE layer: keys and values need
+    the first norm and two projections of every token, everything else is computed for the wanted rows alone, which
+    makes sequences of tens of thousands of tokens at real layer widths affordable on the CPU.  The same functions in
+    the same order as ``forward`` (a test compares the two)."""
+    if cfg["num_hidden_layers"] != 1:
+        raise ValueError("forward_rows_one_layer: the second layer's keys would need every row of the first")
+    S, rows = len(ids), list(rows)
+    positions = list(range(S))
+    eps = cfg.get("rms_norm_eps", 1e-6)
+    nH, nKV = cfg["num_attention_heads"], cfg.get("num_key_value_heads", cfg["num_attention_heads"])
+    d = cfg.get("head_dim") or cfg["hidden_size"] // nH
+    theta = cfg.get("rope_theta", 10000.0)
+    p, a = "model.layers.0", "model.layers.0.self_attn"
+    x = embedding(ids, W["model.embed_tokens.weight"])
+    h = rms_norm(x, W[f"{p}.input_layernorm.weight"], eps)
+    k = rope_split_half(linear(h, W[f"{a}.k_proj.weight"], W.get(f"{a}.k_proj.bias")).view(S, nKV, d), positions, theta)
+    v = linear(h, W[f"{a}.v_proj.weight"], W.get(f"{a}.v_proj.bias")).view(S, nKV, d)
+    q = rope_split_half(linear(h[rows], W[f"{a}.q_proj.weight"], W.get(f"{a}.q_proj.bias")).view(len(rows), nH, d), rows, theta)
+    o = attention(q, k, v, window=layer_window(cfg, 0), q_positions=rows, k_positions=positions)
+    xr = x[rows] + linear(o.reshape(len(rows), nH * d), W[f"{a}.o_proj.weight"])
+    hr = rms_norm(xr, W[f"{p}.post_attention_layernorm.weight"], eps)
+    xr = xr + swiglu(hr, W[f"{p}.mlp.gate_proj.weight"], W[f"{p}.mlp.up_proj.weight"], W[f"{p}.mlp.down_proj.weight"])
+    head = W["lm_head.weight"] if "lm_head.weight" in W else W["model.embed_tokens.weight"]
+    return linear(rms_norm(xr, W["model.norm.weight"], eps), head)
+
+
 def greedy_generate(cfg, W, prompt, n_new):
     """Token ids chosen by argmax (lowest index on ties), recomputing the whole sequence."""
     ids = list(prompt)

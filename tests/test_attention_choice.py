@@ -148,3 +148,21 @@ def test_library_products_are_cut_only_where_slices_fill_the_chip_and_stay_long(
             for K in (2048, 4096, 10000, 65536):
                 S = f(M, N, K)
                 assert S in (1, 2, 4, 8) and K % S == 0 and (S == 1 or (K // S >= 2048 and (K // S) % 8 == 0))
+
+
+def test_row_launch_shape():
+    """Launches with (row, kv head) pairs enough to fill the chip take a pair whole in one workgroup, with about one
+    round of 2,048 waves; fewer pairs are cut into splits that reach past the longest request."""
+    from inferflux_amd.kernels.attention import ROW_MAX_SPLITS, row_launch_shape
+    assert row_launch_shape(64, 4, 4096) == (0, 8, 1)
+    assert row_launch_shape(48, 4, 4096) == (0, 8, 1)
+    assert row_launch_shape(96, 4, 4096) == (0, 4, 1)
+    assert row_launch_shape(128, 4, 4096) == (0, 4, 1)
+    assert row_launch_shape(256, 4, 4096) == (0, 2, 1)
+    assert row_launch_shape(600, 4, 4096) == (0, 1, 1)
+    assert row_launch_shape(64, 4, 4096, max_waves=4) == (0, 4, 1)      # what the kernel's LDS allows at these head counts
+    assert row_launch_shape(64, 2, 4096)[1] == 0                        # 128 pairs: splits
+    for rows, kv_heads, bound in [(1, 4, 4096), (8, 4, 4096), (32, 4, 4096), (1, 1, 131072), (8, 8, 32768), (47, 4, 1024)]:
+        chunk, waves, splits = row_launch_shape(rows, kv_heads, bound)
+        assert waves == 0 and chunk % 32 == 0 and chunk >= 128
+        assert splits * chunk >= bound > (splits - 1) * chunk and splits <= ROW_MAX_SPLITS

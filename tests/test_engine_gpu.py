@@ -196,7 +196,8 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype):
     runner = ModelRunner(model, num_pages=16, max_requests=3)
     assert [g.entries for g in runner.storage.groups] == [(0,)]          # one cache owner; entry 2 reads it
     assert runner.storage.binding(2).writes_cache is False and runner.storage.binding(2).cache is runner.storage.binding(0).cache
-    assert runner.storage.binding(1).state.shape == (3, H) and runner.storage.binding(3).state is not runner.storage.binding(1).state
+    assert runner.storage.binding(1).state.shape == (3 + 1, H)           # (one slot more: for the rows that stand for nobody)
+    assert runner.storage.binding(3).state is not runner.storage.binding(1).state
     ids = seeded_ids(15, 60, V)
     runner.add_request("w")
     whole = runner.step([StepEntry("w", ids, list(range(60)))]).cpu()

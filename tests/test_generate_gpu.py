@@ -232,20 +232,25 @@ def test_logprobs_through_the_engine(model_folders):
     assert engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))[0].logprobs is None
 
 
-def _stateful_toy_runner(pages, slots):
+def _stateful_toy_runner(pages, slots, graph_safe=False, decode_graphs=True):
     """A two-layer model made outside the package: attention, then a mixer that keeps a decayed sum per request in a
-    state slot (no cache).  A state that is not zero when a request starts changes every token after it."""
+    state slot (no cache).  A state that is not zero when a request starts changes every token after it.
+    ``graph_safe``: the mixer takes steps of single tokens with device-side indexing only and says so, which lets
+    the runner capture them."""
     from inferflux_amd.engine.model import Model
     from inferflux_amd.engine.runner import ModelRunner
     from inferflux_amd.parts import LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec, ScheduleEntry, StateSpec, register_part
     from inferflux_amd.parts.base import registered_parts
 
-    H, V, kind = 32, 61, "toy_decay_sum_for_generation"
+    H, V, kind = 32, 61, "toy_decay_sum_for_generation" + ("_in_graphs" if graph_safe else "")
     if kind not in registered_parts("mixer"):
+        from inferflux_amd.kernels import ops
+
         @register_part("mixer", kind)
         class DecaySum(Mixer):
             def __init__(self, name, hidden_size, decay):
                 self.name, self.H, self.decay = name, hidden_size, decay
+                self.graph_safe = graph_safe
             def param_specs(self):
                 return {f"{self.name}.mix.weight": ParamSpec((self.H, self.H), ("normal", 0.3))}
             def load(self, tensors):
@@ -253,6 +258,12 @@ def _stateful_toy_runner(pages, slots):
             def state_spec(self):
                 return StateSpec((self.H,), "float32")
             def forward(self, h, ctx, binding):
+                if self.graph_safe and ctx.n_tokens == ctx.n_requests:
+                    # one token each: the slots come from the step's device array, so a replayed graph follows them
+                    slots = ctx.state_slots.long()
+                    s = binding.state.index_select(0, slots) * self.decay + h.float()
+                    binding.state.index_copy_(0, slots, s)
+                    return ops.gemm_f32(s.to(h.dtype), self.w)
                 out = torch.empty_like(h)
                 for r in range(ctx.n_requests):
                     s = binding.state[int(ctx.h_state_slots[r])]
@@ -277,7 +288,35 @@ def _stateful_toy_runner(pages, slots):
                      final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
                      lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
     model = Model(plan=plan).init_random(4, torch.float32, "cuda")
-    return ModelRunner(model, num_pages=pages, max_requests=slots), V
+    return ModelRunner(model, num_pages=pages, max_requests=slots, decode_graphs=decode_graphs), V
+
+
+def test_a_model_with_state_keeps_padded_decode_graphs():
+    """Six requests with limits of their own, so that the batch shrinks from 6 to 1: the captured steps' batches are
+    filled up to 8, 4, 2 and 1 with rows that use a state slot no request holds, so four layouts serve every size;
+    tokens are those of eager steps, and nothing is started early (a step over state cannot be run twice)."""
+    from inferflux_amd.engine.engine import Engine as Eng
+    from inferflux_amd.engine.scheduler import SchedulerConfig
+    lens, limits = [12, 30, 7, 21, 16, 9], [40, 33, 26, 19, 12, 6]
+
+    def run(**kw):
+        runner, V = _stateful_toy_runner(pages=64, slots=6, graph_safe=True, **kw)
+        eng = Eng(runner, SchedulerConfig(6, 4096, 512))
+        params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in limits]
+        outs = eng.generate([seeded_ids(700 + i, n, V) for i, n in enumerate(lens)], params)
+        runner.manager.check()
+        assert runner.manager.free_pages() == [64]
+        return [o.token_ids for o in outs], runner
+
+    want, eager = run(decode_graphs=False)
+    assert eager.graph_captures == 0 and [len(t) for t in want] == limits
+    got, runner = run()
+    assert runner.model.graph_safe and runner.storage.has_state and not runner.starts_steps_early
+    assert got == want
+    assert 1 <= runner.graph_captures <= 4 and runner.graph_replays >= 30
+    # the rows that stand for nobody wrote to the slot beyond the requests' and to no other
+    state = next(iter(runner.storage._states.values()))
+    assert state.shape[0] == 7 and float(state[6].abs().max()) > 0
 
 
 def test_per_request_state_is_zero_for_every_admission_through_the_engine():
@@ -310,19 +349,29 @@ def test_per_request_state_is_zero_for_every_admission_through_the_engine():
     assert runner.manager.free_pages() == [7]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("early", [True, False])
-def test_requests_added_and_aborted_between_steps_by_hand(early, model_folders):
+def test_requests_added_and_aborted_between_steps_by_hand(early, dtype, model_folders):
     """The engine driven step by step: a request arrives between two decode steps (the step that was started early
     for the others is void), a running request is aborted right after a step that started the next one early (its
     row of that step is dropped), a waiting one is aborted before it ever ran, greedy requests run beside a seeded
-    one.  Survivors' tokens are the plain model's; aborted requests return what they had."""
-    folder, V = model_folders["B"], TINY["B"]["vocab_size"]
+    one.  Survivors' tokens are the plain model's; aborted requests return what they had.  In bfloat16 (configuration A,
+    whose head size the matrix-core kernels take) every token is within rounding of the plain model's best for the
+    prefix it follows."""
+    name = "B" if dtype == "float32" else "A"
+    folder, V = model_folders[name], TINY[name]["vocab_size"]
+    cfg, W = pm.load_folder(folder, torch.float64)
     P = {k: seeded_ids(600 + i, n, V) for i, (k, n) in enumerate({"a": 21, "b": 5, "c": 33, "d": 12, "w": 8, "s": 17, "x": 9}.items())}
     greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)
-    eng = Engine.load(folder, dtype="float32", kv_pages=40, max_batch_size=4, chunked_prefill_tokens=16,
+    eng = Engine.load(folder, dtype=dtype, kv_pages=40, max_batch_size=4, chunked_prefill_tokens=16,
                       start_steps_early=early)
     runner = eng.runner
     done = {}
+
+    def right(rid, tokens, n):
+        if dtype == "bfloat16":
+            return near_best(cfg, W, P[rid], tokens, name)
+        return tokens == plain_greedy(folder, P[rid], n)[:len(tokens)]
 
     def step(n=1):
         for _ in range(n):
@@ -359,27 +408,47 @@ def test_requests_added_and_aborted_between_steps_by_hand(early, model_folders):
     runner.manager.check()
     assert runner.manager.free_pages() == [40] and not runner.manager.live()
     for k, n in (("a", 30), ("c", 10), ("d", 8), ("w", 8)):
-        assert done[k].finish_reason == "length" and done[k].token_ids == plain_greedy(folder, P[k], n), k
-    assert out_b.token_ids == plain_greedy(folder, P["b"], 30)[: len(out_b.token_ids)]
-    # the seeded request alone gives the same tokens: neither the batch nor the arrivals and aborts around it matter
-    alone = Engine.load(folder, dtype="float32", kv_pages=40, max_batch_size=4)
-    assert alone.generate([P["s"]], SamplingParams(temperature=0.9, top_p=0.95, seed=77, max_tokens=12, ignore_eos=True))[0].token_ids \
-        == done["s"].token_ids
+        assert done[k].finish_reason == "length" and len(done[k].token_ids) == n and right(k, done[k].token_ids, n), k
+    assert right("b", out_b.token_ids, 30)
+    if dtype == "float32":
+        # the seeded request alone gives the same tokens: neither the batch nor the arrivals and aborts around it matter
+        alone = Engine.load(folder, dtype="float32", kv_pages=40, max_batch_size=4)
+        assert alone.generate([P["s"]], SamplingParams(temperature=0.9, top_p=0.95, seed=77, max_tokens=12, ignore_eos=True))[0].token_ids \
+            == done["s"].token_ids
 
 
+def near_best(cfg, W, prompt, tokens, name):
+    """Whether every token of ``tokens`` is, for the prefix before it, within rounding of the plain model's best
+    token: its logit at most twice the bfloat16 bound of the configuration below the largest one.  (Among the
+    hundreds of a tiny vocabulary one to three tokens are; the logits of a wrong prefix, page or position put their
+    own best there with a chance of well under a hundredth.)"""
+    from conftest import tol
+    if not tokens:
+        return True
+    full = pm.forward(cfg, W, list(prompt) + list(tokens))
+    for i, tok in enumerate(tokens):
+        row = full[len(prompt) - 1 + i]
+        if row[tok] < row.max() - 2 * tol("bfloat16", name) * row.abs().max():
+            return False
+    return True
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("early", [True, False], ids=["early", "late"])
 @pytest.mark.parametrize("name,seed", [("C", 2), ("A", 3)])
-def test_random_arrivals_aborts_priorities_and_preemptions(name, seed, early, model_folders):
+def test_random_arrivals_aborts_priorities_and_preemptions(name, seed, early, dtype, model_folders):
     """Forty requests of random lengths, limits and priorities arrive at random steps and some are aborted at random,
-    through a cache too small for them (requests are preempted and recomputed).  Every finished request's tokens are
-    the plain model's, every aborted one's a beginning of them, the cache's books are right after every step and
-    every pool is whole at the end."""
+    through a cache too small for them (requests are preempted and recomputed).  In float32 every finished request's
+    tokens are the plain model's and every aborted one's a beginning of them; in bfloat16 (the matrix-core kernels,
+    decode steps as replayed graphs with their batches filled up, steps started early and made void) every token is
+    within rounding of the plain model's best for the prefix it follows.  The cache's books are right after every
+    step and every pool is whole at the end."""
     import random
     folder, V = model_folders[name], TINY[name]["vocab_size"]
     cfg, W = pm.load_folder(folder, torch.float64)
     rng = random.Random(seed * 7 + (1 if early else 0))
     pages = rng.randint(14, 22)
-    eng = Engine.load(folder, dtype="float32", kv_pages=pages, max_batch_size=rng.randint(3, 6),
+    eng = Engine.load(folder, dtype=dtype, kv_pages=pages, max_batch_size=rng.randint(3, 6),
                       chunked_prefill_tokens=rng.choice([8, 16, 24, 48]), max_batch_tokens=rng.choice([32, 64, 256]),
                       start_steps_early=early)
     reqs, done, aborted = {}, {}, {}
@@ -407,9 +476,47 @@ def test_random_arrivals_aborts_priorities_and_preemptions(name, seed, early, mo
     assert eng.runner.manager.free_pages() == [pages] * len(eng.runner.manager.groups) and not eng.runner.manager.live()
     assert set(done) | set(aborted) == set(reqs) and not set(done) & set(aborted)
     assert eng.stats.preemptions > 0 and aborted and len(done) > 10          # the run did meet what it is about
+    if dtype == "bfloat16":
+        assert eng.runner.decode_graphs and eng.runner.graph_replays > 20
     for rid, (prompt, n_new) in reqs.items():
+        out = done.get(rid) or aborted[rid]
+        assert out.finish_reason == ("length" if rid in done else "abort") and len(out.token_ids) <= n_new
+        assert rid in aborted or len(out.token_ids) == n_new
+        if dtype == "bfloat16":
+            assert near_best(cfg, W, prompt, out.token_ids, name), (rid, out.token_ids)
+            continue
         want = pm.greedy_generate(cfg, W, prompt, n_new)
-        if rid in done:
-            assert done[rid].finish_reason == "length" and done[rid].token_ids == want, rid
-        else:
-            assert aborted[rid].finish_reason == "abort" and aborted[rid].token_ids == want[:len(aborted[rid].token_ids)], rid
+        assert out.token_ids == want[:len(out.token_ids)], rid
+
+
+def test_a_seeded_request_with_penalties_keeps_its_tokens_across_a_preemption(model_folders):
+    """A request that samples (temperature 0.9, a seed, a repetition penalty and a frequency penalty) is preempted and
+    recomputed in a pool too small for the three that run: its draw counter and the history its penalties read
+    outlive the preemption, so its tokens are those of the same request in a roomy pool (float32: the logits of a
+    position are the same bits however it was reached).  The invariant of the reference's sampler test, extended
+    over a preemption (tests/unit/test_gpu_sampler.cpp:205-262)."""
+    folder, V = model_folders["A"], TINY["A"]["vocab_size"]
+    prompts = [seeded_ids(820 + i, 40, V) for i in range(3)]
+
+    def params():
+        return [SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True),
+                SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True),
+                SamplingParams(temperature=0.9, seed=4711, repetition_penalty=1.3, frequency_penalty=0.2, penalty_last_n=16,
+                               max_tokens=40, ignore_eos=True)]
+
+    def run(pages):
+        eng = Engine.load(folder, dtype="float32", kv_pages=pages, max_batch_size=4)
+        ids = [eng.add_request(p, sp, priority=pr) for p, sp, pr in zip(prompts, params(), (1, 1, 0))]   # the sampler goes first
+        outs = {}
+        while eng.has_unfinished():
+            for o in eng.step():
+                outs[o.request_id] = o
+        eng.runner.manager.check()
+        assert eng.runner.manager.free_pages() == [pages]
+        return [outs[i] for i in ids]
+
+    roomy, tight = run(64), run(8)                             # 15 pages would be needed
+    assert roomy[2].preemptions == 0 and tight[2].preemptions >= 1
+    assert [o.token_ids for o in tight] == [o.token_ids for o in roomy]
+    alone = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=4).generate([prompts[2]], [params()[2]])[0]
+    assert alone.token_ids == roomy[2].token_ids and len(set(alone.token_ids)) > 8

@@ -523,30 +523,45 @@ MFMA_CASES = [c for c in ATTN_CASES if c[4] % 16 == 0 and c[4] <= 128] + [
 ]
 
 
-def run_rows(q, kc, vc, row_req, positions, table, window, scale, rows=None, chunk=128):
+def run_rows(q, kc, vc, row_req, positions, table, window, scale, rows=None, chunk=128, waves=0, extra_splits=0):
+    """``waves`` 0: one wave per split of ``chunk`` keys and the merge launch (``extra_splits``: the grid reaches that
+    many splits past the longest row, as a captured step's does); 1-8: one workgroup of that many waves per (row, kv head)."""
     T, nH, d = q.shape
     out = torch.zeros(T, nH * d, dtype=q.dtype, device=DEV)
     n = T if rows is None else rows.shape[0]
     max_kv = int(positions.max()) + 1
-    ops.attention_rows(q, kc, vc, out, rows, n, row_req, positions, table, window, scale, chunk, -(-max_kv // chunk))
+    ops.attention_rows(q, kc, vc, out, rows, n, row_req, positions, table, window, scale, chunk,
+                       -(-max_kv // chunk) + extra_splits, waves)
     return out
 
 
-@pytest.mark.parametrize("chunk", [32, 128])
+def close_rows(out, want):
+    """Row attention against float64: element by element, and the largest error against the largest value (a bound
+    that follows the data: outputs here are 0.1-1 in size)."""
+    return torch.allclose(out, want, rtol=1e-2, atol=1e-2) and float((out - want).abs().max()) <= 1e-2 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("chunk,waves", [(32, 0), (128, 0), (1024, 0), (128, 1), (128, 2), (128, 3), (128, 4), (128, 8)])
 @pytest.mark.parametrize("case", MFMA_CASES)
-def test_attention_rows(case, chunk):
+def test_attention_rows(case, chunk, waves):
+    """Every launch shape of the row kernel: one wave per split and the merge launch, and one workgroup of several
+    waves per (row, kv head) whose waves share the row's keys and meet in LDS."""
     lens_q, lens_past, nH, nKV, d, P, window, sharp = case
     (q, kc, vc, row_req, positions, table), want, _ = paged_case(7, lens_q, lens_past, nH, nKV, d, P, BF16, window, sharp=sharp)
-    out = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), chunk=chunk).cpu().double()
+    waves = ops.row_waves_fit(nH, nKV, d, waves)
+    out = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), chunk=chunk, waves=waves)
     assert torch.isfinite(out).all()
-    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
+    assert close_rows(out.cpu().double(), want), float((out.cpu().double() - want).abs().max())
+    # the same launch again, with a grid that reaches past the longest row: the same bits
+    again = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), chunk=chunk, waves=waves, extra_splits=3)
+    assert torch.equal(again, out)
 
 
 @pytest.mark.parametrize("seed", range(30))
 def test_attention_rows_random_cases(seed):
-    """The row kernel and its merge at shapes drawn at random: one to five requests of 1-15 rows behind pasts of
-    0-2,500 keys, head sizes 16-128, pages of 16-256, with and without a window, 1-20 query heads to a kv head,
-    splits of 32-1,024 keys, all rows or a subset; against float64."""
+    """The row kernels at shapes drawn at random: one to five requests of 1-15 rows behind pasts of 0-2,500 keys, head
+    sizes 16-128, pages of 16-256, with and without a window, 1-20 query heads to a kv head, splits of 32-1,024 keys
+    with the merge launch or workgroups of 1-8 waves that take a row whole, all rows or a subset; against float64."""
     import random
     rng = random.Random(500 + seed)
     d = rng.choice([16, 32, 64, 128])
@@ -558,17 +573,19 @@ def test_attention_rows_random_cases(seed):
     lens_past = [rng.choice([0, rng.randint(1, 200), rng.randint(200, 2500)]) for _ in range(n_req)]
     window = rng.choice([None, None, rng.randint(5, 900)])
     chunk = rng.choice([32, 64, 128, 256, 1024])
+    waves = ops.row_waves_fit(nH, nKV, d, rng.choice([1, 2, 4, 5, 8])) if seed % 2 else 0
     (q, kc, vc, row_req, positions, table), want, _ = paged_case(600 + seed, lens_q, lens_past, nH, nKV, d, P, BF16, window,
                                                                  sharp=rng.choice([None, 2, -50]))
     T = q.shape[0]
     rows = None
     if rng.random() < 0.4 and T > 1:
         rows = torch.tensor(sorted(rng.sample(range(T), rng.randint(1, T - 1))), dtype=torch.int32, device=DEV)
-    out = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), rows=rows, chunk=chunk).cpu().double()
+    out = run_rows(q, kc, vc, row_req, positions, table, window, 1.0 / math.sqrt(d), rows=rows, chunk=chunk, waves=waves,
+                   extra_splits=seed % 3).cpu().double()
     sel = list(range(T)) if rows is None else rows.cpu().tolist()
     assert torch.isfinite(out).all()
-    assert torch.allclose(out[sel], want[sel], rtol=1e-2, atol=1e-2), (seed, d, P, nH, nKV, lens_q, lens_past, window, chunk,
-                                                                      float((out[sel] - want[sel]).abs().max()))
+    assert close_rows(out[sel], want[sel]), (seed, d, P, nH, nKV, lens_q, lens_past, window, chunk, waves,
+                                             float((out[sel] - want[sel]).abs().max()))
     rest = [i for i in range(T) if i not in sel]
     assert torch.all(out[rest] == 0)
 
@@ -692,6 +709,15 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     z = torch.zeros(1, dtype=torch.int32, device=DEV)
     with pytest.raises(ops.KernelError, match="head_dim"):
         ops.attention_rows(q, kc, vc, torch.zeros(1, 48, dtype=BF16, device=DEV), None, 1, z, z, z.view(1, 1), None, 1.0, 128, 1)
+    q = torch.zeros(1, 2, 32, dtype=BF16, device=DEV)
+    kc, vc = torch.zeros(2, 1, 16, 32, dtype=BF16, device=DEV), torch.zeros(2, 1, 32, 16, dtype=BF16, device=DEV)
+    with pytest.raises(ops.KernelError, match="waves per workgroup"):
+        ops.attention_rows(q, kc, vc, torch.zeros(1, 64, dtype=BF16, device=DEV), None, 1, z, z, z.view(1, 1), None, 1.0, 128, 1, waves=9)
+    q = torch.zeros(1, 32, 128, dtype=BF16, device=DEV)           # 16 heads of 128 per pass: eight waves' results exceed the LDS
+    kc, vc = torch.zeros(2, 1, 16, 128, dtype=BF16, device=DEV), torch.zeros(2, 1, 128, 16, dtype=BF16, device=DEV)
+    assert ops.row_waves_fit(32, 1, 128, 8) == 4
+    with pytest.raises(ops.KernelError, match="waves per workgroup"):
+        ops.attention_rows(q, kc, vc, torch.zeros(1, 4096, dtype=BF16, device=DEV), None, 1, z, z, z.view(1, 1), None, 1.0, 128, 1, waves=8)
 
 
 # ---- weight-streaming matrix product ---------------------------------------------------------

@@ -189,6 +189,19 @@ def test_only_distances_count(name):
     assert not torch.allclose(pm.forward(cfg, W, ids, positions=range(0, 60, 2)), base, atol=1e-6)
 
 
+@pytest.mark.parametrize("name", list(TINY))
+def test_rows_of_a_one_layer_model_equal_the_whole_forward(name):
+    """The oracle for long sequences at real widths computes everything but keys and values for the wanted rows alone:
+    the same logits as the whole forward, with C's window (on its only layer) and without."""
+    cfg = dict(TINY[name], num_hidden_layers=1, max_window_layers=0)
+    W = random_weights(cfg, 3)
+    ids = [(7 * i + 3) % cfg["vocab_size"] for i in range(50)]
+    rows = [0, 1, 23, 24, 25, 48, 49]
+    assert torch.allclose(pm.forward_rows_one_layer(cfg, W, ids, rows), pm.forward(cfg, W, ids)[rows], atol=1e-12)
+    with pytest.raises(ValueError):
+        pm.forward_rows_one_layer(TINY[name], random_weights(TINY[name]), ids, rows)
+
+
 def test_window_changes_only_windowed_layers_reach():
     cfg = TINY["C"]
     W = random_weights(cfg, 2)

@@ -212,6 +212,33 @@ def test_the_score_hook_is_the_references_priority_plus_age():
     assert [i.seq.rid for i in s2.schedule().items] == ["new"]  # one second of age does not outweigh a priority step
 
 
+def test_a_stream_of_more_important_arrivals_does_not_starve_a_waiting_request():
+    """One place in the batch, a request of priority 0 waiting, and a request of priority 1 arriving every half
+    second: under the default score the old request's age outgrows the newcomers' priority after two seconds and it
+    is admitted; under the priority alone it waits as long as the stream lasts."""
+    from inferflux_amd.engine.scheduler import priority_score
+
+    def admitted_after(score):
+        now = [0.0]
+        m = CacheManager([GroupSpec(None, (0,))], 16, 64, 8)
+        s = Scheduler(m, SchedulerConfig(max_batch_size=1), 4096, score=score, clock=lambda: now[0])
+        s.add("first", [1, 2], 1, priority=1)
+        s.add("patient", [3, 4], 1)
+        for tick in range(1, 41):
+            plan = s.schedule()
+            assert len(plan.items) == 1
+            if plan.items[0].seq.rid == "patient":
+                return tick
+            it = plan.items[0]
+            m.commit(it.seq.rid, len(it.tokens)); s.advance(it); s.finish(it.seq)     # a request takes one step
+            now[0] += 0.5
+            s.add(f"vip{tick}", [5, 6], 1, priority=1)
+        return None
+
+    assert admitted_after(None) is not None and admitted_after(None) <= 8       # about 2 s / 0.5 s, and a few ticks
+    assert admitted_after(priority_score) is None
+
+
 def test_the_victim_is_the_lowest_priority_then_the_youngest():
     m, s = make(pages=4, page_size=16)
     a = s.add("a", list(range(30)), 30)                         # oldest, priority 0
