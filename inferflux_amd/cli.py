@@ -59,7 +59,7 @@ def load_spec_from_args(args):
         return ModelLoadSpec(path=args.model, random_weights=args.random_weights, seed=args.seed, dtype=args.dtype,
                              device=args.device, context_size=args.ctx_size, max_parallel_sequences=args.max_parallel_sequences,
                              kv_pages=args.kv_pages, page_size=args.page_size, max_batch_tokens=args.batch_size,
-                             chunked_prefill_tokens=args.chunked_prefill_tokens,
+                             chunked_prefill_tokens=args.chunked_prefill_tokens, prefill_tokens_alone=args.prefill_tokens_alone,
                              decode_weight_copy=not args.no_decode_weight_copy,
                              strict_weights=not args.allow_unused_tensors, phase_timing=args.phase_timing,
                              library_gemm_tuning=args.gemm_tuning).checked()
@@ -156,7 +156,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     c.add_argument("--ctx-size", type=int, default=4096, help="tokens of context per sequence the cache is sized for")
     c.add_argument("--batch-size", type=int, default=16384, help="most tokens in one step (max_batch_tokens)")
     c.add_argument("--max-parallel-sequences", type=int, default=32, help="most requests in one step (max_batch_size)")
-    c.add_argument("--chunked-prefill-tokens", type=int, default=512)
+    c.add_argument("--chunked-prefill-tokens", type=int, default=512,
+                   help="largest portion of a prompt in a step beside requests that are decoding")
+    c.add_argument("--prefill-tokens-alone", type=int, default=None,
+                   help="largest portion in a step in which nobody decodes (default: 2048, or --chunked-prefill-tokens if that is more)")
     c.add_argument("--kv-pages", type=int, default=None, help="pages in the cache (overrides --ctx-size)")
     c.add_argument("--page-size", type=int, default=16, help="tokens per page of the cache")
     c.add_argument("--device", default=None, help="rocm:N or cuda:N (the same ordinal); default: the current device")

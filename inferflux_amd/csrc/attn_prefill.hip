@@ -100,11 +100,15 @@ __device__ __forceinline__ void direct_load(unsigned long long base, int bytes, 
                : "memory", "m0");
 }
 
-// Wait until at most N of this wave's vector memory loads are still in flight, then meet the other waves.
+// Wait until at most N of this wave's vector memory loads are still in flight and none of its LDS reads is, then
+// meet the other waves.  The barrier says two things at once: "my loads of this tile have landed" (vmcnt) and "I
+// have read everything I will of the tile before" (lgkmcnt: right behind the barrier other waves start loads into
+// that tile's stage, so every LDS read of it must have returned, not merely have been issued; a tile's operands have
+// all been consumed by matrix instructions by then, so this wait costs nothing).
 template <int N>
 __device__ __forceinline__ void wait_loads_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(N) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
 
 struct QueryTile {

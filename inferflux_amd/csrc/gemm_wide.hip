@@ -48,6 +48,22 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+__device__ __forceinline__ void store4(float* p, floatx4 v) { *(floatx4*)p = v; }
+__device__ __forceinline__ void store4(bf16_t* p, floatx4 v) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+  bf16x4 w;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) w[r] = (__bf16)v[r];
+  *(bf16x4*)p = w;
+}
+__device__ __forceinline__ void store2(float* p, float a, float b) { *(float2*)p = float2{a, b}; }
+__device__ __forceinline__ void store2(bf16_t* p, float a, float b) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+  bf16x2 w;
+  w[0] = (__bf16)a; w[1] = (__bf16)b;
+  *(bf16x2*)p = w;
+}
+
 // EPI 0: out[m, n] = sum.  EPI 1: the rows of W alternate gate, up, ...: out[m, n / 2] = silu(gate) * up.
 // ``order``: tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
 template <int MT, typename TO, int EPI>
@@ -134,23 +150,46 @@ __global__ __launch_bounds__((16 * MT > MANY_ROWS ? MIN_WAVES : MAX_WAVES) * WAV
   // acc[mt][r] = out[m = 16 mt + col][n = tile_rows (row tile of the weight) + 4 g + r], for 4 g + r < tile_rows
   const int n0 = tile_rows * (order ? order[tile] : tile) + 4 * g;
   const int held = min(4, tile_rows - 4 * g);      // how many of the lane's four rows the tile holds (even, may be <= 0)
+  // A lane's four sums are four consecutive columns of one output row.  Where the tile holds all four and rows start at
+  // multiples of four columns they go out as one store (16 bytes of float, 8 of bf16) instead of four: the head's
+  // 39 MB of logits at 64 rows otherwise arrive as 4-byte pieces 600 KB apart.
+  const bool whole = held == 4 && n0 + 3 < N && ((N | n0) & 3) == 0;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + col;
     if (m >= M) continue;
     if (gridDim.y > 1) {
+      float* dst = part + ((size_t)blockIdx.y * M + m) * N + n0;
+      if (whole) {
+        *(floatx4*)dst = acc[mt];
+      } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (r < held && n0 + r < N) part[((size_t)blockIdx.y * M + m) * N + n0 + r] = acc[mt][r];
+        for (int r = 0; r < 4; ++r)
+          if (r < held && n0 + r < N) dst[r] = acc[mt][r];
+      }
     } else if (EPI == 0) {
+      TO* dst = out + (size_t)m * N + n0;
+      if (whole) {
+        store4(dst, acc[mt]);
+      } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (r < held && n0 + r < N) out[(size_t)m * N + n0 + r] = from_f<TO>(acc[mt][r]);
+        for (int r = 0; r < 4; ++r)
+          if (r < held && n0 + r < N) dst[r] = from_f<TO>(acc[mt][r]);
+      }
     } else {
+      TO* dst = out + (size_t)m * (N / 2) + n0 / 2;
+      float v[2];
 #pragma unroll
       for (int r = 0; r < 4; r += 2) {   // even: gate at n0 + r, up at n0 + r + 1
         const float gt = acc[mt][r], up = acc[mt][r + 1];
-        if (r < held && n0 + r + 1 < N) out[(size_t)m * (N / 2) + (n0 + r) / 2] = from_f<TO>(gt / (1.0f + expf(-gt)) * up);
+        v[r / 2] = gt / (1.0f + expf(-gt)) * up;
+      }
+      if (whole) {
+        store2(dst, v[0], v[1]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; r += 2)
+          if (r < held && n0 + r + 1 < N) dst[r / 2] = from_f<TO>(v[r / 2]);
       }
     }
   }

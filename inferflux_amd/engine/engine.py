@@ -73,23 +73,26 @@ class Engine:
     def load(cls, model, dtype: str = "bfloat16", kv_pages: Optional[int] = None, page_size: int = 16,
              max_batch_size: int = 32, max_batch_tokens: int = 16384, chunked_prefill_tokens: int = 512,
              ctx_size: int = 4096, phase_timing: bool = False, decode_weight_copy: bool = True,
-             start_steps_early: bool = True, library_gemm_tuning: bool = False) -> "Engine":
+             start_steps_early: bool = True, library_gemm_tuning: bool = False,
+             prefill_tokens_alone: Optional[int] = None) -> "Engine":
         """``model`` is a ``ModelLoadSpec``, or a model folder with the other arguments standing for the spec's
         fields (``max_batch_size`` = max_parallel_sequences, ``ctx_size`` = context_size).  ``kv_pages`` None sizes
         the cache for ``ctx_size`` tokens for each of ``max_batch_size`` requests, within the device memory that is
         free once the weights are loaded.  ``decode_weight_copy`` False saves the second, tiled copy of the weights
-        at the price of slower decoding.  ``library_gemm_tuning`` lets the library time its kernels for the product shapes
+        at the price of slower decoding.  ``prefill_tokens_alone``: the largest portion of a prompt in a step in which
+        nobody decodes (None: 2,048, or ``chunked_prefill_tokens`` if that is more).  ``library_gemm_tuning`` lets the library time its kernels for the product shapes
         of prompts (see ``ops.enable_library_gemm_tuning``)."""
         spec = model if isinstance(model, ModelLoadSpec) else ModelLoadSpec(
             path=model, dtype=dtype, kv_pages=kv_pages, page_size=page_size, max_parallel_sequences=max_batch_size,
             max_batch_tokens=max_batch_tokens, chunked_prefill_tokens=chunked_prefill_tokens, context_size=ctx_size,
-            phase_timing=phase_timing, decode_weight_copy=decode_weight_copy, library_gemm_tuning=library_gemm_tuning)
+            phase_timing=phase_timing, decode_weight_copy=decode_weight_copy, library_gemm_tuning=library_gemm_tuning,
+            prefill_tokens_alone=prefill_tokens_alone)
         runner = load_runner(spec.checked())
         log.info("engine", "model loaded", model=spec.path or spec.random_weights, dtype=spec.dtype,
                  kv_pages=runner.manager.pools[0].num_pages if runner.manager.pools else 0, page_size=spec.page_size,
                  max_batch_size=spec.max_parallel_sequences)
-        return cls(runner, SchedulerConfig(spec.max_parallel_sequences, spec.max_batch_tokens, spec.chunked_prefill_tokens),
-                   start_steps_early)
+        return cls(runner, SchedulerConfig(spec.max_parallel_sequences, spec.max_batch_tokens, spec.chunked_prefill_tokens,
+                                           spec.prefill_tokens_alone), start_steps_early)
 
     # ---- requests -----------------------------------------------------------------
     def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,

@@ -35,7 +35,8 @@ class ModelLoadSpec:
     kv_pages: Optional[int] = None          # pages per cache group; None: context_size * max_parallel_sequences tokens
     page_size: int = 16                     # tokens per page
     max_batch_tokens: int = 16384           # tokens in one step
-    chunked_prefill_tokens: int = 512       # largest portion of a prompt in one step
+    chunked_prefill_tokens: int = 512       # largest portion of a prompt in one step beside requests that are decoding
+    prefill_tokens_alone: Optional[int] = None   # ... in a step in which nobody decodes (None: the larger of that and 2,048)
     decode_weight_copy: bool = True         # keep the tiled second copy of bfloat16 projections for decoding
     strict_weights: bool = True             # tensors in the file that no part reads are an error (else a warning)
     phase_timing: bool = False              # time every phase of every forward pass
@@ -62,6 +63,8 @@ class ModelLoadSpec:
             return "max_batch_tokens must be positive"
         if self.chunked_prefill_tokens <= 0:
             return "chunked_prefill_tokens must be positive"
+        if self.prefill_tokens_alone is not None and self.prefill_tokens_alone <= 0:
+            return "prefill_tokens_alone must be positive"
         if self.seed < 0:
             return "seed must be nonnegative"
         return ""

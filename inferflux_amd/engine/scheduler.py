@@ -3,7 +3,8 @@ decides, the engine executes.
 
 Every step the running set is formed anew: each running request that is decoding contributes one
 token, the rest of the budget is dealt to prompts as portions of at most
-``chunked_prefill_tokens``, and waiting requests are admitted first come first served while a
+``chunked_prefill_tokens`` (of ``prefill_tokens_alone``, 2,048 by default, in a step in which nobody
+decodes and so nobody waits for the prompts), and waiting requests are admitted first come first served while a
 place in the batch, budget and pages for their first portion are there.  Only the last portion
 of a prompt asks for logits.
 
@@ -44,11 +45,27 @@ from ..cache.manager import CacheManager, OutOfPages
 class SchedulerConfig:
     max_batch_size: int = 32           # requests in a step (the reference caps this at 64)
     max_batch_tokens: int = 16384      # tokens in a step
-    chunked_prefill_tokens: int = 512  # largest portion of a prompt in a step
+    chunked_prefill_tokens: int = 512  # largest portion of a prompt in a step beside requests that are decoding
+    # Largest portion in a step in which nobody decodes (None: the larger of chunked_prefill_tokens and 2,048).  Portions are
+    # short so that decoding requests do not wait long for a prompt; while there are none, nobody waits, and the matrix
+    # products of 2,048 rows run at 0.43 of the chip's peak where those of 512 run at 0.27.
+    prefill_tokens_alone: Optional[int] = None
+
+    PREFILL_ALONE = 2048
 
     def validate(self) -> None:
         if self.max_batch_size < 1 or self.max_batch_tokens < 1 or self.chunked_prefill_tokens < 1:
             raise ValueError("scheduler limits must be positive")
+        if self.prefill_tokens_alone is not None and self.prefill_tokens_alone < 1:
+            raise ValueError("prefill_tokens_alone must be positive (or None)")
+
+    @property
+    def portion_alone(self) -> int:
+        return self.prefill_tokens_alone if self.prefill_tokens_alone is not None else max(self.chunked_prefill_tokens, self.PREFILL_ALONE)
+
+    @property
+    def largest_portion(self) -> int:
+        return max(self.chunked_prefill_tokens, self.portion_alone)
 
 
 class RequestRefused(ValueError):
@@ -144,7 +161,7 @@ class Scheduler:
             window = self.manager.groups[g].window
             if window is not None:   # a windowed group holds at most the window, a portion and two partial pages
                 P = self.manager.page_size
-                k = min(k, -(-(window + self.config.chunked_prefill_tokens) // P) + 2)
+                k = min(k, -(-(window + self.config.largest_portion) // P) + 2)
             if k > pool.num_pages:
                 raise RequestRefused(f"request {rid!r} can never fit: {k} pages needed in cache group {g}, the pool has {pool.num_pages}")
         seq = Sequence_(rid, prompt, max_new, arrival=self._arrivals, n_prompt_original=len(prompt),
@@ -200,13 +217,15 @@ class Scheduler:
         cfg = self.config
         plan = StepPlan([], [], [])
         budget = cfg.max_batch_tokens
+        # portions are short for the sake of requests that decode beside them; with none, they may be long
+        portion = cfg.chunked_prefill_tokens if any(not q.is_prefilling for q in self.running) else cfg.portion_alone
         # 1. running requests, oldest admission first (the list is kept in that order: admissions are appended,
         #    preemptions taken out): decodes cost one token, prompts a portion
         for seq in list(self.running):
             if budget <= 0 or (plan.preempted and seq not in self.running):   # nothing left to deal / preempted meanwhile
                 continue
             if seq.is_prefilling:
-                n = min(len(seq.prompt) - seq.computed, cfg.chunked_prefill_tokens, budget)
+                n = min(len(seq.prompt) - seq.computed, portion, budget)
                 toks = seq.prompt[seq.computed: seq.computed + n]
                 wants = seq.computed + n == len(seq.prompt)
             else:
@@ -223,7 +242,7 @@ class Scheduler:
             seq = min(self.waiting, key=lambda q: (-self.score(q, now), q.arrival))
             if seq.rid in plan.preempted:
                 break
-            n = min(len(seq.prompt), cfg.chunked_prefill_tokens, budget)
+            n = min(len(seq.prompt), portion, budget)
             need = self.manager.pages_needed_fresh(n)
             if any(k > f for k, f in zip(need, self.manager.free_pages())) or self.manager.free_slots() == 0:
                 break

@@ -44,16 +44,24 @@ def linear(x, w, b=None):
     return y if b is None else y + b
 
 
-def rope_split_half(x, positions, theta):
+def rope_split_half(x, positions, theta, angle_dtype=None):
     """x [S, heads, d]; pair p joins elements p and p + d/2; f_p = 1 / theta^(2p/d);
     (x0, x1) <- (x0 cos a - x1 sin a, x0 sin a + x1 cos a) with a = position * f_p.
     runtime/backends/cuda/native/cuda_kernels.cu:71-117 (pairing 102-105); the same oracle as
-    tests/unit/test_native_forward.cpp:71-106 with rope_type 2."""
+    tests/unit/test_native_forward.cpp:71-106 with rope_type 2.
+
+    ``angle_dtype`` torch.float32: the angle is the 32-bit product of the position and the frequency rounded to 32
+    bits, as the reference forms it (float freq, float angle: cuda_kernels.cu:91-96); its cosine and sine are then
+    taken in x's type.  At positions beyond ten thousand that rounding (up to 1e-3 rad on the fast pairs) is part of
+    the function a 32-bit implementation computes; without it (the default) the angle is exact in x's type."""
     S, h, d = x.shape
     half = d // 2
     p = torch.arange(half, dtype=x.dtype)
     freq = 1.0 / torch.pow(torch.tensor(theta, dtype=x.dtype), 2.0 * p / d)
-    ang = torch.as_tensor(positions, dtype=x.dtype)[:, None] * freq[None, :]  # [S, half]
+    if angle_dtype is not None:
+        ang = (torch.as_tensor(positions).to(angle_dtype)[:, None] * freq.to(angle_dtype)[None, :]).to(x.dtype)
+    else:
+        ang = torch.as_tensor(positions, dtype=x.dtype)[:, None] * freq[None, :]  # [S, half]
     cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
     x0, x1 = x[..., :half], x[..., half:]
     return torch.cat([x0 * cos - x1 * sin, x0 * sin + x1 * cos], dim=-1)
@@ -162,11 +170,11 @@ def forward(cfg, W, ids, positions=None):
     return linear(h, head)
 
 
-def forward_rows_one_layer(cfg, W, ids, rows):
+def forward_rows_one_layer(cfg, W, ids, rows, angle_dtype=None):
     """Logits [len(rows), V] at the places ``rows`` of a whole sequence, for a model of ONE layer: keys and values need
     the first norm and two projections of every token, everything else is computed for the wanted rows alone, which
     makes sequences of tens of thousands of tokens at real layer widths affordable on the CPU.  The same functions in
-    the same order as ``forward`` (a test compares the two)."""
+    the same order as ``forward`` (a test compares the two).  ``angle_dtype``: see ``rope_split_half``."""
     if cfg["num_hidden_layers"] != 1:
         raise ValueError("forward_rows_one_layer: the second layer's keys would need every row of the first")
     S, rows = len(ids), list(rows)
@@ -178,9 +186,10 @@ def forward_rows_one_layer(cfg, W, ids, rows):
     p, a = "model.layers.0", "model.layers.0.self_attn"
     x = embedding(ids, W["model.embed_tokens.weight"])
     h = rms_norm(x, W[f"{p}.input_layernorm.weight"], eps)
-    k = rope_split_half(linear(h, W[f"{a}.k_proj.weight"], W.get(f"{a}.k_proj.bias")).view(S, nKV, d), positions, theta)
+    k = rope_split_half(linear(h, W[f"{a}.k_proj.weight"], W.get(f"{a}.k_proj.bias")).view(S, nKV, d), positions, theta, angle_dtype)
     v = linear(h, W[f"{a}.v_proj.weight"], W.get(f"{a}.v_proj.bias")).view(S, nKV, d)
-    q = rope_split_half(linear(h[rows], W[f"{a}.q_proj.weight"], W.get(f"{a}.q_proj.bias")).view(len(rows), nH, d), rows, theta)
+    q = rope_split_half(linear(h[rows], W[f"{a}.q_proj.weight"], W.get(f"{a}.q_proj.bias")).view(len(rows), nH, d), rows, theta,
+                        angle_dtype)
     o = attention(q, k, v, window=layer_window(cfg, 0), q_positions=rows, k_positions=positions)
     xr = x[rows] + linear(o.reshape(len(rows), nH * d), W[f"{a}.o_proj.weight"])
     hr = rms_norm(xr, W[f"{p}.post_attention_layernorm.weight"], eps)

@@ -156,8 +156,11 @@ def _write_family_folder(folder, name, max_position=4096, distances=None):
         t[f"{p}.self_attn.q_proj.weight"] = normal(nH * d, H, std=0.005)
         t[f"{p}.self_attn.k_proj.weight"] = normal(nKV * d, H, std=0.005)
         phase = torch.rand(nKV, d // 2, generator=gq, dtype=torch.float64) * 6.283185307179586
-        w = 2.0 * torch.cat([torch.cos(phase), torch.sin(phase)], dim=1)                 # [nKV, d]: every pair of length 2
-        bq = torch.stack([6.0 * _rotate_pairs(w[h // (nH // nKV)], -float(distances[h]), cfg["rope_theta"]) for h in range(nH)])
+        # pair p has length 4 * 0.8^(p/2): the fast pairs, which tell neighbouring positions apart, weigh most, and the
+        # score's peak (about 50) stands 9 above every other key up to 33,000 positions away
+        length = 4.0 * torch.pow(torch.tensor(0.8, dtype=torch.float64), torch.arange(d // 2, dtype=torch.float64) / 2)
+        w = torch.cat([length * torch.cos(phase), length * torch.sin(phase)], dim=1)     # [nKV, d]
+        bq = torch.stack([7.0 * _rotate_pairs(w[h // (nH // nKV)], -float(distances[h]), cfg["rope_theta"]) for h in range(nH)])
         t[f"{p}.self_attn.k_proj.bias"] = w.reshape(-1).to(torch.bfloat16)
         t[f"{p}.self_attn.q_proj.bias"] = bq.reshape(-1).to(torch.bfloat16)
     os.makedirs(folder, exist_ok=True)
@@ -168,33 +171,53 @@ def _write_family_folder(folder, name, max_position=4096, distances=None):
 
 
 # One distance per query head of the 7B shape (28): page edges (15-17), the row kernel's splits (127-129), portions of
-# 2,048, and keys ten and thirty thousand positions back; a head whose distance reaches past the start looks at position 0.
-FAR_DISTANCES = [0, 1, 2, 15, 16, 17, 31, 63, 64, 127, 128, 129, 255, 256, 511, 1023, 1024, 2047, 2048, 2049, 3000, 4095, 4096,
-                 8191, 8192, 12345, 16383, 30000]
-NEAR_DISTANCES = [0, 1, 2, 3, 5, 8, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300, 400, 511, 600]
+# 2,048, and keys tens of thousands of positions back.  A row that cannot reach a head's distance spreads that head's
+# attention over keys whose scores nearly tie, where float32's rounding of the rotation angles alone moves the logits
+# by 5e-4: every list is for rows that reach all of its distances.
+DISTANCES = {
+    "near": [0, 1, 2, 3, 5, 8, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 79, 80, 95, 96, 100, 111, 127, 128, 129, 144, 160],
+    "far16": [0, 1, 15, 16, 17, 63, 64, 127, 128, 129, 255, 256, 511, 1023, 1024, 2047, 2048, 2049, 3000, 4095, 4096, 6000,
+              8191, 8192, 10000, 12345, 15000, 16000],
+    "far32": [0, 1, 16, 17, 127, 128, 129, 511, 1024, 2047, 2048, 2049, 4095, 4096, 8191, 8192, 12345, 16383, 16384, 16385,
+              20000, 24000, 24575, 24576, 28000, 30000, 31000, 31900],
+}
 _PLAIN = {}
+# The bfloat16 engine against the plain model on these folders (rows that reach every distance): 6.2e-3 to 6.9e-3
+# whole, cut, mixed and at 16,384 and 32,000 tokens; the bound is that and half as much again.
+DISTANCE_TOL_BF16 = 1.05e-2
+
+
+class _DistanceFolders(dict):
+    """key of DISTANCES -> a folder with one layer of the 7B shape whose heads look those distances back (written
+    when first asked for)."""
+
+    def __init__(self, factory):
+        super().__init__()
+        self.factory = factory
+
+    def __missing__(self, key):
+        self[key] = str(self.factory.mktemp(f"distance_{key}"))
+        _write_family_folder(self[key], "7B", max_position=32768, distances=DISTANCES[key])
+        return self[key]
 
 
 @pytest.fixture(scope="module")
 def distance_folders(tmp_path_factory):
-    """One layer of the 7B shape whose heads each look a fixed distance back, far and near; and the plain model's
-    weights of whichever was asked for last (float64: 6 GB, so one at a time)."""
-    out = {}
-    for key, dist in (("far", FAR_DISTANCES), ("near", NEAR_DISTANCES)):
-        out[key] = str(tmp_path_factory.mktemp(f"distance_{key}"))
-        _write_family_folder(out[key], "7B", max_position=32768, distances=dist)
-    yield out
-    _PLAIN.clear()
+    yield _DistanceFolders(tmp_path_factory)
+    _PLAIN.clear()           # (the plain model's float64 weights of the folder asked for last: 6 GB, so one at a time)
 
 
-def plain_rows(folder, ids, rows):
-    """The plain model's logits (float64, on the CPU) at ``rows`` of the sequence ``ids`` for a one-layer folder."""
+def plain_rows(folder, ids, rows, angle_dtype=torch.float32):
+    """The plain model's logits (float64, on the CPU) at ``rows`` of the sequence ``ids`` for a one-layer folder.  The
+    rotation angles are formed in 32 bits, as the reference and the engine form them: at positions of thousands that
+    rounding moves logits by more than everything else a 32-bit implementation rounds (at 16,384 tokens the float32
+    engine is 3.5e-6 from this oracle at every row and up to 1.1e-4 from one with exact angles)."""
     import plain_model as pm
     if folder not in _PLAIN:
         _PLAIN.clear()
         _PLAIN[folder] = pm.load_folder(folder, torch.float64)
     cfg, W = _PLAIN[folder]
-    return pm.forward_rows_one_layer(cfg, W, ids, rows)
+    return pm.forward_rows_one_layer(cfg, W, ids, rows, angle_dtype)
 
 
 def test_distance_heads_look_where_they_are_told(distance_folders):
@@ -203,18 +226,15 @@ def test_distance_heads_look_where_they_are_told(distance_folders):
     import math
     import plain_model as pm
     from safetensors.torch import load_file
-    t = load_file(distance_folders["far"] + "/model.safetensors")
-    d, theta, n = 128, 1000000.0, 20000
+    t = load_file(distance_folders["far32"] + "/model.safetensors")
+    d, theta, n = 128, 1000000.0, 33000
     bq = t["model.layers.0.self_attn.q_proj.bias"].double().view(28, d)
     bk = t["model.layers.0.self_attn.k_proj.bias"].double().view(4, d)
     k = pm.rope_split_half(bk[None].expand(n, 4, d).clone(), list(range(n)), theta)
     q = pm.rope_split_half(bq[None], [n - 1], theta)[0]
-    for h, dist in enumerate(FAR_DISTANCES):
+    for h, dist in enumerate(DISTANCES["far32"]):
         s = (k[:, h // 7, :] @ q[h]) / math.sqrt(d)
-        if dist < n:
-            assert int(s.argmax()) == n - 1 - dist and float(s.max() - s[torch.arange(n) != n - 1 - dist].max()) > 8.0, (h, dist)
-        else:
-            assert int(s.argmax()) == 0, (h, dist)
+        assert int(s.argmax()) == n - 1 - dist and float(s.max() - s[torch.arange(n) != n - 1 - dist].max()) > 8.0, (h, dist)
 
 
 @pytest.mark.parametrize("context", [16384, 32000])
@@ -226,7 +246,7 @@ def test_long_contexts_at_the_7b_layer_shape(context, distance_folders):
     block-table widths all have to find single keys."""
     from inferflux_amd.engine.api import load_runner
     from inferflux_amd.engine.context import StepEntry
-    folder = distance_folders["far"]
+    folder = distance_folders["far16" if context <= 16384 else "far32"]
     N = context + 8
     ids = seeded_ids(41 + context, N, FAMILY["7B"]["vocab_size"])
     rows = list(range(context - 16, N))
@@ -247,7 +267,7 @@ def test_long_contexts_at_the_7b_layer_shape(context, distance_folders):
         assert runner.manager.free_pages() == [N // 16 + 2]
         e = rel_err(torch.cat(got), want)
         print(f"7B layer, context {context}, {dtype}: {e:.2e}", flush=True)
-        assert e < (FAMILY_TOL["float32"] if dtype == "float32" else FAMILY_TOL["bfloat16"]["7B"]), (context, dtype, e)
+        assert e < (FAMILY_TOL["float32"] if dtype == "float32" else DISTANCE_TOL_BF16), (context, dtype, e)
         del runner
         torch.cuda.empty_cache()
 
@@ -306,7 +326,7 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(page_size, monkeypatch
     from inferflux_amd.engine.api import load_runner
     from inferflux_amd.engine.context import StepEntry
     from inferflux_amd.kernels import attention
-    folder = distance_folders["far"]
+    folder = distance_folders["near"]
     N, last = 3000, 24
     ids = seeded_ids(5, N, SHAPE["vocab_size"])
     cuttings = ([N], [700, 1100, 64, 500, 636], [1024, 1024, 952], [256] * 11 + [184], [2560, 128, 312])
@@ -335,7 +355,7 @@ def test_portions_behind_long_pasts_at_the_7b_layer_shape(page_size, monkeypatch
     for cuts in cuttings:
         e = rel_err(run(torch.bfloat16, cuts), want)
         print(f"7B layer, 3,000 tokens in {len(cuts)} portions, bfloat16 against the plain model: {e:.2e}", flush=True)
-        assert e < FAMILY_TOL["bfloat16"]["7B"], (cuts, e)
+        assert e < DISTANCE_TOL_BF16, (cuts, e)
     assert {t[0] for t in tilings} == {1, 2} and len({t[1] for t in tilings}) >= 3, tilings
 
 
@@ -345,8 +365,8 @@ def test_mixed_requests_at_the_7b_layer_shape(seed, distance_folders):
     tokens beside single decoded tokens, in a pool so small that pages are used again: steps of 1-16, 17-64, 65-128
     and more rows meet every product kernel (the streaming ones, the one that shares x through LDS up to 128 rows,
     the library whole and in slices of K) and both attention kernels in one batch.  The oracle is the plain model
-    (float64, on the CPU; heads that look fixed distances of up to 600 positions back) on 250 of the rows, drawn from
-    every request: the float32 engine, which runs each request whole, within 2e-5 of it, the bfloat16 engine's mixed
+    (float64, on the CPU; heads that look fixed distances of up to 160 positions back) on 250 of the rows that reach so
+    far back, drawn from every request: the float32 engine, which runs each request whole, within 2e-5 of it, the bfloat16 engine's mixed
     steps within the bound of the shape; and all rows of the bfloat16 engine against the float32 engine's."""
     import random
     import traces
@@ -358,7 +378,7 @@ def test_mixed_requests_at_the_7b_layer_shape(seed, distance_folders):
     steps, expected = traces.mixed(seqs, seed=seed, chunk_sizes=(2, 9, 17, 40, 70, 100, 128, 129, 300, 600))
     rows_per_step = sorted({sum(len(e["tokens"]) for e in st["entries"]) for st in steps})
     assert rows_per_step[0] <= 16 and any(64 < n <= 128 for n in rows_per_step) and rows_per_step[-1] > 256, rows_per_step
-    every = [(step, i, rid, p) for step, rows in expected.items() for i, (rid, p) in enumerate(rows)]
+    every = [(step, i, rid, p) for step, rows in expected.items() for i, (rid, p) in enumerate(rows) if p >= max(DISTANCES["near"])]
     sample = sorted(rng.sample(every, 250))
     plain = {}
     for rid, ids in seqs.items():
@@ -391,6 +411,6 @@ def test_mixed_requests_at_the_7b_layer_shape(seed, distance_folders):
     e = rel_err(torch.cat([got[k] for k in sorted(got)]), torch.stack(want))
     print(f"7B layer, mixed requests, seed {seed}: float32 {e32:.2e} and bfloat16 {e16:.2e} against the plain model on {len(sample)} rows; "
           f"bfloat16 against float32 {e:.2e} over {len(want)} rows, steps of {rows_per_step[0]}-{rows_per_step[-1]} rows", flush=True)
-    assert e16 < FAMILY_TOL["bfloat16"]["7B"] and e < FAMILY_TOL["bfloat16"]["7B"], (e16, e)
+    assert e16 < DISTANCE_TOL_BF16 and e < FAMILY_TOL["bfloat16"]["7B"], (e16, e)
     runner.manager.check()
     assert runner.manager.free_pages() == [pages]

@@ -33,7 +33,8 @@ def test_greedy_generation_equals_the_plain_model(name, model_folders):
     folder = model_folders[name]
     lens, n_new, chunk = WORKLOADS[name]
     prompts = [seeded_ids(50 + i, n, TINY[name]["vocab_size"]) for i, n in enumerate(lens)]
-    engine = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=8, chunked_prefill_tokens=chunk)
+    engine = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=8, chunked_prefill_tokens=chunk,
+                         prefill_tokens_alone=chunk)
     outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True))
     for p, o in zip(prompts, outs):
         assert o.finish_reason == "length" and o.token_ids == plain_greedy(folder, p, n_new)
@@ -102,7 +103,7 @@ def test_more_requests_than_slots_with_limits_stops_and_few_pages(seed, model_fo
 
     def run(early, pages):
         eng = Engine.load(folder, dtype="float32", kv_pages=pages, max_batch_size=4, chunked_prefill_tokens=16,
-                          start_steps_early=early)
+                          prefill_tokens_alone=24, start_steps_early=early)
         params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True, stop_token_ids=stops.get(i, ()))
                   for i, n in enumerate(limits)]
         outs = eng.generate(prompts, params)
@@ -144,7 +145,7 @@ def test_seeded_sampling_follows_the_plain_rule_and_ignores_batch_composition(mo
               SamplingParams(temperature=1.0, top_p=0.9, top_k=50, seed=12, max_tokens=24, ignore_eos=True),
               SamplingParams(temperature=1.2, min_p=0.001, repetition_penalty=1.3, frequency_penalty=0.1,
                              presence_penalty=0.2, seed=13, max_tokens=24, ignore_eos=True)]
-    engine = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=4, chunked_prefill_tokens=32)
+    engine = Engine.load(folder, dtype="float32", kv_pages=64, max_batch_size=4, chunked_prefill_tokens=32, prefill_tokens_alone=32)
     together = [o.token_ids for o in engine.generate(prompts, params)]
     alone = [engine.generate([p], [sp])[0].token_ids for p, sp in zip(prompts, params)]
     assert together == alone                                  # (seed, step) alone decides the draw
@@ -334,14 +335,14 @@ def test_per_request_state_is_zero_for_every_admission_through_the_engine():
     prompts = [seeded_ids(500 + i, n, V) for i, n in enumerate(lens)]
     # two slots for five requests: three of them start in a slot that holds another request's last state
     runner, _ = _stateful_toy_runner(pages=32, slots=2)
-    eng = Eng(runner, SchedulerConfig(2, 4096, 16))
+    eng = Eng(runner, SchedulerConfig(2, 4096, 16, 16))
     assert not runner.starts_steps_early                      # a step over state cannot be run twice
     outs = eng.generate(prompts, sp)
     assert [o.token_ids for o in outs] == want and eng.stats.preemptions == 0
     # three slots and 7 pages: 30+24, 9+24 and 40+24 tokens need 4 + 3 + 4 pages, so somebody is preempted and
     # admitted again (its slot may be the one it had: the state it left there must not survive)
     runner, _ = _stateful_toy_runner(pages=7, slots=3)
-    eng = Eng(runner, SchedulerConfig(3, 4096, 16))
+    eng = Eng(runner, SchedulerConfig(3, 4096, 16, 16))
     outs = eng.generate(prompts, sp)
     assert eng.stats.preemptions >= 1 and any(o.preemptions for o in outs)
     assert [o.token_ids for o in outs] == want
@@ -363,7 +364,7 @@ def test_requests_added_and_aborted_between_steps_by_hand(early, dtype, model_fo
     cfg, W = pm.load_folder(folder, torch.float64)
     P = {k: seeded_ids(600 + i, n, V) for i, (k, n) in enumerate({"a": 21, "b": 5, "c": 33, "d": 12, "w": 8, "s": 17, "x": 9}.items())}
     greedy = lambda n: SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)
-    eng = Engine.load(folder, dtype=dtype, kv_pages=40, max_batch_size=4, chunked_prefill_tokens=16,
+    eng = Engine.load(folder, dtype=dtype, kv_pages=40, max_batch_size=4, chunked_prefill_tokens=16, prefill_tokens_alone=16,
                       start_steps_early=early)
     runner = eng.runner
     done = {}
@@ -448,9 +449,10 @@ def test_random_arrivals_aborts_priorities_and_preemptions(name, seed, early, dt
     cfg, W = pm.load_folder(folder, torch.float64)
     rng = random.Random(seed * 7 + (1 if early else 0))
     pages = rng.randint(14, 22)
-    eng = Engine.load(folder, dtype=dtype, kv_pages=pages, max_batch_size=rng.randint(3, 6),
-                      chunked_prefill_tokens=rng.choice([8, 16, 24, 48]), max_batch_tokens=rng.choice([32, 64, 256]),
-                      start_steps_early=early)
+    batch, chunk = rng.randint(3, 6), rng.choice([8, 16, 24, 48])
+    eng = Engine.load(folder, dtype=dtype, kv_pages=pages, max_batch_size=batch,
+                      chunked_prefill_tokens=chunk, max_batch_tokens=rng.choice([32, 64, 256]),
+                      prefill_tokens_alone=3 * chunk, start_steps_early=early)
     reqs, done, aborted = {}, {}, {}
     n_req, next_id, steps = 40, 0, 0
     while next_id < n_req or eng.has_unfinished():

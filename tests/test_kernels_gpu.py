@@ -297,9 +297,11 @@ def test_gemm_f32_is_true_32_bit():
 
 
 # ---- attention ------------------------------------------------------------------------------
-def paged_case(seed, lens_q, lens_past, nH, nKV, d, P, dtype, window=None, n_pages=None, sharp=None):
+def paged_case(seed, lens_q, lens_past, nH, nKV, d, P, dtype, window=None, n_pages=None, sharp=None, garbage=False):
     """Random q/k/v for several requests, keys and values scattered into shuffled pages.
-    Returns device operands and the plain float64 result for this step's rows."""
+    Returns device operands and the plain float64 result for this step's rows.
+    ``garbage``: everything of the cache that no request holds (pages no table names, the slots of a last page past
+    its request's length) is filled with what a kernel must never let through: NaN keys and values of +-1e30."""
     g = gen(seed)
     R = len(lens_q)
     kv_lens = [a + b for a, b in zip(lens_q, lens_past)]
@@ -308,6 +310,9 @@ def paged_case(seed, lens_q, lens_past, nH, nKV, d, P, dtype, window=None, n_pag
     perm = torch.randperm(n_pages, generator=g).tolist()
     kc = torch.zeros(n_pages, nKV, P, d, dtype=dtype)
     vc = torch.zeros(n_pages, nKV, d, P, dtype=dtype)
+    if garbage:
+        kc.fill_(float("nan"))
+        vc.copy_(torch.where(torch.rand(vc.shape, generator=g) < 0.5, 1e30, -1e30))
     width = max(blocks)
     table = torch.full((R, width), -1, dtype=torch.int32)
     qs, outs, row_req, positions = [], [], [], []
@@ -686,6 +691,55 @@ def test_attention_tiles_random_cases(seed):
         assert torch.isfinite(out).all()
         assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), (seed, chunk, d, qt, lens_q, lens_past, nH, nKV, P, window,
                                                                  float((out - want).abs().max()))
+
+
+GARBAGE_CASES = [
+    # lens_q, lens_past, nH, nKV, d, P, window: requests that end inside a page, a window that starts inside one
+    ([1, 1, 3], [70, 1000, 45], 6, 3, 32, 16, None),
+    ([1, 1], [500, 23], 14, 2, 128, 64, 100),
+    ([70, 20], [200, 1000], 28, 4, 128, 16, None),
+    ([130, 33], [61, 900], 8, 2, 128, 32, 300),
+    ([100, 17], [300, 41], 4, 2, 64, 128, 77),
+]
+
+
+@pytest.mark.parametrize("case", GARBAGE_CASES)
+def test_attention_kernels_let_nothing_through_from_outside_tables_and_lengths(case):
+    """The cache holds NaN keys and values of +-1e30 wherever no request's table and length reach (other pages, the
+    rest of a last page), and inside the pages before a window.  Every matrix-core kernel (rows in splits and whole,
+    tiles of both heights, whole and in key splits) and the plain one still give the float64 result: what lies outside
+    is dropped by a select on the score, never multiplied in."""
+    lens_q, lens_past, nH, nKV, d, P, window = case
+    (q, kc, vc, row_req, positions, table), want, info = paged_case(21, lens_q, lens_past, nH, nKV, d, P, BF16, window, garbage=True)
+    scale = 1.0 / math.sqrt(d)
+    T = q.shape[0]
+    if window:           # the pages wholly before every window of a request: as a windowed cache group hands them back
+        first_needed = [(n - nq - window + 1) // P for n, nq in zip(info["kv_lens"], info["q_lens"])]
+        for r, b in enumerate(first_needed):
+            for blk in range(max(b, 0)):
+                kc[int(table[r, blk])] = float("nan")
+                vc[int(table[r, blk])] = 1e30
+    out = ops.attention_plain(q, kc, vc, row_req, positions, table, window, scale).cpu().double()
+    assert torch.isfinite(out).all() and close_rows(out, want), "plain"
+    for chunk, waves in ((32, 0), (128, 0), (128, 2), (128, 8)):
+        out = run_rows(q, kc, vc, row_req, positions, table, window, scale, chunk=chunk, waves=ops.row_waves_fit(nH, nKV, d, waves),
+                       extra_splits=1).cpu().double()
+        assert torch.isfinite(out).all() and close_rows(out, want), ("rows", chunk, waves, float((out - want).abs().max()))
+    q_len = torch.tensor(info["q_lens"], dtype=torch.int32)
+    q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    for qt in (1, 2):
+        tiles = [(r, q0) for r, n in enumerate(info["q_lens"]) for q0 in range(0, n, ops.attention_tile_rows(d, qt))]
+        for split_chunk in (0, 128):
+            splits = {}
+            if split_chunk:
+                splits = dict(chunk=split_chunk, max_splits=-(-max(info["kv_lens"]) // split_chunk) + 1,
+                              rows=torch.arange(T, dtype=torch.int32, device=DEV), row_req=row_req, positions=positions)
+            out = torch.zeros(T, nH * d, dtype=BF16, device=DEV)
+            ops.attention_tiles(q, kc, vc, out, dev([t[0] for t in tiles]), dev([t[1] for t in tiles]), q_start.to(DEV), q_len.to(DEV),
+                                dev(info["kv_lens"]), table, window, scale, qt, **splits)
+            out = out.cpu().double()
+            assert torch.isfinite(out).all() and close_rows(out, want), ("tiles", qt, split_chunk, float((out - want).abs().max()))
 
 
 def test_attention_tiles_refuses_splits_it_cannot_merge():

@@ -76,6 +76,25 @@ def test_rope_identity_norms_and_relative_positions():
 
 
 # ---- attention ------------------------------------------------------------------------------
+def test_rope_angles_formed_in_32_bits():
+    """The option for long sequences: the angle is the float32 product of the position and the float32 frequency.  At
+    small positions that is the exact angle to 1e-6; at position 30,000 it is tens of microradians to a milliradian off on the fast pairs,
+    exactly as numpy's float32 product says."""
+    import numpy as np
+    d, theta = 16, 1000000.0
+    x = torch.zeros(2, 1, d, dtype=D)
+    x[:, 0, 0] = 1.0                                     # (1, 0) on pair 0, whose frequency is 1
+    x[:, 0, 1] = 1.0                                     # and on pair 1: theta^(-2/16)
+    exact = pm.rope_split_half(x, [7, 30001], theta)
+    got = pm.rope_split_half(x, [7, 30001], theta, angle_dtype=torch.float32)
+    assert torch.allclose(got[0], exact[0], atol=1e-6)
+    f1 = np.float32(1.0 / theta ** (2.0 / d))
+    a = float(np.float32(30001) * f1)                    # the 32-bit product
+    assert abs(a - 30001 / theta ** (2.0 / d)) > 2e-5   # ... is not the exact angle
+    assert abs(float(got[1, 0, 1]) - math.cos(a)) < 1e-12 and abs(float(got[1, 0, 1 + d // 2]) - math.sin(a)) < 1e-12
+    assert abs(float(got[1, 0, 0]) - math.cos(30001.0)) < 1e-12          # pair 0: position times 1 is exact in 32 bits
+
+
 def test_attention_special_cases():
     d = 16
     q, k, v = rand(1, 4, d), rand(1, 2, d), rand(1, 2, d)

@@ -8,7 +8,10 @@ from inferflux_amd.engine.scheduler import RequestRefused, Scheduler, SchedulerC
 
 
 def make(pages=64, page_size=16, slots=8, max_position=4096, groups=None, **cfg):
+    """(Portions are ``chunked_prefill_tokens`` long with or without decoding requests beside them unless a test says
+    ``prefill_tokens_alone``.)"""
     m = CacheManager(groups or [GroupSpec(None, (0,))], page_size, pages, slots)
+    cfg.setdefault("prefill_tokens_alone", cfg.get("chunked_prefill_tokens", 512))
     return m, Scheduler(m, SchedulerConfig(**cfg), max_position)
 
 
@@ -35,7 +38,7 @@ def drive(m, s, max_steps=10000, log=None):
             cached.pop(rid, None)
         for it in plan.items:
             assert m.length(it.seq.rid) == len(cached.get(it.seq.rid, [])) == it.seq.computed   # positions are consistent
-            assert len(it.tokens) <= s.config.chunked_prefill_tokens
+            assert len(it.tokens) <= s.config.largest_portion
             m.reserve(it.seq.rid, len(it.tokens)); m.commit(it.seq.rid, len(it.tokens))       # what runner.step does
             cached.setdefault(it.seq.rid, []).extend(it.tokens)
             s.advance(it)
@@ -69,6 +72,23 @@ def test_a_long_prompt_is_cut_into_portions_with_logits_on_the_last():
     assert log == [[("a", 512, False)], [("a", 512, False)], [("a", 176, True)], [("a", 1, True)], [("a", 1, True)], [("a", 1, True)]]
     assert out["a"] == expected(range(1200), 4)
     assert m.free_pages() == [128] and not m.live()
+
+
+def test_portions_are_long_while_nobody_decodes():
+    """By default a prompt goes in portions of 2,048 while no request decodes (nobody waits for it), and of
+    chunked_prefill_tokens as soon as one does."""
+    m = CacheManager([GroupSpec(None, (0,))], 16, 1024, 8)
+    s = Scheduler(m, SchedulerConfig(), 8192)
+    assert (s.config.chunked_prefill_tokens, s.config.portion_alone, s.config.largest_portion) == (512, 2048, 2048)
+    s.add("a", list(range(5000)), 3)
+    s.add("b", list(range(100)), 40)
+    log = []
+    drive(m, s, log=log)
+    # a alone at first (b joins in the same step: both are prompts), then b decodes beside a's shorter portions
+    assert log[0] == [("a", 2048, False), ("b", 100, True)]
+    assert log[1] == [("a", 512, False), ("b", 1, True)] and log[2] == [("a", 512, False), ("b", 1, True)]
+    assert SchedulerConfig(chunked_prefill_tokens=4096).portion_alone == 4096
+    assert SchedulerConfig(chunked_prefill_tokens=64, prefill_tokens_alone=64).largest_portion == 64
 
 
 def test_decodes_first_then_the_budget_goes_to_prompts():
@@ -151,11 +171,16 @@ def test_refusals():
 def test_windowed_group_lets_long_requests_through_a_small_pool():
     groups = [GroupSpec(None, (0,)), GroupSpec(32, (1,))]
     m = CacheManager(groups, 16, [64, 8], 4)
-    s = Scheduler(m, SchedulerConfig(chunked_prefill_tokens=48), 2048)
+    s = Scheduler(m, SchedulerConfig(chunked_prefill_tokens=48, prefill_tokens_alone=48), 2048)
     s.add("a", list(range(500)), 100)
     out = drive(m, s)
     assert out["a"] == expected(range(500), 100)
     assert m.free_pages() == [64, 8]
+    # with portions of up to 2,048 tokens while nobody decodes (the default) the window's pool of 8 pages cannot take
+    # a portion, and the request is refused when it is added, not when it is half-way
+    s = Scheduler(m, SchedulerConfig(chunked_prefill_tokens=48), 2048)
+    with pytest.raises(RequestRefused, match="can never fit"):
+        s.add("b", list(range(500)), 100)
 
 
 @pytest.mark.parametrize("seed", range(4))
