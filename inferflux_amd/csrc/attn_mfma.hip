@@ -373,14 +373,15 @@ struct TileArgs {
   int max_blocks, nH, nKV, P, window;
   float scale_log2e;
   int page_shift;         // log2(P): the tile kernel takes power-of-two pages and splits positions by shift and mask
-  int n_tiles, per_xcd;   // work items are (tile, head, split); per_xcd = ceil(n_tiles * nH * max_splits / 8)
+  int n_tiles, per_xcd;   // work items are (tile, head, split); per_xcd = ceil(n_tiles * nH * max_splits / n_xcd)
+  int n_xcd;              // the chip's dies, which a launch deals its workgroups to in turn
   // With max_splits > 1 a workgroup takes only the keys [split * chunk, (split + 1) * chunk) (chunk a multiple of
   // 64) and writes unnormalised partial results in the row kernel's format, at the batch row's number; the
   // row kernel's merge finishes them.  For portions of prompts with a long past: few tiles, many keys.
   int chunk, max_splits;
   float* part_o;          // [T, nH, max_splits, D]
   float* part_ml;         // [T, nH, max_splits, 2]
-  // [8 * per_xcd] or nullptr: the work item of each place in the launch (-1: none), place x * per_xcd + i being
+  // [n_xcd * per_xcd] or nullptr: the work item of each place in the launch (-1: none), place x * per_xcd + i being
   // the i-th workgroup that XCD x is given.  The caller orders the items so that the workgroups that come to
   // share a compute unit have about the same number of key tiles between them on every unit.
   const int* order;
@@ -613,8 +614,8 @@ void attn_tiles_kernel(TileArgs a) {
   // workgroups that read one kv head's keys and values share an L2 instead of filling all eight with
   // everything; within a run the tiles with the most keys (the latest rows) come first.
   const int ratio = a.nH / a.nKV;
-  const int place = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
-  if (blockIdx.x / 8 >= a.per_xcd) return;                                              // the whole workgroup leaves together
+  const int place = (blockIdx.x % a.n_xcd) * a.per_xcd + blockIdx.x / a.n_xcd;
+  if (blockIdx.x / a.n_xcd >= a.per_xcd) return;                                              // the whole workgroup leaves together
   const int work = a.order ? a.order[place] : place;
   if (work < 0 || work >= a.n_tiles * a.nH * a.max_splits) return;
   const int item = work / a.max_splits, split = work % a.max_splits;
@@ -710,7 +711,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
                               const int* q_len, const int* kv_len, const int* block_table, int max_blocks,
                               int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
                               float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
-                              const int* positions, const int* order, int order_per_xcd, void* stream) {
+                              const int* positions, const int* order, int order_per_xcd, int n_xcd, void* stream) {
   IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_tiles: page_size %d must be a multiple of 16", page_size);
@@ -725,14 +726,16 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   if (n_tiles == 0) return 0;
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
-             n_tiles, 0, chunk, max_splits, part_o, part_ml, order};
+             n_tiles, 0, n_xcd, chunk, max_splits, part_o, part_ml, order};
   const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
-  IFX_REQUIRE(!order || (order_per_xcd > 0 && 8LL * order_per_xcd >= items && order_per_xcd <= items),
-              "attn_tiles: an order of 8 x %d places cannot hold %lld work items", order_per_xcd, items);
-  a.per_xcd = order ? order_per_xcd : (int)((items + 7) / 8);
+  IFX_REQUIRE(!order || (order_per_xcd > 0 && (long long)n_xcd * order_per_xcd >= items && order_per_xcd <= items),
+              "attn_tiles: an order of %d x %d places cannot hold %lld work items", n_xcd, order_per_xcd, items);
+  IFX_REQUIRE(n_xcd >= 1 && n_xcd <= 64, "%s: %d dies", "attn_tiles", n_xcd);
+  a.n_xcd = n_xcd;
+  a.per_xcd = order ? order_per_xcd : (int)((items + n_xcd - 1) / n_xcd);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(attn_tiles_kernel, dim3(8 * a.per_xcd), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(attn_tiles_kernel, dim3(n_xcd * a.per_xcd), dim3(256), 0, s, a);
   if (max_splits > 1) {
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,

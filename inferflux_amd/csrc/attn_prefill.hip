@@ -74,7 +74,8 @@ struct TileArgs {
   int max_blocks, nH, nKV, P, window;
   float scale_log2e;
   int page_shift;         // log2(P)
-  int n_tiles, per_xcd;   // work items are (tile, head, split); per_xcd = ceil(n_tiles * nH * max_splits / 8)
+  int n_tiles, per_xcd;   // work items are (tile, head, split); per_xcd = ceil(n_tiles * nH * max_splits / n_xcd)
+  int n_xcd;              // the chip's dies, which a launch deals its workgroups to in turn
   int chunk, max_splits;  // as in attn_mfma.hip's tile kernel: keys [split * chunk, (split + 1) * chunk) per workgroup
   float* part_o;          // [T, nH, max_splits, D]
   float* part_ml;         // [T, nH, max_splits, 2]
@@ -212,8 +213,8 @@ void attn_prefill_kernel(TileArgs a) {
   // Work items as in attn_mfma.hip's tile kernel: kv head first, dealt to the 8 XCDs in contiguous runs (an L2
   // then holds a few kv heads' keys and values, not all of them), tiles with the most keys first within a run.
   const int ratio = a.nH / a.nKV;
-  const int place = (blockIdx.x % 8) * a.per_xcd + blockIdx.x / 8;
-  if (blockIdx.x / 8 >= a.per_xcd) return;                                              // the whole workgroup leaves together
+  const int place = (blockIdx.x % a.n_xcd) * a.per_xcd + blockIdx.x / a.n_xcd;
+  if (blockIdx.x / a.n_xcd >= a.per_xcd) return;                                              // the whole workgroup leaves together
   const int work = a.order ? a.order[place] : place;
   if (work < 0 || work >= a.n_tiles * a.nH * a.max_splits) return;
   const int item = work / a.max_splits, split = work % a.max_splits;
@@ -380,7 +381,7 @@ extern "C" int ifx_attn_prefill(const void* q, const void* k_cache, const void* 
                                 const int* q_len, const int* kv_len, const int* block_table, int max_blocks,
                                 int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
                                 float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
-                                const int* positions, const int* order, int order_per_xcd, void* stream) {
+                                const int* positions, const int* order, int order_per_xcd, int n_xcd, void* stream) {
   IFX_REQUIRE(d == D, "attn_prefill: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_prefill: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0, "attn_prefill: page_size %d must be a power of two from 16", page_size);
@@ -400,14 +401,16 @@ extern "C" int ifx_attn_prefill(const void* q, const void* k_cache, const void* 
   }
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
-             n_tiles, 0, chunk, max_splits, part_o, part_ml, order};
+             n_tiles, 0, n_xcd, chunk, max_splits, part_o, part_ml, order};
   const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_prefill: too many tiles for one launch");
-  IFX_REQUIRE(!order || (order_per_xcd > 0 && 8LL * order_per_xcd >= items && order_per_xcd <= items),
-              "attn_prefill: an order of 8 x %d places cannot hold %lld work items", order_per_xcd, items);
-  a.per_xcd = order ? order_per_xcd : (int)((items + 7) / 8);
+  IFX_REQUIRE(!order || (order_per_xcd > 0 && (long long)n_xcd * order_per_xcd >= items && order_per_xcd <= items),
+              "attn_prefill: an order of %d x %d places cannot hold %lld work items", n_xcd, order_per_xcd, items);
+  IFX_REQUIRE(n_xcd >= 1 && n_xcd <= 64, "%s: %d dies", "attn_prefill", n_xcd);
+  a.n_xcd = n_xcd;
+  a.per_xcd = order ? order_per_xcd : (int)((items + n_xcd - 1) / n_xcd);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(8 * a.per_xcd), dim3(64 * NW), NS * STAGE_BYTES, s, a);
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_xcd * a.per_xcd), dim3(64 * NW), NS * STAGE_BYTES, s, a);
   if (max_splits > 1) {
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,

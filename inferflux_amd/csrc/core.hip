@@ -303,10 +303,11 @@ extern "C" int ifx_rope_table(const int* positions, const float* inv_freq, float
 }
 
 // ---------------------------------------------------------------------------------------
-// Per token t: qkv[t] = [q (nH*d) | k (nKV*d) | v (nKV*d)].  Adds the bias, rotates q and k by
+// Per token t: qkv[t] = [q (nH*d) | k (nKV*d) | v (nKV*dv)].  Adds the bias, rotates q and k by
 // the token's position, writes q to q_out[t] and k, v into the paged cache at slot[t]
 // (slot = page * page_size + offset; slot < 0: nothing is written to the cache).
-// Cache layouts: K [page][kv head][offset][d], V [page][kv head][d][offset].
+// Cache layouts: K [page][kv head][offset][d], V [page][kv head][dv][offset]; values may be
+// narrower or wider than keys (dv != d).
 // rope_style: 0 none, 1 split-half pairs (p, p + rot/2), 2 consecutive pairs (2p, 2p+1);
 // cos/sin come from the step's table [T, rotary_dim / 2]; elements at or beyond rotary_dim are
 // copied.  One block per (token, head): q heads, then k heads, then v heads.
@@ -325,13 +326,14 @@ struct RopeArgs {
   void* q_out;
   void* k_cache;
   void* v_cache;
+  int dv;                // width of a value head
 };
 
 template <typename T>
 __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   const int t = blockIdx.x, head = blockIdx.y;
-  const int d = a.d, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
-  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + 2 * kv_width;
+  const int d = a.d, dv = a.dv, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + kv_width + a.nKV * dv;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
   const float* part = (const float*)a.qkv + (size_t)t * row_width;
   // Elements i0 and i1 of the row; partial sums are added in slice order, eight slices of both elements asked for
@@ -386,14 +388,15 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   } else {
     if (slot < 0) return;
     const int kh = head - a.nH - a.nKV;
-    T* vc = (T*)a.v_cache + ((size_t)page * a.nKV + kh) * d * a.page_size + off;
-    for (int e = threadIdx.x; e < d; e += 2 * blockDim.x) {     // two elements per thread and round: their loads go out together
-      const int e1 = min(e + (int)blockDim.x, d - 1);
+    const int vcol = q_width + kv_width + kh * dv;              // value heads are dv wide
+    T* vc = (T*)a.v_cache + ((size_t)page * a.nKV + kh) * dv * a.page_size + off;
+    for (int e = threadIdx.x; e < dv; e += 2 * blockDim.x) {    // two elements per thread and round: their loads go out together
+      const int e1 = min(e + (int)blockDim.x, dv - 1);
       float x, x1;
-      in2(col + e, col + e1, x, x1);
-      if (a.bias) { x += load_dyn(a.bias, a.bias_dtype, col + e); x1 += load_dyn(a.bias, a.bias_dtype, col + e1); }
+      in2(vcol + e, vcol + e1, x, x1);
+      if (a.bias) { x += load_dyn(a.bias, a.bias_dtype, vcol + e); x1 += load_dyn(a.bias, a.bias_dtype, vcol + e1); }
       vc[(size_t)e * a.page_size] = from_f<T>(x);
-      if (e + (int)blockDim.x < d) vc[(size_t)e1 * a.page_size] = from_f<T>(x1);
+      if (e + (int)blockDim.x < dv) vc[(size_t)e1 * a.page_size] = from_f<T>(x1);
     }
   }
 }
@@ -487,9 +490,9 @@ __global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T,
 extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const int* slots,
                                const float* cs, const float* sn, int rope_style, int rotary_dim, int T, int nH,
                                int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, int n_slices,
-                               long long slice_stride, void* stream) {
+                               long long slice_stride, int dv, void* stream) {
   IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || slice_stride > 0), "rope_append: %d slices, %lld apart", n_slices, slice_stride);
-  IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
+  IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0 && dv > 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d dv=%d", T, nH, nKV, d, dv);
   IFX_REQUIRE(rope_style >= 0 && rope_style <= 2, "rope_append: unknown rope style %d", rope_style);
   IFX_REQUIRE(rope_style == 0 || (rotary_dim > 0 && rotary_dim <= d && rotary_dim % 2 == 0 && cs && sn),
               "rope_append: rotary_dim %d must be even, within head_dim %d, with a rotation table", rotary_dim, d);
@@ -497,10 +500,10 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   IFX_REQUIRE(nH + 2 * nKV <= 65535, "rope_append: too many heads for one launch");
   if (T == 0) return 0;
   RopeArgs a{qkv, n_slices, (size_t)slice_stride, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size,
-             q_out, k_cache, v_cache};
+             q_out, k_cache, v_cache, dv};
   hipStream_t s = (hipStream_t)stream;
   // (a few tokens are quicker with one small block per token and head: nothing waits on a loop over tokens)
-  if (T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
+  if (dv == d && T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
       (!slots || page_size % 8 == 0)) {
     const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
     const size_t v_threads = slots ? (size_t)((T + 7) / 8) * nKV * d : 0;

@@ -106,7 +106,7 @@ def choose_tiling(tiled_rows, tiled_keys, n_heads: int, rows_of, tall_direct: bo
     return qt, splits, chunk
 
 
-N_XCD, CUS_PER_XCD = 8, 32     # the launch deals workgroups to the XCDs in turn, and an XCD deals its share to its compute units in turn
+from .device import CUS_PER_XCD, N_XCD      # the launch deals workgroups to the XCDs in turn, and an XCD its share to its compute units in turn
 
 
 def tile_order(first_pos, last_pos, n_heads: int, window: Optional[int], splits: int, chunk: int, period: int = CUS_PER_XCD) -> np.ndarray:
@@ -224,7 +224,7 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     """q [T, nH, d] of this step's rows against ``cache`` (a LayerCache); returns [T, nH*d]."""
     T, nH, d = q.shape
     table = ctx.block_table(cache.group)
-    if not ops.mfma_attention_supported(q.dtype, d, cache.page_size):
+    if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:    # (values of another width: the plain kernel)
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale)
     n_kv = cache.k.shape[1]
     # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often.

@@ -28,7 +28,7 @@ from typing import Dict, Iterable, Optional, Sequence, Tuple
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "csrc")
 CSRC = os.path.normpath(CSRC)
-ARCH = "gfx950"
+from .device import ARCH
 # -packed-fp32-ops is switched off for device code: some packed float forms have given wrong
 # results on this hardware.  The host pass of hipcc does not know the feature and says so.
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",

@@ -26,10 +26,30 @@ GEMM_SHAPES = {"qkv": (4608, 3584), "o": (3584, 3584), "gate_up": (37888, 3584),
                "lm_head": (152064, 3584)}
 
 
-def _time_us(fn, iters: int) -> float:
+def _time_us(fn, iters: int, graph: bool = False) -> float:
     """Average time of a call, after about 50 ms of the same calls (the card's clocks take that long to settle: a
-    kernel of 0.5 ms timed after three warm-up calls reads 10-20 % slow)."""
+    kernel of 0.5 ms timed after three warm-up calls reads 10-20 % slow).  ``graph``: the ``iters`` calls are captured
+    as one HIP graph and the graph is replayed, so that kernels shorter than the host's 10-15 us per call are timed as
+    they run inside a captured decode step, one behind the other."""
     import time
+    if graph:
+        fn(0)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(iters):
+                fn(i)
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.05:
+            g.replay()
+            torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / (5 * iters) * 1e3
     t0 = time.perf_counter()
     n = 0
     while n < 3 or (time.perf_counter() - t0 < 0.05 and n < 2000):
@@ -99,13 +119,13 @@ def attention_rows(args) -> None:
     for chunk in ([int(c) for c in args.chunk.split(",")] if args.chunk else [128, 256, 512, 1024]):
         splits = -(-bound // chunk)
         t = _time_us(lambda i: ops.attention_rows(q, *caches[i % copies], out, None, B, row_req, pos, table, None,
-                                                  1 / math.sqrt(d), chunk, splits), args.iters)
+                                                  1 / math.sqrt(d), chunk, splits), args.iters, args.graph)
         print(f"attention-rows batch={B} context={kv} one wave per split of {chunk} keys ({splits} splits) + merge launch: "
               f"{t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache", flush=True)
     for waves in [int(w) for w in args.waves.split(",") if w]:
         waves = ops.row_waves_fit(nH, nKV, d, waves)
         t = _time_us(lambda i: ops.attention_rows(q, *caches[i % copies], out, None, B, row_req, pos, table, None,
-                                                  1 / math.sqrt(d), 0, 1, waves), args.iters)
+                                                  1 / math.sqrt(d), 0, 1, waves), args.iters, args.graph)
         print(f"attention-rows batch={B} context={kv} one workgroup of {waves} waves per (row, kv head): "
               f"{t:8.1f} us  {gb / t * 1e3:5.2f} TB/s of cache", flush=True)
 
@@ -118,8 +138,8 @@ def gemm(args) -> None:
         ws = [ops.prepare_linear(torch.randn(N, K, device=dev, dtype=torch.bfloat16)) for _ in range(copies)]
         x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
         gb = N * K * 2 / 1e9
-        t = _time_us(lambda i: ops.linear(x, ws[i % copies]), args.iters)
-        t_lib = _time_us(lambda i: torch.matmul(x, ws[i % copies].rows.t()), args.iters)
+        t = _time_us(lambda i: ops.linear(x, ws[i % copies]), args.iters, args.graph)
+        t_lib = _time_us(lambda i: torch.matmul(x, ws[i % copies].rows.t()), args.iters, args.graph)
         print(f"gemm {name:8s} rows={M:3d} [{N} x {K}]: engine's choice {t:8.1f} us ({gb / t * 1e3:5.2f} TB/s of weights)   "
               f"library {t_lib:8.1f} us", flush=True)
         del ws
@@ -171,6 +191,9 @@ def main(argv=None) -> int:
         p = sub.add_parser(name)
         p.set_defaults(fn=fn)
         p.add_argument("--iters", type=int, default=10)
+        if name in ("attention-rows", "gemm"):
+            p.add_argument("--graph", action="store_true", help="time the calls inside a replayed HIP graph (kernels shorter than "
+                           "the host's time per call)")
         if name.startswith("attention"):
             p.add_argument("--heads", type=int, default=28)
             p.add_argument("--kv-heads", type=int, default=4)

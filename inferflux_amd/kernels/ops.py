@@ -13,6 +13,7 @@ from typing import Dict, Iterable, Optional, Tuple
 import torch
 
 from .. import log
+from .device import ARCH, COMPUTE_UNITS, N_XCD
 from .library import KernelModule, Variant, load_module
 
 P = ctypes.c_void_p
@@ -34,7 +35,9 @@ MFMA_MAX_HEAD_DIM = 128
 # size 128 the tall tiles are the kernel of attn_prefill.hip (eight waves of 16 rows, tiles loaded straight into
 # LDS), at the other head sizes attn_mfma.hip's with two query tiles per wave.
 TILE_QTS = (1, 2)
-DIRECT_TILE_HEAD_DIM = 128
+# (that kernel is written in gfx950's own instructions, loads into LDS of 16 bytes a lane among them; built for anything
+# else, the tall tiles of head size 128 are attn_mfma.hip's as well)
+DIRECT_TILE_HEAD_DIM = 128 if ARCH == "gfx950" else None
 
 
 class KernelError(RuntimeError):
@@ -167,16 +170,18 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
 def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                 cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rope_style: int,
                 rotary_dim: int, n_heads: int, n_kv_heads: int, head_dim: int,
-                k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
+                k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int,
+                v_head_dim: Optional[int] = None) -> torch.Tensor:
     """Bias, rotation and cache write of one step's projections; returns q [T, n_heads, head_dim].
 
-    ``qkv`` is [T, (n_heads + 2 n_kv_heads) head_dim] when the keys and values are written
-    (``slots`` int32 [T] = page * page_size + offset), or [T, n_heads head_dim] with
-    ``n_kv_heads`` = 0 for a mixer that only reads another's cache.  ``cos`` / ``sin`` are the
-    step's rotation table [T, rotary_dim / 2] (from rope_table).
+    ``qkv`` is [T, (n_heads + n_kv_heads) head_dim + n_kv_heads v_head_dim] when the keys and values are
+    written (``slots`` int32 [T] = page * page_size + offset; ``v_head_dim`` None: as wide as the keys), or
+    [T, n_heads head_dim] with ``n_kv_heads`` = 0 for a mixer that only reads another's cache.  ``cos`` / ``sin``
+    are the step's rotation table [T, rotary_dim / 2] (from rope_table).
     """
     T = qkv.shape[0]
-    width = (n_heads + 2 * n_kv_heads) * head_dim
+    dv = head_dim if v_head_dim is None else int(v_head_dim)
+    width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * dv
     n_slices = 1
     if isinstance(qkv, SliceSums):                  # partial sums: the kernel adds them in slice order
         _check(qkv.parts, "qkv", (None, T, width), torch.float32)
@@ -192,15 +197,15 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
     if slots is not None:
         _check(slots, "slots", (T,), torch.int32)
         _check(k_cache, "k_cache", (None, n_kv_heads, page_size, head_dim), dtype)
-        _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, head_dim, page_size), dtype)
+        _check(v_cache, "v_cache", (k_cache.shape[0], n_kv_heads, dv, page_size), dtype)
     elif n_kv_heads != 0:
         raise KernelError("rope_append: keys and values given but no slots to write them to")
     q = torch.empty((T, n_heads, head_dim), dtype=dtype, device=qkv.device)
-    _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, P),
+    _call(load_module("core"), "ifx_rope_append", (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, I, P),
           qkv.data_ptr(), _DT[dtype], _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
           _ptr(cos) if rope_style != ROPE_NONE else 0, _ptr(sin) if rope_style != ROPE_NONE else 0, rope_style,
           rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache), _ptr(v_cache),
-          n_slices, T * width, _stream())
+          n_slices, T * width, dv, _stream())
     return q
 
 
@@ -285,7 +290,6 @@ def tile_weights(weight: torch.Tensor, order: Optional[torch.Tensor] = None, til
 
 
 TILE_ROWS = (8, 10, 12, 14, 16)      # rows a tile of the copy may hold
-COMPUTE_UNITS = 256
 
 
 def _tiled_size(N: int, K: int, tile_rows: int) -> int:
@@ -812,14 +816,14 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     per_xcd = 0
     if order is not None:
         _check(order, "order", (None,), torch.int32)
-        if order.shape[0] % 8:
-            raise KernelError("attention_tiles: the order has a place for each of 8 XCDs' workgroups")
-        per_xcd = order.shape[0] // 8
-    _call(mod, entry, (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, P),
+        if order.shape[0] % N_XCD:
+            raise KernelError(f"attention_tiles: the order has a place for each of {N_XCD} XCDs' workgroups")
+        per_xcd = order.shape[0] // N_XCD
+    _call(mod, entry, (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, I, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(),
           n_tiles, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), block_table.data_ptr(),
           block_table.shape[1], nH, nKV, d, page_size, int(window or 0), float(scale), int(chunk), int(max_splits),
-          _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, _stream())
+          _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, N_XCD, _stream())
 
 
 # ----------------------------------------------------------------------------------------

@@ -32,31 +32,35 @@ class PagedAttention(Mixer):
 
     def __init__(self, name: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, bias: bool = True, window: Optional[int] = None,
-                 scale: Optional[float] = None, init_std: float = 0.02):
+                 scale: Optional[float] = None, init_std: float = 0.02, v_head_dim: Optional[int] = None):
+        """``v_head_dim``: the width of a value head where it differs from ``head_dim`` (such a layer runs on the
+        kernels that take both widths: the plain attention kernel and the unfused projection path)."""
         if n_heads % n_kv_heads:
             raise ValueError(f"{name}: {n_heads} query heads are not a multiple of {n_kv_heads} kv heads")
         self.name, self.hidden_size = name, int(hidden_size)
         self.n_heads, self.n_kv_heads, self.head_dim = int(n_heads), int(n_kv_heads), int(head_dim)
+        self.v_head_dim = int(v_head_dim) if v_head_dim else self.head_dim
         self.bias, self.window, self.init_std = bool(bias), (int(window) if window else None), init_std
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = build_part("position", position)
         self.w_qkv = self.b_qkv = self.w_o = self._w_q = None
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(self.n_kv_heads, self.head_dim, self.window)
+        return CacheSpec(self.n_kv_heads, self.head_dim, self.window,
+                         self.v_head_dim if self.v_head_dim != self.head_dim else None)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        H, d, s = self.hidden_size, self.head_dim, ("normal", self.init_std)
+        H, d, dv, s = self.hidden_size, self.head_dim, self.v_head_dim, ("normal", self.init_std)
         out = {
             f"{self.name}.q_proj.weight": ParamSpec((self.n_heads * d, H), s),
             f"{self.name}.k_proj.weight": ParamSpec((self.n_kv_heads * d, H), s),
-            f"{self.name}.v_proj.weight": ParamSpec((self.n_kv_heads * d, H), s),
-            f"{self.name}.o_proj.weight": ParamSpec((H, self.n_heads * d), s),
+            f"{self.name}.v_proj.weight": ParamSpec((self.n_kv_heads * dv, H), s),
+            f"{self.name}.o_proj.weight": ParamSpec((H, self.n_heads * dv), s),
         }
         if self.bias:
             out[f"{self.name}.q_proj.bias"] = ParamSpec((self.n_heads * d,), s)
             out[f"{self.name}.k_proj.bias"] = ParamSpec((self.n_kv_heads * d,), s)
-            out[f"{self.name}.v_proj.bias"] = ParamSpec((self.n_kv_heads * d,), s)
+            out[f"{self.name}.v_proj.bias"] = ParamSpec((self.n_kv_heads * dv,), s)
         return out
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
@@ -72,7 +76,7 @@ class PagedAttention(Mixer):
         row tiles are ordered so that the fused projection + rotation kernel finds both halves of a rotation
         pair in one lane (plain products read the same copy through the order)."""
         order = None
-        if self.head_dim % 32 == 0 and weight.is_cuda and weight.dtype == torch.bfloat16:
+        if self.head_dim % 32 == 0 and self.v_head_dim == self.head_dim and weight.is_cuda and weight.dtype == torch.bfloat16:
             order = torch.tensor(ops.pair_tile_order(heads, self.head_dim), dtype=torch.int32, device=weight.device)
         return ops.prepare_linear(weight, order)
 
@@ -90,7 +94,7 @@ class PagedAttention(Mixer):
         cache = binding.cache
         nH, d = self.n_heads, self.head_dim
         nKV = self.n_kv_heads if binding.writes_cache else 0
-        width = (nH + 2 * nKV) * d
+        width = (nH + nKV) * d + nKV * self.v_head_dim
         style, rotary_dim, cos, sin = self.position.kernel_args(ctx)
         w, b = self.w_qkv, self.b_qkv
         if not binding.writes_cache:  # only the queries: the first nH*d rows of the fused matrix
@@ -115,7 +119,7 @@ class PagedAttention(Mixer):
             qkv, b = self._encode_outside(qkv, b, ctx, nKV), None
         q = ops.rope_append(qkv, b, slots, cos, sin, style, rotary_dim, nH, nKV, d,
                             cache.k if slots is not None else None, cache.v if slots is not None else None,
-                            cache.page_size)
+                            cache.page_size, self.v_head_dim)
         if t is not None:
             t.mark("mixer.qkv")
         a = paged_attention(q, cache, ctx, self.window, self.scale)

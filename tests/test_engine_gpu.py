@@ -794,6 +794,69 @@ def test_a_toy_embedding_that_reads_positions_and_a_toy_mixer_with_narrow_values
     assert not torch.allclose(runner.step([StepEntry("z", ids[:10], list(range(10)))]).cpu(), whole[:10], rtol=1e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d,dv", [(16, 8), (16, 40), (32, 32)])
+def test_builtin_attention_with_values_of_another_width_than_keys(d, dv, dtype):
+    """The package's own attention part with value heads narrower and wider than the key heads (and, as the control,
+    as wide): the plan says ``v_head_dim``, the part sizes its v and o projections and its cache by it, and such a
+    layer runs on the kernels that take both widths (in bfloat16 too: the plain attention kernel, the unfused
+    projection path).  Whole against cut, and against the formulas written out, rotary positions and biases included."""
+    from inferflux_amd.engine.model import Model
+    from inferflux_amd.engine.runner import ModelRunner
+    from inferflux_amd.parts import LayerSpec, ModelPlan, PartSpec, ScheduleEntry
+    H, V, nH, nKV, theta, N = 48, 90, 4, 2, 10000.0, 70
+    p = "toy.layers.0"
+    attn = PartSpec("paged_attention", {"name": f"{p}.attn", "n_heads": nH, "n_kv_heads": nKV, "head_dim": d, "v_head_dim": dv,
+                                        "bias": True, "init_std": 0.3, "position": PartSpec("rotary", {"head_dim": d, "theta": theta})})
+    layer = LayerSpec(p, PartSpec("prenorm"), PartSpec("rmsnorm", {"name": f"{p}.n1", "eps": 1e-5}), attn,
+                      PartSpec("rmsnorm", {"name": f"{p}.n2", "eps": 1e-5}),
+                      PartSpec("swiglu", {"name": f"{p}.mlp", "intermediate_size": 64}))
+    plan = ModelPlan(vocab_size=V, hidden_size=H, max_position=128,
+                     embedding=PartSpec("token_embedding", {"name": "toy.embed", "vocab_size": V}),
+                     layers=(layer,), schedule=(ScheduleEntry(0),),
+                     final_norm=PartSpec("rmsnorm", {"name": "toy.norm", "eps": 1e-5}),
+                     lm_head=PartSpec("linear_head", {"name": "toy.head", "vocab_size": V}))
+    model = Model(plan=plan).init_random(12, DT[dtype], "cuda")
+    specs = model.param_specs()
+    assert specs[f"{p}.attn.v_proj.weight"].shape == (nKV * dv, H) and specs[f"{p}.attn.o_proj.weight"].shape == (H, nH * dv)
+    runner = ModelRunner(model, num_pages=10, max_requests=2)
+    cache = runner.storage.binding(0).cache
+    assert tuple(cache.k.shape[1:]) == (nKV, 16, d) and tuple(cache.v.shape[1:]) == (nKV, dv, 16)
+    ids = seeded_ids(33, N, V)
+    runner.add_request("w")
+    whole = runner.step([StepEntry("w", ids, list(range(N)))]).cpu()
+    runner.free_request("w")
+    runner.add_request("o"); runner.add_request("c")
+    rows, at = [], 0
+    for m in (17, 1, 2, 30, 1, 19):
+        rows.append(runner.step([StepEntry("o", ids[at:at + 1], []), StepEntry("c", ids[at:at + m], list(range(m)))]).cpu()[:m])
+        at += m
+    cut = torch.cat(rows)
+    # the formulas, plainly, from the tensors the parts hold
+    att, blk = model.blocks[0].mixer, model.blocks[0]
+    D = lambda t: t.double().cpu()
+    wqkv, bqkv = D(att.w_qkv.rows), D(att.b_qkv)
+    x = D(model.embedding.table)[ids]
+    h = pm.rms_norm(x, D(blk.norm_in.weight), 1e-5)
+    qkv = h @ wqkv.t() + bqkv
+    q = pm.rope_split_half(qkv[:, :nH * d].reshape(N, nH, d), list(range(N)), theta)
+    k = pm.rope_split_half(qkv[:, nH * d:(nH + nKV) * d].reshape(N, nKV, d), list(range(N)), theta)
+    v = qkv[:, (nH + nKV) * d:].reshape(N, nKV, dv)
+    s = torch.einsum("ihd,jhd->hij", q, k.repeat_interleave(nH // nKV, dim=1)) * d ** -0.5
+    s = s.masked_fill(torch.triu(torch.ones(N, N, dtype=torch.bool), 1), float("-inf"))
+    o = torch.einsum("hij,jhe->ihe", torch.softmax(s, -1), v.repeat_interleave(nH // nKV, dim=1)).reshape(N, nH * dv)
+    x = x + o @ D(att.w_o.rows).t()
+    h = pm.rms_norm(x, D(blk.norm_post.weight), 1e-5)
+    x = x + pm.swiglu(h, D(blk.ffn.w_gate_up.rows)[0::2], D(blk.ffn.w_gate_up.rows)[1::2], D(blk.ffn.w_down.rows))
+    want = pm.rms_norm(x, D(model.final_norm.weight), 1e-5) @ D(model.head.weight.rows).t()
+    if dtype == "float32":
+        assert torch.allclose(cut, whole, rtol=1e-4, atol=1e-5)
+        assert rel_err(whole, want) < REL_TOL["float32"]
+    else:
+        assert rel_err(cut, want) < 3e-2 and rel_err(whole, want) < 3e-2
+    assert runner.manager.free_pages() == [10 - 5 - 1]          # "c" holds 70 tokens, "o" one
+
+
 def test_a_toy_block_with_four_norms_and_no_feed_forward():
     """An arrangement from outside the package that the built-in one does not cover: pre-norm, attention, a norm on
     the attention's output before the add, a norm on the skip path, and no feed-forward at all; the two further

@@ -341,6 +341,12 @@ def paged_case(seed, lens_q, lens_past, nH, nKV, d, P, dtype, window=None, n_pag
             dev(torch.tensor(positions, dtype=torch.int32)), dev(table)), want, dict(q_lens=lens_q, kv_lens=kv_lens)
 
 
+def close_rows(out, want):
+    """Row attention against float64: element by element, and the largest error against the largest value (a bound
+    that follows the data: outputs here are 0.1-1 in size)."""
+    return torch.allclose(out, want, rtol=1e-2, atol=1e-2) and float((out - want).abs().max()) <= 1e-2 * float(want.abs().max())
+
+
 ATTN_CASES = [
     # lens_q, lens_past, nH, nKV, d, P, window, sharp
     ([1], [0], 4, 2, 16, 16, None, None),                       # a single key: the output is its value
@@ -540,12 +546,6 @@ def run_rows(q, kc, vc, row_req, positions, table, window, scale, rows=None, chu
     return out
 
 
-def close_rows(out, want):
-    """Row attention against float64: element by element, and the largest error against the largest value (a bound
-    that follows the data: outputs here are 0.1-1 in size)."""
-    return torch.allclose(out, want, rtol=1e-2, atol=1e-2) and float((out - want).abs().max()) <= 1e-2 * float(want.abs().max())
-
-
 @pytest.mark.parametrize("chunk,waves", [(32, 0), (128, 0), (1024, 0), (128, 1), (128, 2), (128, 3), (128, 4), (128, 8)])
 @pytest.mark.parametrize("case", MFMA_CASES)
 def test_attention_rows(case, chunk, waves):
@@ -599,7 +599,7 @@ def test_attention_rows_subset_leaves_other_rows_alone():
     (q, kc, vc, row_req, positions, table), want, _ = paged_case(8, [5, 1, 3], [10, 99, 40], 6, 2, 32, 16, BF16)
     rows = torch.tensor([5, 0, 8], dtype=torch.int32, device=DEV)
     out = run_rows(q, kc, vc, row_req, positions, table, None, 1.0 / math.sqrt(32), rows=rows).cpu().double()
-    assert torch.allclose(out[[5, 0, 8]], want[[5, 0, 8]], rtol=1e-2, atol=1e-2)
+    assert close_rows(out[[5, 0, 8]], want[[5, 0, 8]])
     rest = [i for i in range(9) if i not in (5, 0, 8)]
     assert torch.all(out[rest] == 0)
 
@@ -627,7 +627,7 @@ def test_attention_tiles(case, qt, split_chunk):
     plain_order = out.clone()
     out = out.cpu().double()
     assert torch.isfinite(out).all()
-    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), float((out - want).abs().max())
+    assert close_rows(out, want), float((out - want).abs().max())
     # the same launch with its workgroups in the balanced order, and in a shuffled one with gaps: the same bits
     import numpy as np
     from inferflux_amd.kernels.attention import tile_order
@@ -689,8 +689,7 @@ def test_attention_tiles_random_cases(seed):
                             dev(info["kv_lens"]), table, window, 1.0 / math.sqrt(d), qt, order=order, **splits)
         out = out.cpu().double()
         assert torch.isfinite(out).all()
-        assert torch.allclose(out, want, rtol=1e-2, atol=1e-2), (seed, chunk, d, qt, lens_q, lens_past, nH, nKV, P, window,
-                                                                 float((out - want).abs().max()))
+        assert close_rows(out, want), (seed, chunk, d, qt, lens_q, lens_past, nH, nKV, P, window, float((out - want).abs().max()))
 
 
 GARBAGE_CASES = [
