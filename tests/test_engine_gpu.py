@@ -471,6 +471,62 @@ def test_replayed_decode_graphs_equal_eager_steps(name, dtype, sharp_folders):
     assert rel_err(got[0], want) < tol(dtype, name)
 
 
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_decode_rows_taken_whole_by_one_workgroup_in_the_engine(name, sharp_folders, monkeypatch):
+    """The row kernel that takes a (row, kv head) pair whole in one workgroup, inside the engine: forced for every
+    step of single tokens (it is chosen from 192 pairs on, which tiny models reach only with 64 requests: the second
+    half of this test), eagerly and in replayed graphs, with C's window of 24 keys and its second cache group.  Every
+    row is the plain model's within the configuration's bound, and the kernel is the one that ran."""
+    from inferflux_amd.kernels import attention, ops
+    folder, V = sharp_folders[name, "bfloat16"], TINY[name]["vocab_size"]
+    used = []
+    real = ops.attention_rows
+    monkeypatch.setattr(ops, "attention_rows", lambda *a: (used.append(a[-1]), real(*a))[1])
+    monkeypatch.setattr(attention, "ROW_WHOLE_MIN_PAIRS", 1)
+    runner = load_runner(folder, torch.bfloat16, num_pages=64, max_requests=4)
+    seqs = {r: seeded_ids(440 + i, n, V) for i, (r, n) in enumerate({"a": 130, "b": 47, "c": 200}.items())}
+    heads = {"a": 90, "b": 7, "c": 161}
+    for rid, ids in seqs.items():
+        runner.add_request(rid)
+        runner.step([StepEntry(rid, ids[:heads[rid]], [])])
+    got = {r: [] for r in seqs}
+    for k in range(39):
+        live = [r for r in seqs if heads[r] + k < len(seqs[r])]
+        logits = runner.step([StepEntry(r, [seqs[r][heads[r] + k]], [0]) for r in live]).float().cpu()
+        for i, r in enumerate(live):
+            got[r].append(logits[i].clone())
+    assert used and all(w >= 1 for w in used) and runner.graph_replays > 20
+    for r, rows in got.items():
+        want = plain_logits(folder, seqs[r])[heads[r]: heads[r] + len(rows)]
+        assert rel_err(torch.stack(rows), want) < tol("bfloat16", name), r
+
+
+def test_sixty_four_requests_decode_together(sharp_folders, monkeypatch):
+    """Sixty-four requests of configuration C (3 kv heads: 192 (row, kv head) pairs, from which on a pair is taken
+    whole by one workgroup) decode together after prompts of 3-60 tokens: every request's rows are the plain model's."""
+    from inferflux_amd.kernels import ops
+    folder, V = sharp_folders["C", "bfloat16"], TINY["C"]["vocab_size"]
+    used = []
+    real = ops.attention_rows
+    monkeypatch.setattr(ops, "attention_rows", lambda *a: (used.append(a[-1]), real(*a))[1])
+    runner = load_runner(folder, torch.bfloat16, num_pages=64 * 5, max_requests=64)
+    seqs = {r: seeded_ids(1500 + r, 3 + (r * 7) % 58 + 12, V) for r in range(64)}
+    for r, ids in seqs.items():
+        runner.add_request(r)
+    runner.step([StepEntry(r, ids[:-12], []) for r, ids in seqs.items()])          # all prompts in one step
+    rows = {r: [] for r in seqs}
+    for k in range(12):
+        logits = runner.step([StepEntry(r, [ids[len(ids) - 12 + k]], [0]) for r, ids in seqs.items()]).float().cpu()
+        for i, r in enumerate(seqs):
+            rows[r].append(logits[i].clone())
+    assert used and all(w >= 1 for w in used[-6:]), used[-6:]                        # decode steps of 64 rows: pairs taken whole
+    worst = max(rel_err(torch.stack(rows[r]), plain_logits(folder, seqs[r])[-12:]) for r in seqs)
+    assert worst < tol("bfloat16", "C"), worst
+    for r in seqs:
+        runner.free_request(r)
+    assert runner.manager.free_pages() == [64 * 5] * 2
+
+
 # ---- other toy parts: a position encoding of its own, a feed-forward with routing --------------------
 def test_toy_position_encoding_and_routed_feed_forward(tmp_path):
     """Two more parts defined here and registered from outside the package: a position encoding that
