@@ -9,7 +9,9 @@
 //          kv head are the 16 columns of the matrix tile, so keys and values are read once for
 //          all of them (any group size; more than 16 heads take several passes).  Partial
 //          results (max, sum, unnormalised output) go to scratch and a second kernel merges
-//          the splits.  For decode tokens and short portions.
+//          the splits.  For decode tokens and short portions.  Where the (row, kv head) pairs of a launch fill the
+//          chip by themselves, one workgroup of several waves takes a pair whole instead: its waves share the
+//          keys, meet in LDS and write the output (no scratch, no second kernel).
 //   tiles  one workgroup of 4 waves per (64 or 128 consecutive rows of one request, query head;
 //          -DTILE_QT=1 or 2 tiles of 16 rows per wave): key and value tiles of 64 positions are
 //          staged in LDS and shared by the 4 waves.  For long portions of prompts.  The keys can
@@ -131,11 +133,18 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   const int split = blockIdx.x, kvh = blockIdx.y, ri = blockIdx.z;
   const int lane = threadIdx.x, col = lane & 15, g4 = lane >> 4;
   const int row = a.rows ? a.rows[ri] : ri;
+  // A step in which every request brings one row (a decode step) says so: the row's request is the row itself, and
+  // without a window a split's first key does not depend on the row's position, so the split's block-table entries
+  // are asked for together with the position instead of after it (one trip to memory fewer before the first keys).
+  const bool early = a.req_is_row && a.window <= 0;
+  const int* early_table = a.block_table + (size_t)row * a.max_blocks;
+  const int early_base = split * a.chunk / a.P;
+  const int early_pages = (early && early_base + lane < a.max_blocks) ? early_table[early_base + lane] : -1;
   const int pos = a.positions[row];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int ka = max(lo, split * a.chunk), kb = min(pos + 1, (split + 1) * a.chunk);  // keys [ka, kb)
   const int ratio = a.nH / a.nKV;
-  const int* table = a.block_table + (size_t)a.row_req[row] * a.max_blocks;
+  const int* table = early ? early_table : a.block_table + (size_t)a.row_req[row] * a.max_blocks;
 
   for (int qt = 0; qt < ratio; qt += 16) {
     const int head = kvh * ratio + qt + col;
@@ -159,8 +168,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 
     RowBlock b0, b1;
     int j0 = (ka / 32) * 32;
-    int page_base = 0, pages = -1;
-    bool have_pages = false;
+    int page_base = early_base, pages = early_pages;
+    bool have_pages = early;
     // the table entries of the block of 32 keys from j: in ``pages`` already, or read now (64 entries from j's)
     auto table_for = [&](int j) {
       if (have_pages && (j + 31) / a.P - page_base < WAVE) return;
@@ -311,10 +320,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // (``max_splits`` * chunk must reach past every row's position; part_o / part_ml are the partial results).
 // ``waves`` 1-8: one workgroup of that many waves per (row, kv head), which shares the row's keys evenly and writes
 // the output itself; chunk, max_splits and the scratch are not used.
+// ``req_is_row``: the caller knows that row_req[r] == r for every row of the step (each request brings one row).
 extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_cache, void* out, const int* rows,
                              const int* row_req, const int* positions, const int* block_table, int max_blocks,
                              int n_rows, int nH, int nKV, int d, int page_size, int window, int chunk,
-                             int max_splits, float scale, float* part_o, float* part_ml, int waves, void* stream) {
+                             int max_splits, float scale, float* part_o, float* part_ml, int waves, int req_is_row,
+                             void* stream) {
   IFX_REQUIRE(d == D, "attn_rows: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_rows >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_rows: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_rows: page_size %d must be a multiple of 16", page_size);
@@ -323,7 +334,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   if (n_rows == 0) return 0;
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-            scale * 1.4426950408889634f, 0, waves};
+            scale * 1.4426950408889634f, 0, waves, req_is_row};
   hipStream_t s = (hipStream_t)stream;
   if (waves > 0) {
     const int nc = nH / nKV < 16 ? nH / nKV : 16;

@@ -81,6 +81,7 @@ struct RowArgs {
   float scale_log2e;
   int part_by_row;        // partial results lie at the batch row's number (the tile kernel's), not at its place in ``rows``
   int waves;              // the row kernel that takes a (row, kv head) whole: waves per workgroup
+  int req_is_row;         // row_req[r] == r for every row (a step of single tokens): table lookups need not wait for it
 };
 
 // out[row, head] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the row's splits, M = max m_s.

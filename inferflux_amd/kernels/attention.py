@@ -243,5 +243,5 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
                             ctx.positions, w["tile_order"])
     if w["n_rows"]:
         ops.attention_rows(q, cache.k, cache.v, out, w["rows"], w["n_rows"], ctx.row_req, ctx.positions, table,
-                           window, scale, w["chunk"], w["max_splits"], w["waves"])
+                           window, scale, w["chunk"], w["max_splits"], w["waves"], ctx.n_tokens == ctx.n_requests)
     return out

@@ -737,13 +737,15 @@ def row_waves_fit(n_heads: int, n_kv_heads: int, head_dim: int, waves: int) -> i
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                    rows: Optional[torch.Tensor], n_rows: int, row_req: torch.Tensor, positions: torch.Tensor,
                    block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int,
-                   waves: int = 0) -> None:
+                   waves: int = 0, req_is_row: bool = False) -> None:
     """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].
 
     ``waves`` 0: split s of a row covers key positions [s*chunk, (s+1)*chunk), one wave each, and a second launch
     merges a row's splits; ``max_splits`` * chunk must reach past the largest position among the rows.
     ``waves`` 1-8: one workgroup of that many waves per (row, kv head) shares the row's keys evenly and writes the
-    output itself (``chunk`` and ``max_splits`` are not used): for launches with pairs enough to fill the chip."""
+    output itself (``chunk`` and ``max_splits`` are not used): for launches with pairs enough to fill the chip.
+    ``req_is_row``: the caller vouches that ``row_req`` is 0, 1, 2, ... (every request brings one row), which lets
+    a wave ask for its block-table entries before it knows anything else."""
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache)
     _check(out, "out", (T, nH * d), torch.bfloat16)
     _check(row_req, "row_req", (T,), torch.int32)
@@ -760,10 +762,12 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if waves == 0:
         part_o = torch.empty((n_rows, nH, max_splits, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
-    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, P),
+    if req_is_row and block_table.shape[0] < T:
+        raise KernelError("attention_rows: req_is_row needs a block-table row for every row of the step")
+    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(rows), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_rows, nH, nKV, d, page_size,
-          int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, _stream())
+          int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, 1 if req_is_row else 0, _stream())
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:

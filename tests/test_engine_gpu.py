@@ -481,7 +481,7 @@ def test_decode_rows_taken_whole_by_one_workgroup_in_the_engine(name, sharp_fold
     folder, V = sharp_folders[name, "bfloat16"], TINY[name]["vocab_size"]
     used = []
     real = ops.attention_rows
-    monkeypatch.setattr(ops, "attention_rows", lambda *a: (used.append(a[-1]), real(*a))[1])
+    monkeypatch.setattr(ops, "attention_rows", lambda *a: (used.append(a[-2]), real(*a))[1])
     monkeypatch.setattr(attention, "ROW_WHOLE_MIN_PAIRS", 1)
     runner = load_runner(folder, torch.bfloat16, num_pages=64, max_requests=4)
     seqs = {r: seeded_ids(440 + i, n, V) for i, (r, n) in enumerate({"a": 130, "b": 47, "c": 200}.items())}
@@ -508,7 +508,7 @@ def test_sixty_four_requests_decode_together(sharp_folders, monkeypatch):
     folder, V = sharp_folders["C", "bfloat16"], TINY["C"]["vocab_size"]
     used = []
     real = ops.attention_rows
-    monkeypatch.setattr(ops, "attention_rows", lambda *a: (used.append(a[-1]), real(*a))[1])
+    monkeypatch.setattr(ops, "attention_rows", lambda *a: (used.append(a[-2]), real(*a))[1])
     runner = load_runner(folder, torch.bfloat16, num_pages=64 * 5, max_requests=64)
     seqs = {r: seeded_ids(1500 + r, 3 + (r * 7) % 58 + 12, V) for r in range(64)}
     for r, ids in seqs.items():

@@ -531,18 +531,23 @@ MFMA_CASES = [c for c in ATTN_CASES if c[4] % 16 == 0 and c[4] <= 128] + [
     # pages larger than a tile of 64 keys: where a tile's keys start inside their page changes from tile to tile
     ([200, 40], [300, 1000], 4, 2, 128, 128, None, 50),
     ([150], [700], 6, 2, 128, 256, 500, None),
+    # steps of single tokens (every request one row: the row kernel then looks its pages up before it knows the position)
+    ([1] * 9, [0, 5, 130, 700, 64, 31, 2000, 15, 16], 28, 4, 128, 16, None, 3),
+    ([1] * 5, [300, 1, 1030, 77, 512], 6, 3, 32, 64, None, None),
 ]
 
 
 def run_rows(q, kc, vc, row_req, positions, table, window, scale, rows=None, chunk=128, waves=0, extra_splits=0):
     """``waves`` 0: one wave per split of ``chunk`` keys and the merge launch (``extra_splits``: the grid reaches that
-    many splits past the longest row, as a captured step's does); 1-8: one workgroup of that many waves per (row, kv head)."""
+    many splits past the longest row, as a captured step's does); 1-8: one workgroup of that many waves per (row, kv head).
+    Where every request brings one row the kernel is told so, as the engine tells it."""
     T, nH, d = q.shape
+    req_is_row = bool(torch.equal(row_req.cpu(), torch.arange(T, dtype=torch.int32)))
     out = torch.zeros(T, nH * d, dtype=q.dtype, device=DEV)
     n = T if rows is None else rows.shape[0]
     max_kv = int(positions.max()) + 1
     ops.attention_rows(q, kc, vc, out, rows, n, row_req, positions, table, window, scale, chunk,
-                       -(-max_kv // chunk) + extra_splits, waves)
+                       -(-max_kv // chunk) + extra_splits, waves, req_is_row)
     return out
 
 
