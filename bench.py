@@ -5,8 +5,9 @@
 A step is one decode step of the whole engine (scheduler, step function, sampling).  Prints one
 JSON line: decoded tokens a second at batch 8 as ``value``, the same at batch 1 and 64 under
 ``points`` (with their step times and roofline shares under ``ms_per_step_b1`` / ``roofline_b1`` and
-``..._b64``), a 2,048-token prefill under ``prefill`` (the best of ``best_of`` runs with the library's
-kernels chosen by timing; ``prefill_untuned`` is the same with the library's default choice) and the
+``..._b64``), a 2,048-token prefill under ``prefill`` (the mean of ``mean_of`` runs with the library's
+kernels chosen by timing, the best of them as ``best_ms``; ``prefill_untuned`` is the same with the library's
+default choice, ``prefill_portions_512`` the same prompt in four portions of 512 tokens) and the
 decode step's share of the HBM roofline under ``roofline``.  Every share is given against the data
 sheet (``frac``) and, unless ``--no-ceilings``, against what this card gives a kernel that only reads
 memory or a large library product (``frac_measured``, the ceilings under ``ceilings``).
