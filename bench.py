@@ -332,7 +332,7 @@ def run_workload(args, w) -> int:
     import torch
     from inferflux_amd import SamplingParams
     from inferflux_amd.config import config_from_dict
-    from inferflux_amd.engine.engine import Engine
+    from inferflux_amd.engine.engine import Engine, quiet_garbage_collector
     from inferflux_amd.engine.model import Model
     from inferflux_amd.engine.runner import ModelRunner
     from inferflux_amd.engine.scheduler import SchedulerConfig
@@ -367,6 +367,7 @@ def run_workload(args, w) -> int:
         eng.stats = type(eng.stats)()
         print(f"[bench] warm-up pass done ({runner.graph_captures} decode layouts captured)", file=sys.stderr, flush=True)
     captures_before, replays_before = runner.graph_captures, runner.graph_replays
+    quiet_garbage_collector()               # as the command line does once its model is loaded
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     outs = eng.generate(prompts, sps(), on_token)

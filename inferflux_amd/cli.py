@@ -69,10 +69,11 @@ def load_spec_from_args(args):
 
 def cmd_completion(args) -> int:
     from . import SamplingParams
-    from .engine.engine import Engine
+    from .engine.engine import Engine, quiet_garbage_collector
     spec = load_spec_from_args(args)
     prompts = _read_ids(args)
     engine = Engine.load(spec)
+    quiet_garbage_collector()
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p,
                             frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
                             repetition_penalty=args.repetition_penalty, penalty_last_n=args.penalty_last_n,

@@ -203,10 +203,24 @@ struct SampleArgs {
   const int* top_k;
   const float* top_p;
   const float* min_p;
-  const float* uniform;  // one number in [0, 1) per row
+  const float* uniform;  // one number in [0, 1) per row, or null:
+  const unsigned* draws; // then [R, 4]: the row's seed and the number of its draw, 64 bits each, low word first
   int* out;
   int V;
 };
+
+// The top 24 bits of the first word of Philox4x32-10 (Salmon et al. 2011) keyed by the seed at counter (step, 0), as a
+// number in [0, 1): it depends on the pair alone, so a request draws the same numbers whatever shares its batch.
+__device__ float philox_uniform(unsigned seed_lo, unsigned seed_hi, unsigned step_lo, unsigned step_hi) {
+  unsigned c0 = step_lo, c1 = step_hi, c2 = 0, c3 = 0, k0 = seed_lo, k1 = seed_hi;
+  for (int round = 0; round < 10; ++round) {
+    const unsigned long long p0 = 0xD2511F53ull * c0, p1 = 0xCD9E8D57ull * c2;
+    const unsigned n0 = (unsigned)(p1 >> 32) ^ c1 ^ k0, n2 = (unsigned)(p0 >> 32) ^ c3 ^ k1;
+    c0 = n0; c1 = (unsigned)p1; c2 = n2; c3 = (unsigned)p0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return (float)(c0 >> 8) * (1.0f / 16777216.0f);
+}
 
 __device__ __forceinline__ int block_sum_int(int v, int* red) {
 #pragma unroll
@@ -220,128 +234,363 @@ __device__ __forceinline__ int block_sum_int(int v, int* red) {
   return t;
 }
 
+// Calls f(i, p[i]) for every i < n, each index from exactly one thread of the block, with 16-byte loads where the
+// row's address allows (a few of them in flight per thread: one workgroup has to keep a whole row moving).
+template <typename F>
+__device__ __forceinline__ void block_visit(const float* __restrict__ p, int n, F f) {
+  const int head = min(n, (int)(((16 - ((size_t)p & 15)) & 15) >> 2));
+  if ((int)threadIdx.x < head) f((int)threadIdx.x, p[threadIdx.x]);
+  const float4* p4 = reinterpret_cast<const float4*>(p + head);
+  const int n4 = (n - head) >> 2;
+#pragma unroll 4
+  for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+    const float4 v = p4[i];
+    const int b = head + 4 * i;
+    f(b, v.x); f(b + 1, v.y); f(b + 2, v.z); f(b + 3, v.w);
+  }
+  const int t = head + 4 * n4 + (int)threadIdx.x;
+  if (t < n) f(t, p[t]);
+}
+
+// q[i] = f(p[i]) for every i < n; 16-byte loads and stores where both rows' addresses allow.
+template <typename F>
+__device__ __forceinline__ void block_map(const float* __restrict__ p, float* __restrict__ q, int n, F f) {
+  if ((((size_t)p ^ (size_t)q) & 15) != 0) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) q[i] = f(p[i]);
+    return;
+  }
+  const int head = min(n, (int)(((16 - ((size_t)p & 15)) & 15) >> 2));
+  if ((int)threadIdx.x < head) q[threadIdx.x] = f(p[threadIdx.x]);
+  const float4* p4 = reinterpret_cast<const float4*>(p + head);
+  float4* q4 = reinterpret_cast<float4*>(q + head);
+  const int n4 = (n - head) >> 2;
+#pragma unroll 4
+  for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+    float4 v = p4[i];
+    v.x = f(v.x); v.y = f(v.y); v.z = f(v.z); v.w = f(v.w);
+    q4[i] = v;
+  }
+  const int t = head + 4 * n4 + (int)threadIdx.x;
+  if (t < n) q[t] = f(p[t]);
+}
+
 __device__ float kept_sum(const float* __restrict__ w, int V, float thr, float* red) {
   float s = 0.f;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const float x = w[i];
-    if (x >= thr) s += x;
-  }
+  block_visit(w, V, [&](int, float x) { if (x >= thr) s += x; });
   return block_sum(s, red);
 }
 
 __device__ int kept_count(const float* __restrict__ w, int V, float thr, int* red) {
   int c = 0;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) c += w[i] >= thr ? 1 : 0;
+  block_visit(w, V, [&](int, float x) { c += x >= thr ? 1 : 0; });
   return block_sum_int(c, red);
 }
 
+// The thresholds of top-k and top-p are exact selections among the weights of one row.  A histogram over the upper
+// bits of the weights' bit patterns (sign and exponent and the first HIST_MANTISSA bits of the mantissa: HIST_BINS
+// bins, the largest weight 1.0 falls into bin 2032) says which bin each threshold lies in; the weights from the
+// lower of these bins upwards (the candidates: usually a few hundred of the row) are gathered in LDS, and one
+// wave bisects over the bit patterns within the bin there.  Counts are integers and sums are sums of the
+// weights in fixed point (units of 2^-40, so a row of a million weights of 1.0 stays below 2^64): neither depends
+// on the order in which the threads add, and the histogram's sums and the candidates' agree exactly.  A row whose
+// candidates do not fit (a nearly flat distribution under top-p) bisects over the whole row instead.
+#define HIST_MANTISSA 4
+#define HIST_SHIFT (23 - HIST_MANTISSA)
+#define HIST_BINS 2048
+#define SAMPLE_CANDIDATES 8192
+typedef unsigned long long u64;
+
+__device__ __forceinline__ u64 weight_fixed(float x) { return (u64)(x * 1099511627776.0f); }   // x * 2^40, x in [0, 1]
+
+__device__ __forceinline__ u64 wave_sum_u64(u64 v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ int wave_sum_int(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+
+struct SampleShared {
+  float cand[SAMPLE_CANDIDATES];
+  unsigned count[HIST_BINS];     // after the scan: the number of weights in this bin or a higher one
+  u64 sum[HIST_BINS];            // after the scan: their sum in fixed point
+  unsigned wave_count[16];
+  u64 wave_sum[16];
+  float seg_sum[16];
+  int seg_last[16];
+  float red_f[16];
+  int red_i[16];
+  unsigned n_cand;
+  int bin_k, bin_p, bin_cand;
+  unsigned thr_bits;
+  int pick;
+};
+
+// count[b] and sum[b] (where SUMS) become the totals over the bins b and above.  Bin 0 (zero and the smallest
+// denormals) is not counted by the threads: it is given what is left of the V weights.  All SAMPLE_THREADS threads, two
+// bins each, the highest bins first.
+template <bool SUMS>
+__device__ void histogram_suffix_scan(unsigned* count, u64* sum, unsigned* wave_count, u64* wave_sum, int V) {
+  const int tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  const int b0 = HIST_BINS - 1 - 2 * tid, b1 = b0 - 1;
+  const unsigned c0 = count[b0], c1 = count[b1];
+  const u64 s0 = SUMS ? sum[b0] : 0, s1 = SUMS ? sum[b1] : 0;
+  unsigned ci = c0 + c1;
+  u64 si = s0 + s1;
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const unsigned oc = __shfl_up(ci, o, WAVE);
+    if (lane >= o) ci += oc;
+    if (SUMS) {
+      const u64 os = __shfl_up(si, o, WAVE);
+      if (lane >= o) si += os;
+    }
+  }
+  if (lane == WAVE - 1) {
+    wave_count[wid] = ci;
+    if (SUMS) wave_sum[wid] = si;
+  }
+  __syncthreads();
+  unsigned cb = 0;
+  u64 sb = 0;
+  for (int i = 0; i < wid; ++i) {
+    cb += wave_count[i];
+    if (SUMS) sb += wave_sum[i];
+  }
+  const unsigned ce = cb + ci - (c0 + c1);
+  count[b0] = ce + c0;
+  count[b1] = b1 == 0 ? (unsigned)V : ce + c0 + c1;
+  if (SUMS) {
+    const u64 se = sb + si - (s0 + s1);
+    sum[b0] = se + s0;
+    sum[b1] = se + s0 + s1;
+  }
+  __syncthreads();
+}
+
+// The largest bin in [lo, hi] whose entry of a non-increasing table is >= need; lo if none is (the caller knows that lo's is).
+template <typename T>
+__device__ __forceinline__ int last_bin_reaching(const T* table, T need, int lo, int hi) {
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[mid] >= need) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// The token at which the cumulative sum of the kept weights (those with bit pattern >= thr_bits), taken in index
+// order, passes uniform * total.  Two rounds in which the 16 waves each sum a sixteenth of the range and the part
+// that holds the target becomes the range, then one wave walks what is left, 64 weights at a time.  Every thread
+// returns the token.  A target that rounding puts past the end of a range gives the range's last kept index.
+__device__ int cumulative_pick(const float* __restrict__ w, int V, unsigned thr_bits, float uniform, SampleShared& sh) {
+  const int tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE, nw = blockDim.x / WAVE;
+  int lo = 0, hi = V;
+  float target = 0.f;
+  for (int level = 0; level < 2; ++level) {
+    const int seg = ((hi - lo + nw - 1) / nw + WAVE - 1) / WAVE * WAVE;
+    const int s0 = min(hi, lo + wid * seg), s1 = min(hi, s0 + seg);
+    float mine = 0.f;
+    int last = -1;
+#pragma unroll 4
+    for (int i = s0 + lane; i < s1; i += WAVE) {
+      const float x = w[i];
+      if (__float_as_uint(x) >= thr_bits) { mine += x; last = i; }
+    }
+    mine = wave_sum(mine);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) last = max(last, __shfl_xor(last, o, WAVE));
+    __syncthreads();   // the arrays may still be read from the round before
+    if (lane == 0) { sh.seg_sum[wid] = mine; sh.seg_last[wid] = last; }
+    __syncthreads();
+    if (level == 0) {
+      float total = 0.f;
+      for (int i = 0; i < nw; ++i) total += sh.seg_sum[i];
+      target = uniform * total;
+    }
+    int sel = -1, last_any = -1;
+    float before = 0.f;
+    for (int i = 0; i < nw; ++i) {
+      const float s = sh.seg_sum[i];
+      last_any = max(last_any, sh.seg_last[i]);
+      if (s > 0.f && target - before < s) { sel = i; break; }
+      before += s;
+    }
+    if (sel < 0) return max(last_any, 0);
+    target -= before;
+    lo = min(hi, lo + sel * seg);
+    hi = min(hi, lo + seg);
+  }
+  __syncthreads();
+  if (wid == 0) {
+    float run = 0.f;
+    int pick = -1, last = -1;
+    for (int g = lo; g < hi && pick < 0; g += WAVE) {
+      const int i = g + lane;
+      const float x = i < hi ? w[i] : 0.f;
+      const bool kept = i < hi && __float_as_uint(x) >= thr_bits;
+      float cum = kept ? x : 0.f;
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const float up = __shfl_up(cum, o, WAVE);
+        if (lane >= o) cum += up;
+      }
+      cum += run;
+      const u64 hit = __ballot(kept && target < cum);
+      const u64 any = __ballot(kept);
+      if (hit) pick = g + __ffsll((long long)hit) - 1;
+      if (any) last = g + 63 - __clzll((long long)any);
+      run = __shfl(cum, WAVE - 1, WAVE);
+    }
+    if (lane == 0) sh.pick = pick >= 0 ? pick : max(last, 0);
+  }
+  __syncthreads();
+  return sh.pick;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
-  __shared__ float red_f[16];
-  __shared__ int red_i[16];
-  __shared__ float part[SAMPLE_THREADS];
-  __shared__ int found;
-  const int r = blockIdx.x, V = a.V;
+  __shared__ SampleShared sh;
+  const int r = blockIdx.x, V = a.V, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
   const float* row = a.logits + (size_t)r * V;
   const float temp = a.temperature[r];
   if (!(temp > 0.f)) {
-    const int best = block_argmax(row, V, red_f, red_i);
-    if (threadIdx.x == 0) a.out[r] = best;
+    const int best = block_argmax(row, V, sh.red_f, sh.red_i);
+    if (tid == 0) a.out[r] = best;
     return;
   }
   float* w = a.weights + (size_t)r * V;
   const float inv_t = 1.0f / temp;
+  const int k = a.top_k[r];
+  const float top_p = a.top_p[r];
+  const bool k_on = k > 0 && k < V, p_on = top_p > 0.f && top_p < 1.f;
+
   float mx = -INFINITY;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
-  mx = block_max(mx, red_f);
-  for (int i = threadIdx.x; i < V; i += blockDim.x) w[i] = expf(row[i] * inv_t - mx);
-  __syncthreads();
+  block_visit(row, V, [&](int, float l) { mx = fmaxf(mx, l * inv_t); });
+  mx = block_max(mx, sh.red_f);
 
   // Thresholds as bit patterns: for non-negative floats the order of the values is the order
   // of their bits.  The largest weight is exp(0) = 1.
   const unsigned one_bits = __float_as_uint(1.0f);
   unsigned thr_bits = 0;  // keep everything
-  const int k = a.top_k[r];
-  if (k > 0 && k < V) {
-    unsigned lo = 0, hi = one_bits;  // count(w >= f(lo)) >= k holds for lo = 0
-    while (lo < hi) {
-      const unsigned mid = lo + (hi - lo + 1) / 2;
-      if (kept_count(w, V, __uint_as_float(mid), red_i) >= k) lo = mid; else hi = mid - 1;
+  if (!k_on && !p_on) {
+    block_map(row, w, V, [&](float l) { return expf(l * inv_t - mx); });
+    __syncthreads();
+  } else {
+    for (int b = tid; b < HIST_BINS; b += blockDim.x) { sh.count[b] = 0; sh.sum[b] = 0; }
+    if (tid == 0) sh.n_cand = 0;
+    __syncthreads();
+    block_map(row, w, V, [&](float l) {
+      const float x = expf(l * inv_t - mx);
+      const unsigned b = __float_as_uint(x) >> HIST_SHIFT;
+      if (b && b < HIST_BINS) {   // (a NaN's pattern lies beyond the last bin)
+        atomicAdd(&sh.count[b], 1u);
+        atomicAdd(&sh.sum[b], weight_fixed(x));
+      }
+      return x;
+    });
+    __syncthreads();
+    histogram_suffix_scan<true>(sh.count, sh.sum, sh.wave_count, sh.wave_sum, V);
+    if (tid == 0) {
+      const int top_bin = one_bits >> HIST_SHIFT;
+      int bk = 0, bp = 0, bc = top_bin;
+      if (k_on) { bk = last_bin_reaching(sh.count, (unsigned)k, 0, top_bin); bc = min(bc, bk); }
+      if (p_on) {
+        // at least what the exact rule will ask for: top-k keeps no more than the bins from bk upwards hold
+        const u64 need = (u64)((double)top_p * (double)sh.sum[bk]);
+        bp = last_bin_reaching(sh.sum, need, 0, top_bin);
+        bc = min(bc, bp);
+      }
+      sh.bin_k = bk; sh.bin_p = bp; sh.bin_cand = bc;
     }
-    thr_bits = lo;
-  }
-  const float top_p = a.top_p[r];
-  if (top_p > 0.f && top_p < 1.f) {
-    const float need = top_p * kept_sum(w, V, __uint_as_float(thr_bits), red_f);
-    unsigned lo = thr_bits, hi = one_bits;  // sum(w >= f(lo)) >= need holds for lo = thr_bits
-    while (lo < hi) {
-      const unsigned mid = lo + (hi - lo + 1) / 2;
-      if (kept_sum(w, V, __uint_as_float(mid), red_f) >= need) lo = mid; else hi = mid - 1;
+    __syncthreads();
+    const int bk = sh.bin_k, bc = sh.bin_cand;
+    if (sh.count[bc] <= SAMPLE_CANDIDATES) {
+      const unsigned first_bits = (unsigned)bc << HIST_SHIFT;
+      block_visit(w, V, [&](int, float x) {
+        if (__float_as_uint(x) >= first_bits) {
+          const unsigned at = atomicAdd(&sh.n_cand, 1u);
+          if (at < SAMPLE_CANDIDATES) sh.cand[at] = x;
+        }
+      });
+      __syncthreads();
+      if (wid == 0) {
+        const int n = min(sh.n_cand, (unsigned)SAMPLE_CANDIDATES);
+        if (k_on) {  // the largest pattern that at least k weights reach: it lies in bin bk
+          unsigned lo = (unsigned)bk << HIST_SHIFT, hi = min(((unsigned)(bk + 1) << HIST_SHIFT) - 1, one_bits);
+          while (lo < hi) {
+            const unsigned mid = lo + (hi - lo + 1) / 2;
+            int c = 0;
+            for (int i = lane; i < n; i += WAVE) c += __float_as_uint(sh.cand[i]) >= mid ? 1 : 0;
+            if (wave_sum_int(c) >= k) lo = mid; else hi = mid - 1;
+          }
+          thr_bits = lo;
+        }
+        if (p_on) {  // the largest pattern whose weights and all larger ones sum to top_p of what top-k kept
+          u64 kept = 0;
+          for (int i = lane; i < n; i += WAVE) {
+            const float x = sh.cand[i];
+            if (__float_as_uint(x) >= thr_bits) kept += weight_fixed(x);
+          }
+          const u64 kept_all = k_on ? wave_sum_u64(kept) : sh.sum[0];   // without top-k: the whole row, not the candidates
+          const u64 need = (u64)((double)top_p * (double)kept_all);
+          const int tb = thr_bits >> HIST_SHIFT;
+          const int b = last_bin_reaching(sh.sum, need, tb, (int)(one_bits >> HIST_SHIFT));
+          unsigned lo = max(thr_bits, (unsigned)b << HIST_SHIFT), hi = min(((unsigned)(b + 1) << HIST_SHIFT) - 1, one_bits);
+          while (lo < hi) {
+            const unsigned mid = lo + (hi - lo + 1) / 2;
+            u64 s = 0;
+            for (int i = lane; i < n; i += WAVE) {
+              const float x = sh.cand[i];
+              if (__float_as_uint(x) >= mid) s += weight_fixed(x);
+            }
+            if (wave_sum_u64(s) >= need) lo = mid; else hi = mid - 1;
+          }
+          thr_bits = lo;
+        }
+        if (lane == 0) sh.thr_bits = thr_bits;
+      }
+      __syncthreads();
+      thr_bits = sh.thr_bits;
+    } else {
+      if (k_on) {
+        unsigned lo = 0, hi = one_bits;  // count(w >= f(lo)) >= k holds for lo = 0
+        while (lo < hi) {
+          const unsigned mid = lo + (hi - lo + 1) / 2;
+          if (kept_count(w, V, __uint_as_float(mid), sh.red_i) >= k) lo = mid; else hi = mid - 1;
+        }
+        thr_bits = lo;
+      }
+      if (p_on) {
+        const float need = top_p * kept_sum(w, V, __uint_as_float(thr_bits), sh.red_f);
+        unsigned lo = thr_bits, hi = one_bits;  // sum(w >= f(lo)) >= need holds for lo = thr_bits
+        while (lo < hi) {
+          const unsigned mid = lo + (hi - lo + 1) / 2;
+          if (kept_sum(w, V, __uint_as_float(mid), sh.red_f) >= need) lo = mid; else hi = mid - 1;
+        }
+        thr_bits = lo;
+      }
     }
-    thr_bits = lo;
   }
   const float min_p = a.min_p[r];
   if (min_p > 0.f) {
     const unsigned mb = __float_as_uint(fminf(min_p, 1.0f));
     if (mb > thr_bits) thr_bits = mb;
   }
-  const float thr = __uint_as_float(thr_bits);
-
-  // Cumulative walk in index order: thread t owns the indices [t*chunk, (t+1)*chunk).
-  const int chunk = (V + blockDim.x - 1) / blockDim.x;
-  const int c0 = min(V, (int)threadIdx.x * chunk), c1 = min(V, c0 + chunk);
-  float mine = 0.f;
-  int last_kept = -1;
-  for (int i = c0; i < c1; ++i)
-    if (w[i] >= thr) { mine += w[i]; last_kept = i; }
-  part[threadIdx.x] = mine;
-  if (threadIdx.x == 0) found = -1;
-  __syncthreads();
-  if (threadIdx.x == 0) {  // exclusive prefix in place, sequential: one fixed order of additions
-    float run = 0.f;
-    for (int t = 0; t < (int)blockDim.x; ++t) { const float v = part[t]; part[t] = run; run += v; }
-    red_f[0] = run;
-  }
-  __syncthreads();
-  const float total = red_f[0];
-  const float target = a.uniform[r] * total;
-  const float before = part[threadIdx.x];
-  const float after = threadIdx.x + 1 < blockDim.x ? part[threadIdx.x + 1] : total;
-  if (mine > 0.f && before <= target && target < after) {
-    float cum = before;
-    int pick = last_kept;
-    for (int i = c0; i < c1; ++i) {
-      if (w[i] >= thr) {
-        cum += w[i];
-        if (target < cum) { pick = i; break; }
-      }
-    }
-    found = pick;
-  }
-  // Fallback (target >= total through rounding): the last kept index.
-  int lk = last_kept;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) lk = max(lk, __shfl_xor(lk, o, WAVE));
-  const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, nw = blockDim.x / WAVE;
-  __syncthreads();
-  if (lane == 0) red_i[wid] = lk;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int best = found;
-    if (best < 0) {
-      best = red_i[0];
-      for (int i = 1; i < nw; ++i) best = max(best, red_i[i]);
-      if (best < 0) best = 0;
-    }
-    a.out[r] = best;
-  }
+  const float u = a.uniform ? a.uniform[r]
+                            : philox_uniform(a.draws[4 * r], a.draws[4 * r + 1], a.draws[4 * r + 2], a.draws[4 * r + 3]);
+  const int pick = cumulative_pick(w, V, thr_bits, u, sh);
+  if (tid == 0) a.out[r] = pick;
 }
 
 extern "C" int ifx_sample(const float* logits, float* weights, const float* temperature, const int* top_k,
-                          const float* top_p, const float* min_p, const float* uniform, int* out, int R, int V,
-                          void* stream) {
+                          const float* top_p, const float* min_p, const float* uniform, const unsigned* draws, int* out,
+                          int R, int V, void* stream) {
   IFX_REQUIRE(R >= 0 && V > 0, "sample: bad sizes R=%d V=%d", R, V);
+  IFX_REQUIRE((uniform != nullptr) != (draws != nullptr), "sample: either the uniform numbers or the seeds and counters of the draws");
   if (R == 0) return 0;
-  SampleArgs a{logits, weights, temperature, top_k, top_p, min_p, uniform, out, V};
+  SampleArgs a{logits, weights, temperature, top_k, top_p, min_p, uniform, draws, out, V};
   hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, a);
   IFX_LAUNCH_CHECK();
 }
@@ -354,46 +603,117 @@ extern "C" int ifx_sample(const float* logits, float* weights, const float* temp
 // equals).  The k-th is found as the largest element that comes after the (k-1)-th in that
 // order, so the logits are not modified.
 #define MAX_TOP_LOGPROBS 20
+#define LOGPROB_CANDIDATES 4096
 
+struct LogprobShared {
+  float cand_v[LOGPROB_CANDIDATES];
+  int cand_i[LOGPROB_CANDIDATES];
+  unsigned count[HIST_BINS];
+  unsigned wave_count[16];
+  float red_f[16];
+  float red_v[16];
+  int red_i[16];
+  unsigned n_cand;
+  int bin;
+};
+
+// The top_n are looked for among few candidates where that is possible: the pass that sums exp(l - max) also counts the
+// terms by the upper bits of their patterns (the histogram of the sampling kernel), the logits whose terms reach the
+// bin below the one that holds the top_n-th (a bin's width is far more than what rounding could do to the order of
+// two terms) are gathered in LDS with their indices, and one wave picks from them.  A row whose candidates do not fit
+// (its top_n-th logit among thousands of near-equal ones, or fewer than top_n finite logits) takes one pass over the
+// whole row per rank instead.
 __global__ __launch_bounds__(SAMPLE_THREADS) void logprobs_kernel(const float* __restrict__ logits, const int* __restrict__ chosen,
                                                                  int V, int top_n, float* __restrict__ lp,
                                                                  int* __restrict__ top_ids, float* __restrict__ top_lp) {
-  __shared__ float red_f[16];
-  __shared__ float red_v[16];
-  __shared__ int red_i[16];
-  const int r = blockIdx.x;
+  __shared__ LogprobShared sh;
+  const int r = blockIdx.x, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE, nw = blockDim.x / WAVE;
   const float* row = logits + (size_t)r * V;
   float mx = -INFINITY;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i]);
-  mx = block_max(mx, red_f);
+  block_visit(row, V, [&](int, float l) { mx = fmaxf(mx, l); });
+  mx = block_max(mx, sh.red_f);
+  if (top_n > 0) {
+    for (int b = tid; b < HIST_BINS; b += blockDim.x) sh.count[b] = 0;
+    if (tid == 0) sh.n_cand = 0;
+    __syncthreads();
+  }
   float sum = 0.f;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) sum += expf(row[i] - mx);
-  sum = block_sum(sum, red_f);
+  block_visit(row, V, [&](int, float l) {
+    const float x = expf(l - mx);
+    sum += x;
+    if (top_n > 0) {
+      const unsigned b = __float_as_uint(x) >> HIST_SHIFT;
+      if (b && b < HIST_BINS) atomicAdd(&sh.count[b], 1u);
+    }
+  });
+  sum = block_sum(sum, sh.red_f);
   const float lse = mx + logf(sum);
-  if (threadIdx.x == 0) lp[r] = row[chosen[r]] - lse;
+  if (tid == 0) lp[r] = row[chosen[r]] - lse;
+  if (top_n <= 0) return;
+  histogram_suffix_scan<false>(sh.count, nullptr, sh.wave_count, nullptr, V);
+  if (tid == 0) {
+    const int bn = last_bin_reaching(sh.count, (unsigned)top_n, 0, (int)(__float_as_uint(1.0f) >> HIST_SHIFT));
+    sh.bin = max(bn - 1, 0);
+  }
+  __syncthreads();
+  const int bc = sh.bin;
+  if (sh.count[bc] <= LOGPROB_CANDIDATES) {
+    const unsigned first_bits = (unsigned)bc << HIST_SHIFT;
+    block_visit(row, V, [&](int i, float l) {
+      if (__float_as_uint(expf(l - mx)) >= first_bits) {
+        const unsigned at = atomicAdd(&sh.n_cand, 1u);
+        if (at < LOGPROB_CANDIDATES) { sh.cand_v[at] = l; sh.cand_i[at] = i; }
+      }
+    });
+    __syncthreads();
+    if (wid != 0) return;
+    const int n = min(sh.n_cand, (unsigned)LOGPROB_CANDIDATES);
+    float last_v = INFINITY;
+    int last_i = -1;
+    for (int k = 0; k < top_n; ++k) {
+      float bv = -INFINITY;
+      int bi = V;
+      for (int j = lane; j < n; j += WAVE) {
+        const float x = sh.cand_v[j];
+        const int i = sh.cand_i[j];
+        const bool after = x < last_v || (x == last_v && i > last_i);   // not yet reported
+        if (after && (x > bv || (x == bv && i < bi))) { bv = x; bi = i; }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, WAVE);
+        const int oi = __shfl_xor(bi, o, WAVE);
+        argmax_merge(bv, bi, ov, oi);
+      }
+      if (lane == 0) {
+        top_ids[r * top_n + k] = bi < V ? bi : -1;
+        top_lp[r * top_n + k] = bi < V ? bv - lse : -INFINITY;
+      }
+      last_v = bv; last_i = bi;
+    }
+    return;
+  }
   float last_v = INFINITY;
   int last_i = -1;
   for (int k = 0; k < top_n; ++k) {
     float bv = -INFINITY;
     int bi = V;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-      const float x = row[i];
+    block_visit(row, V, [&](int i, float x) {
       const bool after = x < last_v || (x == last_v && i > last_i);   // not yet reported
       if (after && (x > bv || (x == bv && i < bi))) { bv = x; bi = i; }
-    }
+    });
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
       const float ov = __shfl_xor(bv, o, WAVE);
       const int oi = __shfl_xor(bi, o, WAVE);
       argmax_merge(bv, bi, ov, oi);
     }
-    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, nw = blockDim.x / WAVE;
     __syncthreads();
-    if (lane == 0) { red_v[wid] = bv; red_i[wid] = bi; }
+    if (lane == 0) { sh.red_v[wid] = bv; sh.red_i[wid] = bi; }
     __syncthreads();
-    bv = red_v[0]; bi = red_i[0];
-    for (int w = 1; w < nw; ++w) argmax_merge(bv, bi, red_v[w], red_i[w]);
-    if (threadIdx.x == 0) {
+    bv = sh.red_v[0]; bi = sh.red_i[0];
+    for (int w = 1; w < nw; ++w) argmax_merge(bv, bi, sh.red_v[w], sh.red_i[w]);
+    if (tid == 0) {
       top_ids[r * top_n + k] = bi < V ? bi : -1;
       top_lp[r * top_n + k] = bi < V ? bv - lse : -INFINITY;
     }

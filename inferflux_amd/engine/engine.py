@@ -55,6 +55,16 @@ class _Live:
         self.sampling = SamplingState.start(params)
 
 
+def quiet_garbage_collector() -> None:
+    """For a process that is about to serve: collect once, then move everything alive now (the interpreter's and the
+    libraries' millions of objects, the loaded model) out of the collector's sight.  A full collection walks all of them
+    (tens of milliseconds with torch imported) and comes every few hundred steps of a busy engine otherwise.  What
+    is alive now is then only freed by reference counts, so this is for the entry points to call, not the library."""
+    import gc
+    gc.collect()
+    gc.freeze()
+
+
 class Engine:
     def __init__(self, runner: ModelRunner, scheduler_config: Optional[SchedulerConfig] = None,
                  start_steps_early: bool = True):

@@ -868,20 +868,29 @@ def add_logit_bias(logits: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, 
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           min_p: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
-    """One token per row of float32 ``logits`` [R, V]; rows with temperature <= 0 take the argmax."""
+           min_p: torch.Tensor, uniform: Optional[torch.Tensor] = None, draws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of float32 ``logits`` [R, V]; rows with temperature <= 0 take the argmax.  The number in
+    [0, 1) that a row's draw uses is either given (``uniform`` [R]) or made by the kernel from ``draws`` (int32
+    [R, 4]: the row's seed and the count of its draws so far, 64 bits each, low word first), as
+    ``sampling.params.philox_uniform`` makes it."""
     _check(logits, "logits", (None, None), torch.float32)
     R, V = logits.shape
     _check(temperature, "temperature", (R,), torch.float32)
     _check(top_k, "top_k", (R,), torch.int32)
     _check(top_p, "top_p", (R,), torch.float32)
     _check(min_p, "min_p", (R,), torch.float32)
-    _check(uniform, "uniform", (R,), torch.float32)
+    if (uniform is None) == (draws is None):
+        raise KernelError("sample: either uniform numbers or seeds and counters")
+    if uniform is not None:
+        _check(uniform, "uniform", (R,), torch.float32)
+    else:
+        _check(draws, "draws", (R, 4), torch.int32)
     weights = torch.empty_like(logits)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    _call(load_module("sampling"), "ifx_sample", (P, P, P, P, P, P, P, P, I, I, P),
+    _call(load_module("sampling"), "ifx_sample", (P, P, P, P, P, P, P, P, P, I, I, P),
           logits.data_ptr(), weights.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
-          min_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), R, V, _stream())
+          min_p.data_ptr(), uniform.data_ptr() if uniform is not None else None,
+          draws.data_ptr() if draws is not None else None, out.data_ptr(), R, V, _stream())
     return out
 
 

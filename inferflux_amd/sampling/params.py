@@ -53,6 +53,8 @@ class SamplingParams:
             raise ValueError("penalty_last_n must be >= 0 and max_tokens >= 1")
         if self.logprobs is not None and not (0 <= self.logprobs <= 20):
             raise ValueError("logprobs must be None or between 0 and 20")
+        if not (0 <= int(self.seed) < 1 << 64):
+            raise ValueError("seed must be a non-negative number of at most 64 bits")
 
     @property
     def greedy(self) -> bool:

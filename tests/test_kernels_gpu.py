@@ -1,6 +1,7 @@
 """Each HIP kernel alone against a plain float64 reference of the same operation, at sizes other
 than the tiny models' (widths that are no power of two, odd row counts, several head sizes)."""
 import math
+import numpy as np
 
 import pytest
 import torch
@@ -495,6 +496,55 @@ def test_sample_random_vocabularies_and_filters(seed):
         cum = torch.cumsum(w, 0) / w.sum()
         lo = float(cum[got[r] - 1]) if got[r] > 0 else 0.0
         assert lo - 1e-4 <= float(u[r]) <= float(cum[got[r]]) + 1e-4, (case, got[r], lo, float(u[r]), float(cum[got[r]]))
+
+
+SAMPLE_SHAPES = [
+    # (name, V, logits builder, temperature, top_k, top_p, min_p)
+    ("flat under top-p", 40001, lambda g, V: 0.01 * torch.randn(V, generator=g), 1.0, 0, 0.9, 0.0),
+    ("flat under a wide top-k", 40001, lambda g, V: 0.01 * torch.randn(V, generator=g), 0.7, 20000, 1.0, 0.0),
+    ("flat under both", 30003, lambda g, V: 0.02 * torch.randn(V, generator=g), 1.0, 12000, 0.95, 0.0),
+    ("one token far above", 152064, lambda g, V: torch.randn(V, generator=g).index_fill_(0, torch.tensor([77777]), 40.0), 1.0, 50, 0.9, 0.0),
+    ("mostly masked", 9999, lambda g, V: torch.where(torch.rand(V, generator=g) < 0.9, torch.tensor(-float("inf")), 2.0 * torch.randn(V, generator=g)), 0.8, 40, 0.9, 0.0),
+    ("top-p alone, peaked", 152064, lambda g, V: 6.0 * torch.randn(V, generator=g), 0.6, 0, 0.95, 0.0),
+    ("top-p alone, wide", 152064, lambda g, V: 1.5 * torch.randn(V, generator=g), 1.0, 0, 0.9, 0.0),
+]
+
+
+@pytest.mark.parametrize("case", range(len(SAMPLE_SHAPES)), ids=[c[0] for c in SAMPLE_SHAPES])
+def test_sample_rows_of_every_shape(case):
+    """Rows that the thresholds' two ways take differently: few candidates above the thresholds' bins (gathered and
+    bisected by one wave) and more than fit (bisected over the whole row), equal weights (kept or dropped together), rows
+    that are mostly masked, and a vocabulary that is no multiple of four (rows that start at any address)."""
+    name, V, build, temp, k, p, mp = SAMPLE_SHAPES[case]
+    g = gen(1500 + case)
+    R = 5
+    logits = torch.stack([build(g, V) for _ in range(R)])
+    u = torch.tensor([0.0, 0.25, 0.5, 0.75, 0.999999])
+    full = lambda v, dt: torch.full((R,), v, dtype=dt, device=DEV)
+    got = ops.sample(logits.to(DEV), full(temp, torch.float32), full(k, torch.int32), full(p, torch.float32),
+                     full(mp, torch.float32), u.to(DEV)).cpu().tolist()
+    for r in range(R):
+        w = pm.filtered_probs(logits[r], temp, k, p, mp)
+        assert w[got[r]] > 0, (name, r, "a filtered-out token was drawn")
+        cum = torch.cumsum(w.double(), 0) / w.double().sum()
+        lo = float(cum[got[r] - 1]) if got[r] > 0 else 0.0
+        assert lo - 1e-4 <= float(u[r]) <= float(cum[got[r]]) + 1e-4, (name, r, got[r], lo, float(u[r]), float(cum[got[r]]))
+
+
+@pytest.mark.parametrize("V,every,k,p", [(5000, 1, 10, 0.5), (20000, 7, 100, 0.8), (152064, 3, 0, 0.3)])
+def test_sample_keeps_equal_weights_together(V, every, k, p):
+    """Tokens of equal weight are kept or dropped together: with every ``every``-th token at one logit and the rest far
+    below, top-k and top-p smaller than that group keep all of it, and the draw falls evenly over it.  (All threads
+    of a wave then add to one bin of the histogram: the slowest row there is.)"""
+    logits = torch.where(torch.arange(V) % every == 0, torch.tensor(3.0), torch.tensor(-9.0)).repeat(4, 1)
+    u = torch.tensor([0.0, 0.3, 0.6, 0.95])
+    full = lambda v, dt: torch.full((4,), v, dtype=dt, device=DEV)
+    got = ops.sample(logits.to(DEV), full(1.0, torch.float32), full(k, torch.int32), full(p, torch.float32),
+                     full(0.0, torch.float32), u.to(DEV)).cpu().tolist()
+    n = (V + every - 1) // every
+    for r in range(4):
+        assert got[r] % every == 0, (r, got[r])
+        assert abs(got[r] // every - float(u[r]) * n) <= 1 + 1e-4 * n, (r, got[r], float(u[r]) * n)
 
 
 def test_sample_histogram_follows_the_probabilities():
@@ -1362,6 +1412,58 @@ def test_logprobs_against_log_softmax_and_topk():
         assert torch.allclose(tlp[r].double(), want[r, order], atol=1e-4)
     assert ids[1, :2].tolist() == [7, 100]
     assert ops.logprobs(logits.to(DEV), chosen.to(DEV), 0)[1].shape == (R, 0)
+
+
+LOGPROB_ROWS = [
+    ("wide", 152064, lambda g, V: 3.0 * torch.randn(V, generator=g)),
+    ("one token far above", 152063, lambda g, V: torch.randn(V, generator=g).index_fill_(0, torch.tensor([40000]), 60.0)),
+    ("flat: more near-equal logits than candidates fit", 30001, lambda g, V: 1e-3 * torch.randn(V, generator=g)),
+    ("all equal", 9000, lambda g, V: torch.zeros(V)),
+    ("fewer finite logits than ranks", 5000, lambda g, V: torch.full((V,), -float("inf")).index_put_((torch.tensor([3, 4000, 77]),), torch.tensor([1.0, 2.0, 1.0]))),
+    ("fewer tokens than ranks", 5, lambda g, V: torch.randn(V, generator=g)),
+    ("the ranks far apart", 70000, lambda g, V: (-200.0 + torch.randn(V, generator=g)).index_put_((torch.arange(8) * 9000,), 100.0 - 35.0 * torch.arange(8.0))),
+]
+
+
+@pytest.mark.parametrize("case", range(len(LOGPROB_ROWS)), ids=[c[0] for c in LOGPROB_ROWS])
+def test_logprobs_rows_of_every_shape(case):
+    """The most probable tokens where they are picked from few candidates and where the whole row is searched per rank:
+    order by value, then index; ranks beyond the vocabulary come back as -1 and -inf."""
+    name, V, build = LOGPROB_ROWS[case]
+    g = gen(1600 + case)
+    R, N = 3, 8
+    logits = torch.stack([build(g, V) for _ in range(R)])
+    chosen = torch.tensor([int(logits[r].argmax()) for r in range(R)], dtype=torch.int32)
+    lp, ids, tlp = (t.cpu() for t in ops.logprobs(logits.to(DEV), chosen.to(DEV), N))
+    want = torch.log_softmax(logits.double(), -1)
+    assert torch.allclose(lp.double(), want[torch.arange(R), chosen.long()], atol=1e-4), name
+    for r in range(R):
+        order = sorted(range(V), key=lambda i: (-float(logits[r, i]), i))[:N]
+        assert ids[r, :len(order)].tolist() == order, (name, r)              # (masked tokens rank last, by index)
+        assert torch.allclose(tlp[r, :len(order)].double(), want[r, order], atol=1e-4, rtol=1e-5), (name, r)
+        assert ids[r, len(order):].tolist() == [-1] * (N - len(order)) and bool((tlp[r, len(order):] == -float("inf")).all())
+
+
+def test_sample_draws_its_own_numbers_as_the_host_does():
+    """Given seeds and counters instead of numbers in [0, 1), the kernel makes the number params.philox_uniform makes:
+    the same tokens either way, with seeds and counters beyond 32 bits among them."""
+    from inferflux_amd.sampling.params import philox_uniform
+    R, V = 64, 5000
+    g = gen(31)
+    logits = 0.5 * torch.randn(R, V, generator=g)
+    seeds = np.array([0, 1, 2**32 - 1, 2**32, 2**63 + 5, 2**64 - 1] + [int(x) for x in torch.randint(0, 2**62, (R - 6,), generator=g)], dtype=np.uint64)
+    steps = np.array([0, 2**32, 7, 2**40 + 3, 1, 2**64 - 1] + list(range(R - 6)), dtype=np.uint64)
+    draws = torch.from_numpy(np.stack([seeds, steps], 1).view(np.uint32).view(np.int32).reshape(R, 4)).to(DEV)
+    u = torch.from_numpy(philox_uniform(seeds, steps)).to(DEV)
+    full = lambda v, dt: torch.full((R,), v, dtype=dt, device=DEV)
+    a = (logits.to(DEV), full(1.0, torch.float32), full(0, torch.int32), full(1.0, torch.float32), full(0.0, torch.float32))
+    by_kernel = ops.sample(*a, draws=draws).cpu().tolist()
+    assert by_kernel == ops.sample(*a, uniform=u).cpu().tolist()
+    assert len(set(by_kernel)) > R // 2                                  # and they are not all one token
+    with pytest.raises(ops.KernelError, match="either"):
+        ops.sample(*a)
+    with pytest.raises(ops.KernelError, match="either"):
+        ops.sample(*a, uniform=u, draws=draws)
 
 
 def test_measurement_kernels_copy_what_they_read():
