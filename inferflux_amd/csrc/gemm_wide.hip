@@ -37,7 +37,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 constexpr int DEPTH = 3;                                           // rounds of W and x on their way
-constexpr int MIN_WAVES = 8, MAX_WAVES = 16;
+constexpr int MIN_WAVES = 8, MAX_WAVES = 16;                     // of the kernel's usual form
+constexpr int FEW_WAVES = 4;                                       // of its form for workgroups of 4-7 waves (up to MANY_ROWS rows)
 constexpr int MAX_ROWS = 128, MANY_ROWS = 64;                     // beyond MANY_ROWS a workgroup has exactly MIN_WAVES waves
 constexpr int WK = 128, WK_TILES = WK / 32, WK_PIECES = WK / 8;   // k-values, k-tiles and 16-byte pieces of a round
 
@@ -66,14 +67,16 @@ __device__ __forceinline__ void store2(bf16_t* p, float a, float b) {
 
 // EPI 0: out[m, n] = sum.  EPI 1: the rows of W alternate gate, up, ...: out[m, n / 2] = silu(gate) * up.
 // ``order``: tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
-template <int MT, typename TO, int EPI>
-__global__ __launch_bounds__((16 * MT > MANY_ROWS ? MIN_WAVES : MAX_WAVES) * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
+// ``MINW``: the fewest waves a workgroup of this form may have (each thread then copies more pieces of x to LDS and
+// holds them in more registers, which a workgroup of at most 8 waves has).
+template <int MT, typename TO, int EPI, int MINW>
+__global__ __launch_bounds__((16 * MT > MANY_ROWS || MINW < MIN_WAVES ? MIN_WAVES : MAX_WAVES) * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
                                                                      TO* __restrict__ out, float* __restrict__ part, int M,
                                                                      int N, int K, int k_tiles, int rounds_per_slice,
                                                                      const int* __restrict__ order, int tile_rows) {
   constexpr int R = MT * 16;                                  // rows of x in LDS
   constexpr int X_PIECES = R * WK_PIECES;                     // 16-byte pieces of a round's x
-  constexpr int X_PER_THREAD = (X_PIECES + MIN_WAVES * WAVE - 1) / (MIN_WAVES * WAVE);
+  constexpr int X_PER_THREAD = (X_PIECES + MINW * WAVE - 1) / (MINW * WAVE);
   __shared__ __attribute__((aligned(16))) bf16x8 xs[2][X_PIECES];
   const int tid = threadIdx.x, threads = blockDim.x, waves = threads / WAVE;
   const int wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g = lane >> 4;
@@ -216,20 +219,27 @@ extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S
 
 // Waves per workgroup and slices of K for a shape.  ``waves`` / ``slices`` 0: chosen here (about one workgroup
 // for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
-// several workgroups to a unit; 8 waves for more than 64 rows; then slices of at least four rounds, at most eight);
+// several workgroups to a unit; 8 waves for more than 64 rows; then slices of at least two rounds, at most eight);
 // the gate/up epilogue takes one slice.  Returns waves * 256 + slices.
+// Fewer than 8 waves are chosen for 33-64 rows only: there the tall weights of narrow models (gate/up with 600-1,700
+// tiles) take 4-17 % less time with one workgroup of 4-7 waves on every unit than with 8 waves on two thirds of
+// them; up to 32 rows the form for few waves is the slower one at every shape measured.
 extern "C" int ifx_wide_gemm_plan(int rows, int N, int K, int waves, int slices, int epi, int tile_rows) {
   if (tile_rows < 8 || tile_rows > 16) tile_rows = 16;
   const int n_tiles = (N + tile_rows - 1) / tile_rows, n_rounds = (K + WK - 1) / WK;
-  if (waves <= 0) waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
-  waves = waves < MIN_WAVES ? MIN_WAVES : (waves > MAX_WAVES ? MAX_WAVES : waves);
+  if (waves <= 0) {
+    waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
+    if (waves < MIN_WAVES && (rows <= 32 || n_tiles < 2 * 256)) waves = MIN_WAVES;   // (weights of few rows are cut into slices of K instead)
+  }
+  const int fewest = rows > MANY_ROWS ? MIN_WAVES : FEW_WAVES;
+  waves = waves < fewest ? fewest : (waves > MAX_WAVES ? MAX_WAVES : waves);
   if (rows > MANY_ROWS) waves = MIN_WAVES;
   const int groups = (n_tiles + waves - 1) / waves;
   if (epi != 0) slices = 1;
   if (slices <= 0) {
     slices = 256 / groups;
     if (slices > 8) slices = 8;
-    if (slices > n_rounds / 4) slices = n_rounds / 4;
+    if (slices > n_rounds / 2) slices = n_rounds / 2;
   }
   if (slices < 1) slices = 1;
   if (slices > n_rounds) slices = n_rounds;
@@ -243,13 +253,21 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
   const int n_tiles = (N + tile_rows - 1) / tile_rows;
   const dim3 grid((n_tiles + waves - 1) / waves, slices);
   const int k_tiles = (K + 63) / 64 * 2;
-#define GO(TO_, EPI_)                                                                                         \
-  hipLaunchKernelGGL((wide_gemm_kernel<MT, TO_, EPI_>), grid, dim3(waves * WAVE), 0, s, (const bf16_t*)x,     \
+#define GO(TO_, EPI_, MINW_)                                                                                       \
+  hipLaunchKernelGGL((wide_gemm_kernel<MT, TO_, EPI_, MINW_>), grid, dim3(waves * WAVE), 0, s, (const bf16_t*)x,   \
                      (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order, tile_rows)
-  if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0);
-  else if (out_dtype == DT_BF16) GO(bf16_t, 1);
-  else if (epi == 0) GO(float, 0);
-  else GO(float, 1);
+#define GO_ALL(MINW_)                                    \
+  if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0, MINW_); \
+  else if (out_dtype == DT_BF16) GO(bf16_t, 1, MINW_);        \
+  else if (epi == 0) GO(float, 0, MINW_);                     \
+  else GO(float, 1, MINW_)
+  if (waves >= MIN_WAVES) {
+    GO_ALL(MIN_WAVES);
+  } else {
+    if constexpr (16 * MT <= MANY_ROWS) { GO_ALL(FEW_WAVES); }
+    else IFX_FAIL("wide_gemm: more than %d rows take workgroups of %d waves", MANY_ROWS, MIN_WAVES);
+  }
+#undef GO_ALL
 #undef GO
   if (slices > 1 && add_slices) {
     const size_t n = (size_t)M * N;
@@ -277,8 +295,8 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
   IFX_REQUIRE(epi == 0 || (epi == 1 && N % 2 == 0 && !order && slices == 1), "wide_gemm: epilogue %d with N=%d, %d slices%s", epi, N,
               slices, order ? ", a tile order" : "");
   const int n_rounds = (K + WK - 1) / WK;
-  IFX_REQUIRE(waves >= MIN_WAVES && waves <= MAX_WAVES && slices >= 1 && slices <= n_rounds, "wide_gemm: %d waves (%d-%d), %d slices of %d rounds",
-              waves, MIN_WAVES, MAX_WAVES, slices, n_rounds);
+  IFX_REQUIRE(waves >= FEW_WAVES && waves <= MAX_WAVES && slices >= 1 && slices <= n_rounds, "wide_gemm: %d waves (%d-%d), %d slices of %d rounds",
+              waves, FEW_WAVES, MAX_WAVES, slices, n_rounds);
   IFX_REQUIRE(M <= MANY_ROWS || waves == MIN_WAVES, "wide_gemm: %d rows take workgroups of %d waves, not %d", M, MIN_WAVES, waves);
   IFX_REQUIRE(slices == 1 || part, "wide_gemm: %d slices of K need a scratch buffer", slices);
   if (M == 0) return 0;

@@ -529,7 +529,7 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
 def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
               slices: int = 0, swiglu_pairs: bool = False, keep_slices: bool = False):
     """bfloat16 x [M <= 128, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
-    of a workgroup: the product for 17-64 rows, and for 65-128 rows of weights with few rows.  ``waves`` (8-16 per
+    of a workgroup: the product for 17-64 rows, and for 65-128 rows of weights with few rows.  ``waves`` (4-16 per
     workgroup, 8 beyond 64 rows; one tile of weight rows each) and ``slices`` of K (added in a fixed order): 0 lets the
     kernel choose.  With ``keep_slices`` a product of
     several slices comes back as ``SliceSums``."""

@@ -1025,7 +1025,8 @@ def test_fused_qkv_random_shapes(seed):
 
 
 @pytest.mark.parametrize("M", [9, 17, 32, 33, 50, 64, 65, 81, 100, 128])
-@pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136)])
+@pytest.mark.parametrize("N,K", [(50, 64), (130, 200), (577, 1000), (4608, 3584), (200, 2104), (4100, 136),
+                                 (9000, 264)])                     # tall enough for workgroups of fewer than 8 waves at 33-64 rows
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
 @pytest.mark.parametrize("tile_rows", [16, 14, 10])
 def test_wide_gemm(M, N, K, out_dtype, tile_rows):
@@ -1042,7 +1043,8 @@ def test_wide_gemm(M, N, K, out_dtype, tile_rows):
         assert torch.equal(ops.linear(x.to(DEV), lw, out_dtype).cpu().double(), got)   # what linear picks at these rows
 
 
-@pytest.mark.parametrize("waves,slices,M", [(8, 1, 41), (8, 3, 41), (11, 2, 41), (16, 1, 41), (16, 8, 41), (8, 1, 113), (8, 4, 113), (8, 9, 70)])
+@pytest.mark.parametrize("waves,slices,M", [(8, 1, 41), (8, 3, 41), (11, 2, 41), (16, 1, 41), (16, 8, 41), (8, 1, 113), (8, 4, 113), (8, 9, 70),
+                                            (4, 1, 41), (5, 2, 17), (6, 1, 64), (7, 3, 33), (4, 9, 50), (5, 1, 100)])
 def test_wide_gemm_every_launch_shape_gives_the_same_product(waves, slices, M):
     g = gen(41)
     N, K = 333, 1096                           # 9 rounds of 128 k-values, the last one short; 21 row tiles, the last one short
@@ -1076,7 +1078,7 @@ def test_wide_gemm_gate_up_pairs_and_tile_order():
         ops.wide_gemm(torch.zeros(129, K, dtype=BF16, device=DEV), lq)
     x65 = torch.randn(65, K, generator=g).to(BF16).to(DEV)
     assert torch.equal(ops.wide_gemm(x65, lq, F32, waves=16), ops.wide_gemm(x65, lq, F32))   # beyond 64 rows: taken as 8 waves
-    assert torch.equal(ops.wide_gemm(x.to(DEV), lq, F32, waves=3).cpu().double(), out)    # fewer than 8 waves: taken as 8
+    assert torch.equal(ops.wide_gemm(x.to(DEV), lq, F32, waves=3).cpu().double(), out)    # fewer than 4 waves: taken as 4
 
 
 def test_partial_sums_of_a_product_are_added_by_the_kernel_that_reads_them():
