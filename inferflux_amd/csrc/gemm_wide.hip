@@ -221,15 +221,16 @@ extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S
 // for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
 // several workgroups to a unit; 8 waves for more than 64 rows; then slices of at least two rounds, at most eight);
 // the gate/up epilogue takes one slice.  Returns waves * 256 + slices.
-// Fewer than 8 waves are chosen for 33-64 rows only: there the tall weights of narrow models (gate/up with 600-1,700
-// tiles) take 4-17 % less time with one workgroup of 4-7 waves on every unit than with 8 waves on two thirds of
-// them; up to 32 rows the form for few waves is the slower one at every shape measured.
+// Fewer than 8 waves are chosen for the gate/up epilogue at 33-64 rows only: there the tall weights of narrow models
+// (600-1,700 tiles) take 4-17 % less time with one workgroup of 4-7 waves on every unit than with 8 waves on two thirds
+// of them; up to 32 rows the form for few waves is the slower one at every shape measured, and the other products
+// fill the chip with slices of K.
 extern "C" int ifx_wide_gemm_plan(int rows, int N, int K, int waves, int slices, int epi, int tile_rows) {
   if (tile_rows < 8 || tile_rows > 16) tile_rows = 16;
   const int n_tiles = (N + tile_rows - 1) / tile_rows, n_rounds = (K + WK - 1) / WK;
   if (waves <= 0) {
     waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
-    if (waves < MIN_WAVES && (rows <= 32 || n_tiles < 2 * 256)) waves = MIN_WAVES;   // (weights of few rows are cut into slices of K instead)
+    if (waves < MIN_WAVES && (rows <= 32 || epi == 0)) waves = MIN_WAVES;   // (products that may be cut into slices of K fill the chip that way)
   }
   const int fewest = rows > MANY_ROWS ? MIN_WAVES : FEW_WAVES;
   waves = waves < fewest ? fewest : (waves > MAX_WAVES ? MAX_WAVES : waves);
