@@ -26,6 +26,8 @@ IFX_DEFINE_LAST_ERROR()
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
+constexpr int UNITS = 256;   // compute units of the chip that the launch plans below are measured on
+
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
 #pragma unroll
@@ -464,20 +466,28 @@ extern "C" int ifx_skinny_gemm(const void* x, const void* W, void* out, int out_
   // Choices measured on the 7B shapes at 1-16 rows: two row tiles per wave pay off only for very tall
   // weights; deeper unrolling than 4 blocks spills; about 1500-2500 waves fill the chip.
   if (tiled && mt == 1) {
-    // Measured on the tiled copy (7B shapes, 1-16 rows): two row tiles per wave halve the reads of x and
-    // win wherever they leave 128 workgroups or more, except for the tallest weights at 1-4 rows; tall
-    // weights want 8 waves per workgroup up to 8 rows of x and one beyond; the others enough waves to
-    // reach fifteen hundred (eight to a workgroup where every compute unit has one).
+    // Measured on the tiled copy (shapes of the 0.5B to 72B models, 1-16 rows).  Two row tiles per wave halve the
+    // reads of x; they win where they leave 128 workgroups or more and do not make the fullest compute unit fuller
+    // (every workgroup of a launch is resident at once, so what counts is how many tiles the unit with the most gets:
+    // 1,728 tiles are 7 to a unit one by one and 8 in pairs), except up to 4 rows of x for weights of more than 512
+    // tiles, where x is little to read.  Tall weights want 8 waves per workgroup up to 8 rows of x and one beyond;
+    // the others enough waves to have 1,536 in flight up to 4 rows (4,096 for weights of more than 512 tiles) and
+    // 1,200 beyond (fewer waves split K less and read less of x), at most 8 to a workgroup of tile pairs.  Against one rule for all (pairs from 256 tiles on,
+    // 1,536 waves) gate/up of the 0.5B, 1.5B, 3B and 14B shapes takes 10-15 % less time at 1-16 rows.
     const bool tall = N >= 32768;
     const int n_tiles = (N + tile_rows - 1) / tile_rows;
-    if (nt == 0) nt = tall ? (M <= 4 ? 1 : 2) : ((n_tiles + 1) / 2 >= 128 && tile_rows == 16 ? 2 : 1);
+    auto fullest_unit = [&](int nt_) { return ((n_tiles + nt_ - 1) / nt_ + UNITS - 1) / UNITS * nt_; };
+    if (nt == 0) {
+      const bool pairs_fit = tile_rows == 16 && (n_tiles + 1) / 2 >= 128 && fullest_unit(2) <= fullest_unit(1);
+      nt = tall ? (M <= 4 ? 1 : 2) : (pairs_fit && (M > 4 || n_tiles <= 512) ? 2 : 1);
+    }
     if (unroll == 0) unroll = (nt == 1 && M <= 4) ? 4 : 2;
     if (waves == 0) {
       const int groups = (n_tiles + nt - 1) / nt;
       waves = 1;
       if (tall) waves = M <= 8 ? 8 : 1;
       else
-        while (waves < 16 && groups * waves < 1536) waves *= 2;
+        while (waves < (nt == 2 ? 8 : 16) && groups * waves < (M > 4 ? 1200 : n_tiles > 512 ? 4096 : 1536)) waves *= 2;
       while (waves > 1 && nkb < waves * 2) waves /= 2;
     }
   }
