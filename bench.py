@@ -2,7 +2,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
 
-A step is one decode step of the whole engine (scheduler, step function, sampling).  Prints one
+A step is one decode step of the whole engine (scheduler, step function, sampling); before the W warm-up steps of a
+decode measurement its freshly captured graph is replayed SETTLE_STEPS times (see there; reported as ``settle_steps``).  Prints one
 JSON line: decoded tokens a second at batch 8 as ``value``, the same at batch 1 and 64 under
 ``points`` (with their step times and roofline shares under ``ms_per_step_b1`` / ``roofline_b1`` and
 ``..._b64``), a 2,048-token prefill under ``prefill`` (the mean of ``mean_of`` runs with the library's
@@ -52,6 +53,13 @@ WORKLOADS = {
 CONTEXT = 4096
 PROMPT = 2048
 DECODE_KV_START = 3072      # mean context of a 2,048-token decode after a 2,048-token prompt
+# Decode steps that every decode measurement runs, untimed, before its W warm-up steps.  A decode step is a replayed
+# HIP graph, and the first replays of a graph that has just been captured run slower on this card (the 7B shape at
+# batch 8: 3.44 ms for the first 37 replays, then 3.24 ms from one step to the next and for good, also after idling
+# and for later requests on the same graph; 15 replays at batch 1; every weight-streaming kernel is 5-12 % slower in
+# that phase, the same kernels on the same data).  An engine captures a layout once and replays it for as long as it
+# serves, so the steady state is what a step costs; the contexts are counted as grown by these steps.
+SETTLE_STEPS = 48
 PAGE = 16
 
 
@@ -135,7 +143,7 @@ def main() -> int:
         """tokens/s and ms/step of ``steps`` decode steps at ``batch`` with contexts from ``--context``."""
         # While the last prompts are still coming in, the first requests already decode: give every
         # request enough tokens (and pages) that none finishes before the timed steps are over.
-        slack = -(-batch * kv_start // 16384) + 2
+        slack = -(-batch * kv_start // 16384) + 2 + SETTLE_STEPS
         eng = make_engine(batch, kv_start + steps + warmup + slack + 2)
         sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + slack + 1, ignore_eos=True)
         for _ in range(batch):
@@ -144,7 +152,7 @@ def main() -> int:
             eng.step()                                            # prompts in; every request now decodes
         note(f"batch {batch}: prompts are in, decoding")
         ops.pause_library_gemm_tuning(False)
-        for _ in range(warmup):
+        for _ in range(SETTLE_STEPS + warmup):
             eng.step()
         ops.pause_library_gemm_tuning(True)
         torch.cuda.synchronize()
@@ -154,7 +162,7 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         assert len(eng.scheduler.running) == batch and eng.stats.preemptions == 0, "a request finished or was preempted while timing"
-        kv_mean = kv_start + warmup + steps / 2
+        kv_mean = kv_start + SETTLE_STEPS + warmup + steps / 2
         del eng
         torch.cuda.empty_cache()
         return batch * steps / dt, dt / steps * 1e3, kv_mean
@@ -281,9 +289,9 @@ def main() -> int:
     out = {
         "metric": f"decode tok/s at batch {args.batch} (" + shape_name + f", {args.dtype}, random weights)",
         "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "settle_steps": SETTLE_STEPS, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (uniform random token ids, seeded N(0,0.02) weights)",
-        "config": {"model": shape_name, "global_batch": args.batch, "seq_len": max(CONTEXT, kv_start + args.steps + args.warmup), "parallelism": "1 GPU",
+        "config": {"model": shape_name, "global_batch": args.batch, "seq_len": max(CONTEXT, kv_start + SETTLE_STEPS + args.steps + args.warmup), "parallelism": "1 GPU",
                    "num_hidden_layers": layers_full, "layers_run": L, "hidden_size": H, "num_attention_heads": nH,
                    "num_key_value_heads": nKV, "head_dim": d, "intermediate_size": I, "vocab_size": V,
                    "prompt_len": PROMPT, "decode_kv_start": kv_start, "kv_page_size": PAGE,
