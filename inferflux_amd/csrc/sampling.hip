@@ -274,18 +274,6 @@ __device__ __forceinline__ void block_map(const float* __restrict__ p, float* __
   if (t < n) q[t] = f(p[t]);
 }
 
-__device__ float kept_sum(const float* __restrict__ w, int V, float thr, float* red) {
-  float s = 0.f;
-  block_visit(w, V, [&](int, float x) { if (x >= thr) s += x; });
-  return block_sum(s, red);
-}
-
-__device__ int kept_count(const float* __restrict__ w, int V, float thr, int* red) {
-  int c = 0;
-  block_visit(w, V, [&](int, float x) { c += x >= thr ? 1 : 0; });
-  return block_sum_int(c, red);
-}
-
 // The thresholds of top-k and top-p are exact selections among the weights of one row.  A histogram over the upper
 // bits of the weights' bit patterns (sign and exponent and the first HIST_MANTISSA bits of the mantissa: HIST_BINS
 // bins, the largest weight 1.0 falls into bin 2032) says which bin each threshold lies in; the weights from the
@@ -293,11 +281,13 @@ __device__ int kept_count(const float* __restrict__ w, int V, float thr, int* re
 // wave bisects over the bit patterns within the bin there.  Counts are integers and sums are sums of the
 // weights in fixed point (units of 2^-40, so a row of a million weights of 1.0 stays below 2^64): neither depends
 // on the order in which the threads add, and the histogram's sums and the candidates' agree exactly.  A row whose
-// candidates do not fit (a nearly flat distribution under top-p) bisects over the whole row instead.
+// candidates do not fit (more than SAMPLE_CANDIDATES: a wide nucleus) goes over the whole row twice more per threshold
+// instead: the weights of the threshold's bin are counted by their next ten bits, then those of that sub-bin by
+// their last nine (refine_threshold).
 #define HIST_MANTISSA 4
 #define HIST_SHIFT (23 - HIST_MANTISSA)
 #define HIST_BINS 2048
-#define SAMPLE_CANDIDATES 8192
+#define SAMPLE_CANDIDATES 3072
 typedef unsigned long long u64;
 
 __device__ __forceinline__ u64 weight_fixed(float x) { return (u64)(x * 1099511627776.0f); }   // x * 2^40, x in [0, 1]
@@ -379,6 +369,71 @@ __device__ __forceinline__ int last_bin_reaching(const T* table, T need, int lo,
     if (table[mid] >= need) lo = mid; else hi = mid - 1;
   }
   return lo;
+}
+
+// The exact threshold inside bin ``bin1`` of the histogram, over the whole row: the largest pattern t for which the
+// weights >= t number at least ``need`` (BY_SUM false) or sum to at least ``need`` in fixed point (BY_SUM true), given
+// what lies above the bin (``above_count`` weights that sum to ``above_sum``) and that the bin's lower edge satisfies
+// it.  Two passes: the bin's weights by the next ten bits of their patterns, then the chosen sub-bin's by the last
+// nine.  The histograms live in the memory of the candidates, which such a row does not use.  Every thread returns
+// the pattern and the sum of the weights that reach it.
+struct Refined { unsigned bits; u64 sum_from; };
+
+template <bool BY_SUM>
+__device__ Refined refine_threshold(const float* __restrict__ w, int V, unsigned bin1, unsigned above_count, u64 above_sum,
+                                    u64 need, SampleShared& sh) {
+  static_assert(SAMPLE_THREADS == 1024 && SAMPLE_CANDIDATES * sizeof(float) >= 1024 * (sizeof(unsigned) + sizeof(u64)),
+                "one sub-bin per thread, in the candidates' memory");
+  unsigned* c2 = reinterpret_cast<unsigned*>(sh.cand);
+  u64* s2 = reinterpret_cast<u64*>(sh.cand + 1024);
+  const int tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  unsigned prefix = bin1;      // the pattern's bits from ``shift`` upwards
+  int shift = HIST_SHIFT;
+  u64 reach_sum = 0;
+  for (int level = 0; level < 2; ++level) {
+    const int width = level == 0 ? 10 : shift;     // 10 bits, then the 9 that are left
+    const int below = shift - width;
+    const unsigned mask = (1u << width) - 1;
+    __syncthreads();                               // (the last level's tables have been read)
+    c2[tid] = 0;
+    s2[tid] = 0;
+    __syncthreads();
+    block_visit(w, V, [&](int, float x) {
+      const unsigned b = __float_as_uint(x);
+      if ((b >> shift) == prefix) {
+        const unsigned sub = (b >> below) & mask;
+        atomicAdd(&c2[sub], 1u);
+        atomicAdd(&s2[sub], weight_fixed(x));
+      }
+    });
+    __syncthreads();
+    // totals over the sub-bins from each one upwards: thread t has sub-bin 1023 - t
+    unsigned ci = c2[1023 - tid];
+    u64 si = s2[1023 - tid];
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+      const unsigned oc = __shfl_up(ci, o, WAVE);
+      const u64 os = __shfl_up(si, o, WAVE);
+      if (lane >= o) { ci += oc; si += os; }
+    }
+    if (lane == WAVE - 1) { sh.wave_count[wid] = ci; sh.wave_sum[wid] = si; }
+    __syncthreads();
+    for (int i = 0; i < wid; ++i) { ci += sh.wave_count[i]; si += sh.wave_sum[i]; }
+    c2[1023 - tid] = ci;
+    s2[1023 - tid] = si;
+    __syncthreads();
+    int lo = 0, hi = (int)mask;                    // (every thread searches: the tables are in LDS)
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      const bool reached = BY_SUM ? above_sum + s2[mid] >= need : (u64)above_count + c2[mid] >= need;
+      if (reached) lo = mid; else hi = mid - 1;
+    }
+    reach_sum = above_sum + s2[lo];
+    if (lo < (int)mask) { above_count += c2[lo + 1]; above_sum += s2[lo + 1]; }
+    prefix = (prefix << width) | (unsigned)lo;
+    shift = below;
+  }
+  return Refined{prefix, reach_sum};
 }
 
 // The token at which the cumulative sum of the kept weights (those with bit pattern >= thr_bits), taken in index
@@ -554,22 +609,18 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
       __syncthreads();
       thr_bits = sh.thr_bits;
     } else {
+      const int top_bin = one_bits >> HIST_SHIFT;
+      u64 kept_all = sh.sum[0];
       if (k_on) {
-        unsigned lo = 0, hi = one_bits;  // count(w >= f(lo)) >= k holds for lo = 0
-        while (lo < hi) {
-          const unsigned mid = lo + (hi - lo + 1) / 2;
-          if (kept_count(w, V, __uint_as_float(mid), sh.red_i) >= k) lo = mid; else hi = mid - 1;
-        }
-        thr_bits = lo;
+        const Refined t = refine_threshold<false>(w, V, bk, sh.count[bk + 1], sh.sum[bk + 1], (u64)k, sh);
+        thr_bits = t.bits;
+        kept_all = t.sum_from;
       }
       if (p_on) {
-        const float need = top_p * kept_sum(w, V, __uint_as_float(thr_bits), sh.red_f);
-        unsigned lo = thr_bits, hi = one_bits;  // sum(w >= f(lo)) >= need holds for lo = thr_bits
-        while (lo < hi) {
-          const unsigned mid = lo + (hi - lo + 1) / 2;
-          if (kept_sum(w, V, __uint_as_float(mid), sh.red_f) >= need) lo = mid; else hi = mid - 1;
-        }
-        thr_bits = lo;
+        const u64 need = (u64)((double)top_p * (double)kept_all);
+        const int b = last_bin_reaching(sh.sum, need, 0, top_bin);
+        const Refined t = refine_threshold<true>(w, V, b, sh.count[b + 1], sh.sum[b + 1], need, sh);
+        thr_bits = max(thr_bits, t.bits);   // (it is at least top-k's: the weights that reach that one sum to kept_all >= need)
       }
     }
   }

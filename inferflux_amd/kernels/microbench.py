@@ -3,6 +3,7 @@
     python -m inferflux_amd.kernels.microbench attention-tiles --rows 8192 [--query-tiles 2]
     python -m inferflux_amd.kernels.microbench attention-rows --batch 64 --context 3072 [--chunk 512]
     python -m inferflux_amd.kernels.microbench gemm --rows 8 [--shape gate_up]
+    python -m inferflux_amd.kernels.microbench sampling --batch 8 [--vocab 152064]
     python -m inferflux_amd.kernels.microbench ceilings
 
 Sizes default to the Qwen2.5-7B shape (28 query heads, 4 kv heads, head size 128, hidden 3584,
@@ -145,6 +146,28 @@ def gemm(args) -> None:
         del ws
 
 
+def sampling(args) -> None:
+    """The sampling kernels on ``--batch`` rows of ``--vocab`` logits (a normal spread of ``--spread``), each call
+    inside a replayed graph: greedy, a draw at a temperature, with top-k and top-p, with top-p alone (more
+    candidates), and the log-probabilities with five alternatives."""
+    dev, R, V = "cuda", args.batch, args.vocab
+    logits = torch.randn(R, V, device=dev) * args.spread
+    full = lambda v, dt=torch.float32: torch.full((R,), v, dtype=dt, device=dev)
+    u = torch.rand(R, device=dev)
+    chosen = ops.argmax(logits)
+    t08, t1, k0, k50, p1, p09, m0, m001 = (full(0.8), full(1.0), full(0, torch.int32), full(50, torch.int32), full(1.0), full(0.9),
+                                           full(0.0), full(0.01))
+    cases = [("argmax", lambda i: ops.argmax(logits)),
+             ("temperature 0.8", lambda i: ops.sample(logits, t08, k0, p1, m0, u)),
+             ("temperature 0.8, top-k 50, top-p 0.9", lambda i: ops.sample(logits, t08, k50, p09, m0, u)),
+             ("temperature 0.8, top-p 0.9", lambda i: ops.sample(logits, t08, k0, p09, m0, u)),
+             ("temperature 1, min-p 0.01", lambda i: ops.sample(logits, t1, k0, p1, m001, u)),
+             ("log-probabilities, 5 alternatives", lambda i: ops.logprobs(logits, chosen, 5)),
+             ("log-probability of the token alone", lambda i: ops.logprobs(logits, chosen, 0))]
+    for name, fn in cases:
+        print(f"sampling rows={R} vocabulary={V} {name}: {_time_us(fn, args.iters, True):8.1f} us", flush=True)
+
+
 def ceilings(args) -> None:
     """What a kernel that only reads (or copies) gets from this card's memory, and the library's large products."""
     dev = "cuda"
@@ -187,7 +210,7 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="python -m inferflux_amd.kernels.microbench")
     sub = ap.add_subparsers(dest="what", required=True)
     for name, fn in (("attention-tiles", attention_tiles), ("attention-rows", attention_rows), ("gemm", gemm),
-                     ("ceilings", ceilings)):
+                     ("sampling", sampling), ("ceilings", ceilings)):
         p = sub.add_parser(name)
         p.set_defaults(fn=fn)
         p.add_argument("--iters", type=int, default=10)
@@ -216,6 +239,10 @@ def main(argv=None) -> int:
             p.add_argument("--rotate-gb", type=float, default=2.0,
                            help="memory the launches rotate through (a model's step touches tens of GB between two uses of a cache)")
             p.add_argument("--pages", choices=["shuffled", "in-order"], default="shuffled", help="how a request's pages lie in the pool")
+        if name == "sampling":
+            p.add_argument("--batch", type=int, default=8)
+            p.add_argument("--vocab", type=int, default=152064)
+            p.add_argument("--spread", type=float, default=3.0, help="standard deviation of the logits")
         if name == "ceilings":
             p.add_argument("--pool-gb", type=float, default=16.0, help="memory the reads and copies rotate through")
         if name == "gemm":

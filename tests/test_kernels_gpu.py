@@ -507,6 +507,10 @@ SAMPLE_SHAPES = [
     ("mostly masked", 9999, lambda g, V: torch.where(torch.rand(V, generator=g) < 0.9, torch.tensor(-float("inf")), 2.0 * torch.randn(V, generator=g)), 0.8, 40, 0.9, 0.0),
     ("top-p alone, peaked", 152064, lambda g, V: 6.0 * torch.randn(V, generator=g), 0.6, 0, 0.95, 0.0),
     ("top-p alone, wide", 152064, lambda g, V: 1.5 * torch.randn(V, generator=g), 1.0, 0, 0.9, 0.0),
+    # a nearly flat row is all candidates: as many as fit, and one more (which takes the passes over the whole row)
+    ("as many tokens as candidates fit", 3072, lambda g, V: 0.05 * torch.randn(V, generator=g), 1.0, 3000, 0.999, 0.0),
+    ("one token more than candidates fit", 3073, lambda g, V: 0.05 * torch.randn(V, generator=g), 1.0, 3000, 0.999, 0.0),
+    ("wide nucleus inside a wide top-k", 100003, lambda g, V: 0.7 * torch.randn(V, generator=g), 1.3, 60000, 0.97, 0.0),
 ]
 
 
