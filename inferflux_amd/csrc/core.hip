@@ -40,6 +40,47 @@ extern "C" int ifx_embedding(const int* ids, const void* table, int table_dtype,
   IFX_LAUNCH_CHECK();
 }
 
+// The same for up to 16 tokens, with what the RMS norm that reads the stream first needs written beside it, so that
+// the norm takes no kernel of its own: rows[t, :] = bf16(out[t, :] * norm_w[:]) and pieces[run][t] = the sum of the
+// squares of out[t, :] over run ``run`` of 4,096 columns (zero for t >= n_rows; ``pieces`` is [runs][16]).  The
+// product that reads ``rows`` multiplies its sums by rsqrt(sum of the pieces / H + eps) (RowScale in gemm_bf16.hip).
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_norm_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                                            const bf16_t* __restrict__ norm_w, float* __restrict__ out,
+                                                            bf16_t* __restrict__ rows, float* __restrict__ pieces,
+                                                            int n_rows, int H) {
+  __shared__ float red[16];
+  const int t = blockIdx.x, run = blockIdx.y, i0 = run * 4096, i1 = min(H, i0 + 4096);
+  float ss = 0.f;
+  if (t < n_rows) {
+    const T* src = table + (size_t)ids[t] * H;
+    for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) {
+      const float x = to_f(src[i]);
+      out[(size_t)t * H + i] = x;
+      rows[(size_t)t * H + i] = (bf16_t)(x * to_f(norm_w[i]));
+      ss += x * x;
+    }
+  }
+  ss = block_sum(ss, red);
+  if (threadIdx.x == 0) pieces[run * 16 + t] = ss;
+}
+
+extern "C" int ifx_embedding_norm(const int* ids, const void* table, int table_dtype, const void* norm_w, float* out,
+                                  void* rows, float* pieces, int T, int H, void* stream) {
+  IFX_REQUIRE(T >= 0 && T <= 16 && H > 0, "embedding_norm: T=%d must be at most 16 (H=%d)", T, H);
+  IFX_REQUIRE(norm_w && out && rows && pieces, "embedding_norm: needs the norm's weight and three outputs");
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(16, (H + 4095) / 4096);
+  if (table_dtype == DT_F32)
+    hipLaunchKernelGGL(embedding_norm_kernel<float>, grid, dim3(256), 0, s, ids, (const float*)table, (const bf16_t*)norm_w, out, (bf16_t*)rows, pieces, T, H);
+  else if (table_dtype == DT_BF16)
+    hipLaunchKernelGGL(embedding_norm_kernel<bf16_t>, grid, dim3(256), 0, s, ids, (const bf16_t*)table, (const bf16_t*)norm_w, out, (bf16_t*)rows, pieces, T, H);
+  else
+    IFX_FAIL("embedding_norm: unknown dtype %d", table_dtype);
+  IFX_LAUNCH_CHECK();
+}
+
 // ---------------------------------------------------------------------------------------
 // x = residual[src] (+ delta[src]);  if write_back: residual[src] = x
 // out[r, :] = x * rsqrt(mean(x^2) + eps) * weight         src = rows ? rows[r] : r

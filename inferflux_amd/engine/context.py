@@ -94,6 +94,9 @@ class StepContext:
         rows.extend(range(self.n_real_tokens, T))            # rows that stand for nobody: last, dropped by the caller
         self.h_logit_rows = np.asarray(rows, dtype=np.int32)
         self.n_logit_rows = len(rows)
+        # every row of the step wants its logits, in order (a step of single tokens): the rows that the last product of the
+        # layers prepares for the final norm are then the head's input as they are
+        self.all_rows_wanted = rows == list(range(T))
         self.h_state_slots = arrays["state_slots"]
         n_groups = len(manager.groups)
         self.h_block_tables: List[np.ndarray] = arrays["block_tables"]

@@ -15,6 +15,7 @@ from .. import architectures  # noqa: F401  (registers the known architectures)
 from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.registry import plan_for
 from ..parts.base import build_part
+from ..parts.block import normed_for
 from ..parts.plan import ModelPlan, ParamSpec
 from ..weights.loader import load_weights, random_tensor
 
@@ -100,15 +101,24 @@ class Model:
         if t is not None:
             t.begin()
             t.enter("embed")
-        residual = self.embedding.forward(ctx)
+        schedule = self.plan.schedule
+        pending = None
+        first_norm = self.blocks[schedule[0].layer].entry_norm() if schedule else None
+        if first_norm is not None and getattr(self.embedding, "prepares_norm_rows", False):
+            residual = self.embedding.forward(ctx, norm=first_norm)     # (an embedding that can do so prepares the first norm's rows)
+            if isinstance(residual, tuple):
+                residual, pending = residual
+        else:
+            residual = self.embedding.forward(ctx)
         if t is not None:
             t.mark("embed")
-        pending = None
-        schedule = self.plan.schedule
         for i, e in enumerate(schedule):
             block = self.blocks[e.layer]
             # a block that can hand on rows prepared for the next block's first norm is told that norm
-            following = self.blocks[schedule[i + 1].layer].entry_norm() if i + 1 < len(schedule) else None
+            if i + 1 < len(schedule):
+                following = self.blocks[schedule[i + 1].layer].entry_norm()
+            else:       # the last block may prepare the final norm's rows where the head takes every row of the step
+                following = self.final_norm if ctx.all_rows_wanted else None
             if following is not None and block.entry_norm() is not None:
                 residual, pending = block.forward(residual, pending, ctx, storage.binding(i), following=following)
             else:
@@ -118,7 +128,10 @@ class Model:
         else:
             if t is not None:
                 t.enter("final_norm")
-            h = self.final_norm.forward(residual, pending, ctx.act_dtype, rows=ctx.logit_rows)
+            if ctx.all_rows_wanted:
+                h = normed_for(self.final_norm, self.head, residual, pending, ctx)
+            else:
+                h = self.final_norm.forward(residual, pending, ctx.act_dtype, rows=ctx.logit_rows)
             if t is not None:
                 t.mark("final_norm")
                 t.enter("lm_head")

@@ -127,6 +127,24 @@ def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.Tensor, eps: float):
+    """``embedding`` for up to 16 tokens that also prepares the RMS norm (bfloat16 weight ``norm_weight`` [H]) which
+    reads the stream first: returns (the float32 stream [T, H], that norm's rows up to the factor per row)."""
+    _check(ids, "ids", (None,), torch.int32)
+    _check(table, "table", (None, None))
+    T, H = ids.shape[0], table.shape[1]
+    _check(norm_weight, "norm_weight", (H,), torch.bfloat16)
+    if T > 16:
+        raise KernelError(f"embedding_scaled: {T} rows (at most 16)")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    rows = torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
+    pieces = torch.empty((-(-H // 4096), 16), dtype=torch.float32, device=table.device)
+    _call(load_module("core"), "ifx_embedding_norm", (P, P, I, P, P, P, P, I, I, P),
+          ids.data_ptr(), table.data_ptr(), _dt(table), norm_weight.data_ptr(), out.data_ptr(), rows.data_ptr(),
+          pieces.data_ptr(), T, H, _stream())
+    return out, ScaledRows(rows, pieces, H, eps, norm_weight)
+
+
 def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``residual`` [T, H] float32 (+= ``delta`` in place when given and no ``rows``), then RMSNorm.

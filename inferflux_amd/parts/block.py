@@ -18,7 +18,7 @@ from .base import Block, MixerBinding, StreamSink, build_part, register_part
 from .plan import LayerSpec
 
 
-def _normed(norm, reader, residual, pending, ctx):
+def normed_for(norm, reader, residual, pending, ctx):
     """What ``reader`` is given: the norm of the stream plus ``pending``."""
     if isinstance(pending, ScaledRows):          # the delta is in the stream already
         accepts = getattr(reader, "accepts_scaled_rows", None)
@@ -67,12 +67,12 @@ class PreNormBlock(Block):
     def forward(self, residual, pending, ctx, binding: MixerBinding, following=None):
         t = ctx.timer
         if t is None:
-            h = _normed(self.norm_in, self.mixer, residual, pending, ctx)
+            h = normed_for(self.norm_in, self.mixer, residual, pending, ctx)
             delta = self._mixer(h, ctx, binding, residual)
-            h = _normed(self.norm_post, self.ffn, residual, delta, ctx)
+            h = normed_for(self.norm_post, self.ffn, residual, delta, ctx)
             return residual, self._ffn(h, ctx, residual, following)
-        t.enter("norm"); h = _normed(self.norm_in, self.mixer, residual, pending, ctx); t.mark("norm")
+        t.enter("norm"); h = normed_for(self.norm_in, self.mixer, residual, pending, ctx); t.mark("norm")
         t.enter("mixer"); delta = self._mixer(h, ctx, binding, residual); t.mark("mixer")
-        t.enter("norm"); h = _normed(self.norm_post, self.ffn, residual, delta, ctx); t.mark("norm")
+        t.enter("norm"); h = normed_for(self.norm_post, self.ffn, residual, delta, ctx); t.mark("norm")
         t.enter("ffn"); out = self._ffn(h, ctx, residual, following); t.mark("ffn")
         return residual, out

@@ -32,7 +32,16 @@ class TokenEmbedding(Part):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.table = tensors[f"{self.name}.weight"]
 
-    def forward(self, ctx) -> torch.Tensor:
+    prepares_norm_rows = True
+
+    def forward(self, ctx, norm=None):
+        """The float32 stream of the step's tokens.  Told the norm that reads the stream first (``norm``), a step of few
+        tokens in bfloat16 also gets that norm's rows up to a factor per row, (stream, ``ops.ScaledRows``), which
+        saves the norm a kernel of its own where the layer's first product takes such rows."""
+        params = norm.rms_params() if norm is not None else None
+        if (params is not None and 0 < ctx.n_tokens <= 16 and ctx.act_dtype == torch.bfloat16
+                and params[0].dtype == torch.bfloat16):
+            return ops.embedding_scaled(ctx.token_ids, self.table, params[0], params[1])
         return ops.embedding(ctx.token_ids, self.table)
 
 
@@ -54,5 +63,8 @@ class LinearHead(Part):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = ops.prepare_linear(tensors[self.tied_to or f"{self.name}.weight"])
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def accepts_scaled_rows(self, n_rows: int) -> bool:
+        return ops.takes_scaled_rows(n_rows, self.weight)
+
+    def forward(self, h) -> torch.Tensor:
         return ops.linear(h, self.weight, out_dtype=torch.float32)

@@ -256,8 +256,9 @@ def test_a_layer_that_reads_another_entries_cache_in_bfloat16():
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_steps_of_few_rows_need_no_kernel_for_the_norms_between_products(name, sharp_folders, monkeypatch):
     """In bfloat16 a step of up to 16 rows adds each sub-block's output to the stream in its last product's epilogue
-    and applies the next norm's factor in the next product: only the first layer's first norm and the final norm
-    keep a kernel.  Logits agree with the plain model, and with the same step run with a kernel for every norm."""
+    and applies the next norm's factor in the next product; the embedding prepares the first layer's first norm the
+    same way and the head takes the final norm's rows (these steps want every row's logits): no norm keeps a kernel.
+    Logits agree with the plain model, and with the same step run with a kernel for every norm."""
     from inferflux_amd.kernels import ops
     folder, V, L = sharp_folders[name, "bfloat16"], TINY[name]["vocab_size"], TINY[name]["num_hidden_layers"]
     ids = seeded_ids(31, 60, V)
@@ -279,8 +280,9 @@ def test_steps_of_few_rows_need_no_kernel_for_the_norms_between_products(name, s
 
     yield_calls = []
     fused = run(load_runner(folder, torch.bfloat16, num_pages=16))
-    assert yield_calls == [(17, 2 * L + 1)] + [(m, 2) for m in (16, 1, 9, 16, 1)], yield_calls
+    assert yield_calls == [(17, 2 * L + 1)] + [(m, 0) for m in (16, 1, 9, 16, 1)], yield_calls
     monkeypatch.setattr(ops, "adds_into_stream", lambda *a: False)
+    monkeypatch.setattr(ops, "takes_scaled_rows", lambda *a: False)
     yield_calls = []
     separate = run(load_runner(folder, torch.bfloat16, num_pages=16))
     assert all(n == 2 * L + 1 for _, n in yield_calls), yield_calls

@@ -38,6 +38,32 @@ def test_embedding(dtype):
     assert torch.equal(ops.embedding(pick.to(DEV), wide.to(DEV)).cpu(), wide.float()[pick.long()])
 
 
+@pytest.mark.parametrize("T,H", [(1, 104), (5, 896), (16, 3584), (9, 9008)])
+def test_embedding_that_prepares_the_first_norm(T, H):
+    """The stream as ``embedding`` gives it, the rows times the norm's weight, and sums of squares by runs of 4,096
+    columns that add up to each row's (zeros for the rows a step of fewer than 16 tokens does not have); what a product
+    makes of such rows is the norm's output times the weight."""
+    g = gen(3)
+    eps = 1e-5
+    table = torch.randn(50, H, generator=g).to(BF16)
+    nw = (1 + 0.3 * torch.randn(H, generator=g)).to(BF16)
+    ids = torch.randint(0, 50, (T,), generator=g).to(torch.int32)
+    stream, scaled = ops.embedding_scaled(ids.to(DEV), table.to(DEV), nw.to(DEV), eps)
+    x = table.float()[ids.long()]
+    assert torch.equal(stream.cpu(), x)
+    assert torch.equal(scaled.rows.cpu(), (x * nw.float()).to(BF16))
+    pieces = scaled.pieces.cpu().double()
+    assert pieces.shape == (-(-H // 4096), 16) and bool((pieces[:, T:] == 0).all())
+    assert torch.allclose(pieces.sum(0)[:T], (x.double() ** 2).sum(-1), rtol=1e-5)
+    assert scaled.width == H and scaled.eps == eps
+    w = (torch.randn(64, H, generator=g) * 0.1).to(BF16)
+    got = ops.linear(scaled, ops.prepare_linear(w.to(DEV)), F32).cpu().double()
+    want = pm.rms_norm(x.double(), nw.double(), eps) @ w.double().t()
+    assert float((got - want).abs().max()) <= 1e-2 * float(want.abs().max())
+    with pytest.raises(ops.KernelError, match="at most 16"):
+        ops.embedding_scaled(torch.zeros(17, dtype=torch.int32, device=DEV), table.to(DEV), nw.to(DEV), eps)
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("H", [100, 3584])
 @pytest.mark.parametrize("wdtype", [F32, BF16])
