@@ -34,7 +34,11 @@ optional for every part; one that declares nothing is run as above.
             ``SliceSums``.
             ``accepts_scaled_rows(n_rows)`` True: forward takes ``ScaledRows`` for h.
   block     ``entry_norm()`` -> the norm that first reads the stream, if ``pending`` may be ``ScaledRows`` made
-            for it; forward then takes ``following=`` the next block's entry norm (or None).
+            for it; forward then takes ``following=`` the next block's entry norm (or None; for the last block the
+            final norm, in steps that want every row's logits).
+  embedding ``prepares_norm_rows`` True: forward takes ``norm=`` the first block's entry norm and may return
+            (stream, ``ScaledRows`` made for that norm).
+  head      ``accepts_scaled_rows(n_rows)`` True: forward takes ``ScaledRows`` for the normalised rows.
 """
 from __future__ import annotations
 
