@@ -350,7 +350,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   IFX_REQUIRE(part_o && part_ml, "attn_rows: splits need scratch for their partial results");
   if (n_rows >= ROW_STREAM_MIN_ROWS) hipLaunchKernelGGL(attn_rows_kernel<true>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
   else hipLaunchKernelGGL(attn_rows_kernel<false>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
-  hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, a);
+  hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, a);
   IFX_LAUNCH_CHECK();
 }
 
@@ -751,7 +751,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
               scale * 1.4426950408889634f, 1};
-    hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, m);
+    hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, m);
   }
   IFX_LAUNCH_CHECK();
 }

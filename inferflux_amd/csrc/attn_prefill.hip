@@ -415,7 +415,7 @@ extern "C" int ifx_attn_prefill(const void* q, const void* k_cache, const void* 
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
               scale * 1.4426950408889634f, 1};
-    hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, m);
+    hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, m);
   }
   IFX_LAUNCH_CHECK();
 }

@@ -29,9 +29,12 @@ TILE_SPLIT_FEW_MIN_LONGEST = 1024   # this many keys on, and may be as short as
 TILE_SPLIT_FEW_MIN_KEYS = 256       # this while the walk is short
 TILE_MAX_SPLITS = 16
 TILE_ORDER_MIN_ITEMS = 64       # launches of more workgroups than this get them in tile_order
-ROW_CHUNK = 128     # keys per split of the row kernel: doubled while the launch keeps more than ROW_MIN_WAVES
-ROW_MIN_WAVES = 1536  # waves (a split costs a fixed start-up, so longer splits pay when there are waves enough),
-ROW_MAX_SPLITS = 128  # and until a row has at most this many splits (one row over 131,072 keys: 91 us against 133 at 64)
+ROW_CHUNK = 64      # keys per split of the row kernel: doubled while the launch keeps ROW_MIN_WAVES (ROW_MIN_WAVES_128
+ROW_MIN_WAVES_128 = 1000   # for the step from 64 to 128) waves or more: a split costs a fixed start-up, so longer splits
+ROW_MIN_WAVES = 1536       # pay when there are waves enough; and until a row has at most ROW_MAX_SPLITS splits.  The merge
+ROW_MAX_SPLITS = 512       # launch shares a row of many splits among up to 8 waves, so one request over a long context may
+                           # have hundreds (one row over 32,000 keys: 23.6 us in 250 splits against 35.8 in 125 with a
+                           # merge of one wave; over 3,100 keys 11.8 us in 49 splits of 64 against 13.7 in 25 of 128).
 ROW_WHOLE_MIN_PAIRS = 192   # (row, kv head) pairs from which a workgroup takes a pair's keys whole
 ROW_WAVE_SLOTS = 2048       # waves the chip holds at the row kernel's two per SIMD
 
@@ -215,7 +218,7 @@ def row_launch_shape(n_rows: int, n_kv_heads: int, max_kv: int, max_waves: int =
         return 0, waves, 1
     chunk = ROW_CHUNK
     while (-(-max_kv // chunk) > ROW_MAX_SPLITS
-           or pairs * -(-max_kv // (2 * chunk)) >= ROW_MIN_WAVES):
+           or pairs * -(-max_kv // (2 * chunk)) >= (ROW_MIN_WAVES_128 if chunk == ROW_CHUNK else ROW_MIN_WAVES)):
         chunk *= 2
     return chunk, 0, -(-max_kv // chunk)
 

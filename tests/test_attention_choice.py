@@ -162,7 +162,9 @@ def test_row_launch_shape():
     assert row_launch_shape(600, 4, 4096) == (0, 1, 1)
     assert row_launch_shape(64, 4, 4096, max_waves=4) == (0, 4, 1)      # what the kernel's LDS allows at these head counts
     assert row_launch_shape(64, 2, 4096)[1] == 0                        # 128 pairs: splits
+    assert row_launch_shape(1, 4, 4096) == (64, 0, 64) and row_launch_shape(1, 4, 32768) == (128, 0, 256)   # one request: many short splits
+    assert row_launch_shape(16, 4, 4096) == (128, 0, 32) and row_launch_shape(32, 4, 4096) == (256, 0, 16)
     for rows, kv_heads, bound in [(1, 4, 4096), (8, 4, 4096), (32, 4, 4096), (1, 1, 131072), (8, 8, 32768), (47, 4, 1024)]:
         chunk, waves, splits = row_launch_shape(rows, kv_heads, bound)
-        assert waves == 0 and chunk % 32 == 0 and chunk >= 128
+        assert waves == 0 and chunk % 32 == 0 and chunk >= 64
         assert splits * chunk >= bound > (splits - 1) * chunk and splits <= ROW_MAX_SPLITS
