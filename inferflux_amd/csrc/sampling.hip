@@ -277,13 +277,12 @@ __device__ __forceinline__ void block_map(const float* __restrict__ p, float* __
 // The thresholds of top-k and top-p are exact selections among the weights of one row.  A histogram over the upper
 // bits of the weights' bit patterns (sign and exponent and the first HIST_MANTISSA bits of the mantissa: HIST_BINS
 // bins, the largest weight 1.0 falls into bin 2032) says which bin each threshold lies in; the weights from the
-// lower of these bins upwards (the candidates: usually a few hundred of the row) are gathered in LDS, and one
-// wave bisects over the bit patterns within the bin there.  Counts are integers and sums are sums of the
+// lower of these bins upwards (the candidates: usually a few hundred of the row) are gathered in LDS, where the
+// threshold's bin is counted by the next ten bits of the patterns and that sub-bin by the last nine.  Counts are integers and sums are sums of the
 // weights in fixed point (units of 2^-40, so a row of a million weights of 1.0 stays below 2^64): neither depends
 // on the order in which the threads add, and the histogram's sums and the candidates' agree exactly.  A row whose
-// candidates do not fit (more than SAMPLE_CANDIDATES: a wide nucleus) goes over the whole row twice more per threshold
-// instead: the weights of the threshold's bin are counted by their next ten bits, then those of that sub-bin by
-// their last nine (refine_threshold).
+// candidates do not fit (more than SAMPLE_CANDIDATES: a wide nucleus) makes the same two passes per threshold over
+// the whole row instead (refine_threshold).
 #define HIST_MANTISSA 4
 #define HIST_SHIFT (23 - HIST_MANTISSA)
 #define HIST_BINS 2048
@@ -292,21 +291,12 @@ typedef unsigned long long u64;
 
 __device__ __forceinline__ u64 weight_fixed(float x) { return (u64)(x * 1099511627776.0f); }   // x * 2^40, x in [0, 1]
 
-__device__ __forceinline__ u64 wave_sum_u64(u64 v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
-}
-__device__ __forceinline__ int wave_sum_int(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
-}
-
 struct SampleShared {
   float cand[SAMPLE_CANDIDATES];
   unsigned count[HIST_BINS];     // after the scan: the number of weights in this bin or a higher one
   u64 sum[HIST_BINS];            // after the scan: their sum in fixed point
+  unsigned sub_count[1024];      // the same for the sub-bins of one bin (refine_threshold)
+  u64 sub_sum[1024];
   unsigned wave_count[16];
   u64 wave_sum[16];
   float seg_sum[16];
@@ -374,18 +364,17 @@ __device__ __forceinline__ int last_bin_reaching(const T* table, T need, int lo,
 // The exact threshold inside bin ``bin1`` of the histogram, over the whole row: the largest pattern t for which the
 // weights >= t number at least ``need`` (BY_SUM false) or sum to at least ``need`` in fixed point (BY_SUM true), given
 // what lies above the bin (``above_count`` weights that sum to ``above_sum``) and that the bin's lower edge satisfies
-// it.  Two passes: the bin's weights by the next ten bits of their patterns, then the chosen sub-bin's by the last
-// nine.  The histograms live in the memory of the candidates, which such a row does not use.  Every thread returns
-// the pattern and the sum of the weights that reach it.
+// it.  Two passes over ``w`` [V] (the candidates in LDS, or in memory where they do not fit there): the bin's weights
+// by the next ten bits of their patterns, then the chosen sub-bin's by the last nine.  Every thread returns the
+// pattern and the sum of the weights that reach it.
 struct Refined { unsigned bits; u64 sum_from; };
 
 template <bool BY_SUM>
 __device__ Refined refine_threshold(const float* __restrict__ w, int V, unsigned bin1, unsigned above_count, u64 above_sum,
                                     u64 need, SampleShared& sh) {
-  static_assert(SAMPLE_THREADS == 1024 && SAMPLE_CANDIDATES * sizeof(float) >= 1024 * (sizeof(unsigned) + sizeof(u64)),
-                "one sub-bin per thread, in the candidates' memory");
-  unsigned* c2 = reinterpret_cast<unsigned*>(sh.cand);
-  u64* s2 = reinterpret_cast<u64*>(sh.cand + 1024);
+  static_assert(SAMPLE_THREADS == 1024, "one sub-bin per thread");
+  unsigned* c2 = sh.sub_count;
+  u64* s2 = sh.sub_sum;
   const int tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
   unsigned prefix = bin1;      // the pattern's bits from ``shift`` upwards
   int shift = HIST_SHIFT;
@@ -505,9 +494,61 @@ __device__ int cumulative_pick(const float* __restrict__ w, int V, unsigned thr_
   return sh.pick;
 }
 
+// Thread 0 of the workgroup: the bins that hold the thresholds of top-k (sh.bin_k) and top-p (sh.bin_p, found with at
+// least what the exact rule will ask for: top-k keeps no more than the bins from bin_k upwards hold) and the lower of
+// them (sh.bin_cand: the weights from there upwards are the candidates), from the scanned histogram.
+__device__ void choose_bins(SampleShared& sh, bool k_on, int k, bool p_on, float top_p) {
+  const int top_bin = __float_as_uint(1.0f) >> HIST_SHIFT;
+  int bk = 0, bp = 0, bc = top_bin;
+  if (k_on) { bk = last_bin_reaching(sh.count, (unsigned)k, 0, top_bin); bc = min(bc, bk); }
+  if (p_on) {
+    const u64 need = (u64)((double)top_p * (double)sh.sum[bk]);
+    bp = last_bin_reaching(sh.sum, need, 0, top_bin);
+    bc = min(bc, bp);
+  }
+  sh.bin_k = bk; sh.bin_p = bp; sh.bin_cand = bc;
+}
+
+// The whole workgroup: the exact thresholds from ``w`` [n], which holds at least every weight from the candidates' bin
+// upwards (the candidates in LDS; the list of them in memory, or the whole row, where they do not fit), by two passes
+// per threshold.  Thresholds are bit patterns: for non-negative floats the order of the values is the order of their
+// bits; the largest weight is 1.
+__device__ unsigned thresholds_by_refinement(const float* __restrict__ w, int n, SampleShared& sh, bool k_on, int k, bool p_on,
+                                             float top_p) {
+  const int top_bin = __float_as_uint(1.0f) >> HIST_SHIFT, bk = sh.bin_k;
+  unsigned thr_bits = 0;
+  u64 kept_all = sh.sum[0];
+  if (k_on) {
+    const Refined t = refine_threshold<false>(w, n, bk, sh.count[bk + 1], sh.sum[bk + 1], (u64)k, sh);
+    thr_bits = t.bits;
+    kept_all = t.sum_from;
+  }
+  if (p_on) {
+    const u64 need = (u64)((double)top_p * (double)kept_all);
+    const int b = last_bin_reaching(sh.sum, need, 0, top_bin);
+    const Refined t = refine_threshold<true>(w, n, b, sh.count[b + 1], sh.sum[b + 1], need, sh);
+    thr_bits = max(thr_bits, t.bits);   // (it is at least top-k's: the weights that reach that one sum to kept_all >= need)
+  }
+  return thr_bits;
+}
+
+__device__ __forceinline__ unsigned with_min_p(unsigned thr_bits, float min_p) {
+  if (min_p > 0.f) {
+    const unsigned mb = __float_as_uint(fminf(min_p, 1.0f));
+    if (mb > thr_bits) thr_bits = mb;
+  }
+  return thr_bits;
+}
+
+__device__ __forceinline__ float row_uniform(const SampleArgs& a, int r) {
+  return a.uniform ? a.uniform[r] : philox_uniform(a.draws[4 * r], a.draws[4 * r + 1], a.draws[4 * r + 2], a.draws[4 * r + 3]);
+}
+
+// One workgroup takes a row whole: the form for vocabularies below SLICED_MIN_V tokens and for more than
+// SLICED_MAX_ROWS rows (below).
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   __shared__ SampleShared sh;
-  const int r = blockIdx.x, V = a.V, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  const int r = blockIdx.x, V = a.V, tid = threadIdx.x, wid = tid / WAVE;
   const float* row = a.logits + (size_t)r * V;
   const float temp = a.temperature[r];
   if (!(temp > 0.f)) {
@@ -525,9 +566,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   block_visit(row, V, [&](int, float l) { mx = fmaxf(mx, l * inv_t); });
   mx = block_max(mx, sh.red_f);
 
-  // Thresholds as bit patterns: for non-negative floats the order of the values is the order
-  // of their bits.  The largest weight is exp(0) = 1.
-  const unsigned one_bits = __float_as_uint(1.0f);
   unsigned thr_bits = 0;  // keep everything
   if (!k_on && !p_on) {
     block_map(row, w, V, [&](float l) { return expf(l * inv_t - mx); });
@@ -547,20 +585,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
     });
     __syncthreads();
     histogram_suffix_scan<true>(sh.count, sh.sum, sh.wave_count, sh.wave_sum, V);
-    if (tid == 0) {
-      const int top_bin = one_bits >> HIST_SHIFT;
-      int bk = 0, bp = 0, bc = top_bin;
-      if (k_on) { bk = last_bin_reaching(sh.count, (unsigned)k, 0, top_bin); bc = min(bc, bk); }
-      if (p_on) {
-        // at least what the exact rule will ask for: top-k keeps no more than the bins from bk upwards hold
-        const u64 need = (u64)((double)top_p * (double)sh.sum[bk]);
-        bp = last_bin_reaching(sh.sum, need, 0, top_bin);
-        bc = min(bc, bp);
-      }
-      sh.bin_k = bk; sh.bin_p = bp; sh.bin_cand = bc;
-    }
+    if (tid == 0) choose_bins(sh, k_on, k, p_on, top_p);
     __syncthreads();
-    const int bk = sh.bin_k, bc = sh.bin_cand;
+    const int bc = sh.bin_cand;
     if (sh.count[bc] <= SAMPLE_CANDIDATES) {
       const unsigned first_bits = (unsigned)bc << HIST_SHIFT;
       block_visit(w, V, [&](int, float x) {
@@ -570,79 +597,364 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
         }
       });
       __syncthreads();
-      if (wid == 0) {
-        const int n = min(sh.n_cand, (unsigned)SAMPLE_CANDIDATES);
-        if (k_on) {  // the largest pattern that at least k weights reach: it lies in bin bk
-          unsigned lo = (unsigned)bk << HIST_SHIFT, hi = min(((unsigned)(bk + 1) << HIST_SHIFT) - 1, one_bits);
-          while (lo < hi) {
-            const unsigned mid = lo + (hi - lo + 1) / 2;
-            int c = 0;
-            for (int i = lane; i < n; i += WAVE) c += __float_as_uint(sh.cand[i]) >= mid ? 1 : 0;
-            if (wave_sum_int(c) >= k) lo = mid; else hi = mid - 1;
-          }
-          thr_bits = lo;
-        }
-        if (p_on) {  // the largest pattern whose weights and all larger ones sum to top_p of what top-k kept
-          u64 kept = 0;
-          for (int i = lane; i < n; i += WAVE) {
-            const float x = sh.cand[i];
-            if (__float_as_uint(x) >= thr_bits) kept += weight_fixed(x);
-          }
-          const u64 kept_all = k_on ? wave_sum_u64(kept) : sh.sum[0];   // without top-k: the whole row, not the candidates
-          const u64 need = (u64)((double)top_p * (double)kept_all);
-          const int tb = thr_bits >> HIST_SHIFT;
-          const int b = last_bin_reaching(sh.sum, need, tb, (int)(one_bits >> HIST_SHIFT));
-          unsigned lo = max(thr_bits, (unsigned)b << HIST_SHIFT), hi = min(((unsigned)(b + 1) << HIST_SHIFT) - 1, one_bits);
-          while (lo < hi) {
-            const unsigned mid = lo + (hi - lo + 1) / 2;
-            u64 s = 0;
-            for (int i = lane; i < n; i += WAVE) {
-              const float x = sh.cand[i];
-              if (__float_as_uint(x) >= mid) s += weight_fixed(x);
-            }
-            if (wave_sum_u64(s) >= need) lo = mid; else hi = mid - 1;
-          }
-          thr_bits = lo;
-        }
-        if (lane == 0) sh.thr_bits = thr_bits;
-      }
-      __syncthreads();
-      thr_bits = sh.thr_bits;
+      thr_bits = thresholds_by_refinement(sh.cand, min(sh.n_cand, (unsigned)SAMPLE_CANDIDATES), sh, k_on, k, p_on, top_p);
     } else {
-      const int top_bin = one_bits >> HIST_SHIFT;
-      u64 kept_all = sh.sum[0];
-      if (k_on) {
-        const Refined t = refine_threshold<false>(w, V, bk, sh.count[bk + 1], sh.sum[bk + 1], (u64)k, sh);
-        thr_bits = t.bits;
-        kept_all = t.sum_from;
-      }
-      if (p_on) {
-        const u64 need = (u64)((double)top_p * (double)kept_all);
-        const int b = last_bin_reaching(sh.sum, need, 0, top_bin);
-        const Refined t = refine_threshold<true>(w, V, b, sh.count[b + 1], sh.sum[b + 1], need, sh);
-        thr_bits = max(thr_bits, t.bits);   // (it is at least top-k's: the weights that reach that one sum to kept_all >= need)
-      }
+      thr_bits = thresholds_by_refinement(w, V, sh, k_on, k, p_on, top_p);
     }
   }
-  const float min_p = a.min_p[r];
-  if (min_p > 0.f) {
-    const unsigned mb = __float_as_uint(fminf(min_p, 1.0f));
-    if (mb > thr_bits) thr_bits = mb;
-  }
-  const float u = a.uniform ? a.uniform[r]
-                            : philox_uniform(a.draws[4 * r], a.draws[4 * r + 1], a.draws[4 * r + 2], a.draws[4 * r + 3]);
-  const int pick = cumulative_pick(w, V, thr_bits, u, sh);
+  thr_bits = with_min_p(thr_bits, a.min_p[r]);
+  const int pick = cumulative_pick(w, V, thr_bits, row_uniform(a, r), sh);
   if (tid == 0) a.out[r] = pick;
 }
 
+// ---------------------------------------------------------------------------------------
+// The same draw for large vocabularies with SAMPLE_SLICES workgroups to a row.  One workgroup pulls a row through one
+// compute unit, 12 us a pass over 152,064 weights; here each pass is a launch of its own in which every wave of every
+// workgroup takes one of the row's SAMPLE_SEGMENTS segments, and what the passes hand each other lies in scratch
+// memory:
+//   1. the largest logit of each slice;
+//   2. the weights, and for rows with top-k or top-p the histogram (each workgroup's in LDS, added to the row's with
+//      integer atomics: no order to depend on); rows without them get their segments' sums here already;
+//   3. the candidates: every workgroup scans the row's histogram for itself, finds the candidates' bin and appends
+//      its slice's candidates to the row's list (their order depends on timing, nothing computed from them does);
+//   4. the thresholds, again by every workgroup for itself (in LDS from up to SAMPLE_CANDIDATES candidates, else by
+//      refinement over the list), and the sum of the kept weights of each segment;
+//   5. one wave per row finds the segment where the cumulative sum passes uniform * total and walks it.
+// Rows with temperature <= 0 are left to an argmax launch.  The result depends on the row and its number alone.
+// Measured on 152,064-token rows inside a replayed graph, us one workgroup a row / sliced: a temperature alone 35 / 17
+// at one row, 36 / 21 at 8, 50 / 45 at 64; with top-k 50 and top-p 0.9: 73 / 49, 74 / 52, 96 / 162 (every workgroup scans
+// the row's histogram and finds the thresholds for itself: with 64 rows that is 1,024 times), so up to 16 rows are sliced.
+#define SAMPLE_SLICES 16
+#define SAMPLE_SEGMENTS (SAMPLE_SLICES * (SAMPLE_THREADS / WAVE))
+#define SLICED_MIN_V 32768        // smaller vocabularies, and
+#define SLICED_MAX_ROWS 16        // more rows (which fill compute units enough by themselves): one workgroup a row, one launch;
+#define SLICED_MAX_ROWS_PLAIN 64  // without top-k and top-p (three short launches) the sliced form pays up to this many
+
+struct SlicedArgs {
+  SampleArgs a;
+  float* slice_max;       // [R, SAMPLE_SLICES]
+  u64* hist_sum;          // [R, HIST_BINS]
+  unsigned* hist_count;   // [R, HIST_BINS]
+  float* cand;            // [R, V]
+  unsigned* n_cand;       // [R]
+  unsigned* thr_bits;     // [R]
+  float* seg_sum;         // [R, SAMPLE_SEGMENTS]
+  int* seg_last;          // [R, SAMPLE_SEGMENTS]
+  int seg;                // elements of a segment (a multiple of 64)
+  int any_filters;        // 0: top-k and top-p are taken as off in every row
+};
+
+struct RowFilters { bool k_on, p_on; int k; float top_p; };
+__device__ __forceinline__ RowFilters row_filters(const SlicedArgs& g, int r) {
+  const int k = g.a.top_k[r];
+  const float top_p = g.a.top_p[r];
+  return RowFilters{g.any_filters && k > 0 && k < g.a.V, g.any_filters && top_p > 0.f && top_p < 1.f, k, top_p};
+}
+
+// The sum of the weights of segment [a0, a1) that reach thr_bits, and the last index that does (-1: none): one wave.
+__device__ __forceinline__ void segment_kept(const float* __restrict__ w, int a0, int a1, unsigned thr_bits, float& sum, int& last) {
+  const int lane = threadIdx.x % WAVE;
+  float mine = 0.f;
+  last = -1;
+  for (int i = a0 + lane; i < a1; i += WAVE) {
+    const float x = w[i];
+    if (__float_as_uint(x) >= thr_bits) { mine += x; last = i; }
+  }
+  sum = wave_sum(mine);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) last = max(last, __shfl_xor(last, o, WAVE));
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sliced_max_kernel(SlicedArgs g) {
+  __shared__ float red[16];
+  const int sl = blockIdx.x, r = blockIdx.y, V = g.a.V, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  const float temp = g.a.temperature[r];
+  if (!(temp > 0.f)) return;
+  const float inv_t = 1.0f / temp;
+  const float* row = g.a.logits + (size_t)r * V;
+  const int j = sl * (SAMPLE_THREADS / WAVE) + wid, a0 = min(V, j * g.seg), a1 = min(V, a0 + g.seg);
+  float mx = -INFINITY;
+  for (int i = a0 + lane; i < a1; i += WAVE) mx = fmaxf(mx, row[i] * inv_t);
+  mx = block_max(mx, red);
+  if (tid == 0) g.slice_max[r * SAMPLE_SLICES + sl] = mx;
+  // this workgroup's share of the row's histogram starts at zero, and the row's list of candidates empty
+  constexpr int share = HIST_BINS / SAMPLE_SLICES;
+  if (tid < share) {
+    g.hist_count[(size_t)r * HIST_BINS + sl * share + tid] = 0;
+    g.hist_sum[(size_t)r * HIST_BINS + sl * share + tid] = 0;
+  }
+  if (sl == 0 && tid == 0) g.n_cand[r] = 0;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sliced_weights_kernel(SlicedArgs g) {
+  __shared__ unsigned count[HIST_BINS];
+  __shared__ u64 sum[HIST_BINS];
+  const int sl = blockIdx.x, r = blockIdx.y, V = g.a.V, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  const float temp = g.a.temperature[r];
+  if (!(temp > 0.f)) return;
+  const float inv_t = 1.0f / temp;
+  const float* row = g.a.logits + (size_t)r * V;
+  float* w = g.a.weights + (size_t)r * V;
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < SAMPLE_SLICES; ++i) mx = fmaxf(mx, g.slice_max[r * SAMPLE_SLICES + i]);
+  const RowFilters f = row_filters(g, r);
+  const bool filters = f.k_on || f.p_on;
+  if (filters) {
+    for (int b = tid; b < HIST_BINS; b += blockDim.x) { count[b] = 0; sum[b] = 0; }
+    __syncthreads();
+  }
+  const int j = sl * (SAMPLE_THREADS / WAVE) + wid, a0 = min(V, j * g.seg), a1 = min(V, a0 + g.seg);
+  const unsigned thr_bits = with_min_p(0, g.a.min_p[r]);     // (without top-k and top-p the threshold is known here)
+  float mine = 0.f;
+  int last = -1;
+  for (int i = a0 + lane; i < a1; i += WAVE) {
+    const float x = expf(row[i] * inv_t - mx);
+    w[i] = x;
+    if (filters) {
+      const unsigned b = __float_as_uint(x) >> HIST_SHIFT;
+      if (b && b < HIST_BINS) {   // (a NaN's pattern lies beyond the last bin)
+        atomicAdd(&count[b], 1u);
+        atomicAdd(&sum[b], weight_fixed(x));
+      }
+    } else if (__float_as_uint(x) >= thr_bits) {
+      mine += x;
+      last = i;
+    }
+  }
+  if (filters) {
+    __syncthreads();
+    for (int b = tid; b < HIST_BINS; b += blockDim.x) {
+      const unsigned c = count[b];
+      if (c) {
+        atomicAdd(&g.hist_count[(size_t)r * HIST_BINS + b], c);
+        atomicAdd(&g.hist_sum[(size_t)r * HIST_BINS + b], sum[b]);
+      }
+    }
+    return;
+  }
+  mine = wave_sum(mine);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) last = max(last, __shfl_xor(last, o, WAVE));
+  if (lane == 0) {
+    g.seg_sum[r * SAMPLE_SEGMENTS + j] = mine;
+    g.seg_last[r * SAMPLE_SEGMENTS + j] = last;
+  }
+  if (sl == 0 && tid == 0) g.thr_bits[r] = thr_bits;
+}
+
+// The row's histogram from memory into sh, scanned, and the bins chosen (the same in every workgroup of the row).
+__device__ void load_row_bins(const SlicedArgs& g, int r, const RowFilters& f, SampleShared& sh) {
+  const int tid = threadIdx.x;
+  for (int b = tid; b < HIST_BINS; b += blockDim.x) {
+    sh.count[b] = g.hist_count[(size_t)r * HIST_BINS + b];
+    sh.sum[b] = g.hist_sum[(size_t)r * HIST_BINS + b];
+  }
+  __syncthreads();
+  histogram_suffix_scan<true>(sh.count, sh.sum, sh.wave_count, sh.wave_sum, g.a.V);
+  if (tid == 0) choose_bins(sh, f.k_on, f.k, f.p_on, f.top_p);
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sliced_gather_kernel(SlicedArgs g) {
+  __shared__ SampleShared sh;
+  __shared__ unsigned wave_n[SAMPLE_THREADS / WAVE + 1];
+  const int sl = blockIdx.x, r = blockIdx.y, V = g.a.V, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  if (!(g.a.temperature[r] > 0.f)) return;
+  const RowFilters f = row_filters(g, r);
+  if (!f.k_on && !f.p_on) return;
+  load_row_bins(g, r, f, sh);
+  const unsigned first_bits = (unsigned)sh.bin_cand << HIST_SHIFT;
+  const float* w = g.a.weights + (size_t)r * V;
+  const int j = sl * (SAMPLE_THREADS / WAVE) + wid, a0 = min(V, j * g.seg), a1 = min(V, a0 + g.seg);
+  unsigned mine = 0;
+  for (int i0 = a0; i0 < a1; i0 += WAVE) {
+    const int i = i0 + lane;
+    mine += __popcll(__ballot(i < a1 && __float_as_uint(w[i]) >= first_bits));
+  }
+  if (lane == 0) wave_n[wid] = mine;
+  __syncthreads();
+  if (tid == 0) {   // one place in the row's list for the workgroup's candidates, wave after wave
+    unsigned total = 0;
+    for (int i = 0; i < SAMPLE_THREADS / WAVE; ++i) { const unsigned c = wave_n[i]; wave_n[i] = total; total += c; }
+    wave_n[SAMPLE_THREADS / WAVE] = total ? atomicAdd(&g.n_cand[r], total) : 0;
+  }
+  __syncthreads();
+  unsigned at = wave_n[SAMPLE_THREADS / WAVE] + wave_n[wid];
+  float* cand = g.cand + (size_t)r * V;
+  for (int i0 = a0; i0 < a1; i0 += WAVE) {
+    const int i = i0 + lane;
+    const float x = i < a1 ? w[i] : 0.f;
+    const bool is = i < a1 && __float_as_uint(x) >= first_bits;
+    const u64 m = __ballot(is);
+    if (is) cand[at + __popcll(m & ((1ull << lane) - 1))] = x;
+    at += __popcll(m);
+  }
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sliced_sums_kernel(SlicedArgs g) {
+  __shared__ SampleShared sh;
+  const int sl = blockIdx.x, r = blockIdx.y, V = g.a.V, tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+  if (!(g.a.temperature[r] > 0.f)) return;
+  const RowFilters f = row_filters(g, r);
+  if (!f.k_on && !f.p_on) return;                  // (such a row's sums were made with its weights)
+  load_row_bins(g, r, f, sh);
+  const int n = (int)g.n_cand[r];
+  const float* cand = g.cand + (size_t)r * V;
+  unsigned thr_bits;
+  if (n <= SAMPLE_CANDIDATES) {
+    for (int i = tid; i < n; i += blockDim.x) sh.cand[i] = cand[i];
+    __syncthreads();
+    thr_bits = thresholds_by_refinement(sh.cand, n, sh, f.k_on, f.k, f.p_on, f.top_p);
+  } else {
+    thr_bits = thresholds_by_refinement(cand, n, sh, f.k_on, f.k, f.p_on, f.top_p);
+  }
+  thr_bits = with_min_p(thr_bits, g.a.min_p[r]);
+  const int j = sl * (SAMPLE_THREADS / WAVE) + wid, a0 = min(V, j * g.seg), a1 = min(V, a0 + g.seg);
+  float kept;
+  int last;
+  segment_kept(g.a.weights + (size_t)r * V, a0, a1, thr_bits, kept, last);
+  if (lane == 0) {
+    g.seg_sum[r * SAMPLE_SEGMENTS + j] = kept;
+    g.seg_last[r * SAMPLE_SEGMENTS + j] = last;
+  }
+  if (sl == 0 && tid == 0) g.thr_bits[r] = thr_bits;
+}
+
+// One wave per row: lane l holds the segments 4 l ... 4 l + 3 (SAMPLE_SEGMENTS = 256), their sums are added in segment
+// order, and the segment in which the cumulative sum passes uniform * total is walked 64 weights at a time.  A target
+// that rounding puts past the end of the segment, or of the row, gives the last kept index there.
+__global__ __launch_bounds__(WAVE) void sliced_pick_kernel(SlicedArgs g) {
+  static_assert(SAMPLE_SEGMENTS == 4 * WAVE, "four segments to a lane");
+  const int r = blockIdx.x, V = g.a.V, lane = threadIdx.x;
+  if (!(g.a.temperature[r] > 0.f)) return;
+  const float* w = g.a.weights + (size_t)r * V;
+  const unsigned thr_bits = g.thr_bits[r];
+  float s[4], mine = 0.f;
+  int last_any = -1;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    s[q] = g.seg_sum[r * SAMPLE_SEGMENTS + 4 * lane + q];
+    mine += s[q];
+    last_any = max(last_any, g.seg_last[r * SAMPLE_SEGMENTS + 4 * lane + q]);
+  }
+  float upto = mine;      // the sum of this lane's segments and all before them
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const float up = __shfl_up(upto, o, WAVE);
+    if (lane >= o) upto += up;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) last_any = max(last_any, __shfl_xor(last_any, o, WAVE));
+  const float total = __shfl(upto, WAVE - 1, WAVE);
+  float target = row_uniform(g.a, r) * total;
+  // the first segment with anything kept whose end the target lies before
+  float before = upto - mine;
+  int found = -1;
+  float found_before = 0.f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (found < 0 && s[q] > 0.f && target - before < s[q]) { found = 4 * lane + q; found_before = before; }
+    before += s[q];
+  }
+  const u64 any = __ballot(found >= 0);
+  int pick = max(last_any, 0);
+  if (any) {
+    const int src = __ffsll((long long)any) - 1;
+    const int j = __shfl(found, src, WAVE);
+    target -= __shfl(found_before, src, WAVE);
+    const int a0 = min(V, j * g.seg), a1 = min(V, a0 + g.seg);
+    float run = 0.f;
+    int hit_at = -1, last = -1;
+    for (int i0 = a0; i0 < a1 && hit_at < 0; i0 += WAVE) {
+      const int i = i0 + lane;
+      const float x = i < a1 ? w[i] : 0.f;
+      const bool kept = i < a1 && __float_as_uint(x) >= thr_bits;
+      float cum = kept ? x : 0.f;
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const float up = __shfl_up(cum, o, WAVE);
+        if (lane >= o) cum += up;
+      }
+      cum += run;
+      const u64 hit = __ballot(kept && target < cum);
+      const u64 keeps = __ballot(kept);
+      if (hit) hit_at = i0 + __ffsll((long long)hit) - 1;
+      if (keeps) last = i0 + 63 - __clzll((long long)keeps);
+      run = __shfl(cum, WAVE - 1, WAVE);
+    }
+    pick = hit_at >= 0 ? hit_at : max(last, 0);
+  }
+  if (lane == 0) g.a.out[r] = pick;
+}
+
+// Rows with temperature <= 0 of a launch whose other rows are drawn by the sliced kernels.
+__global__ __launch_bounds__(SAMPLE_THREADS) void greedy_rows_kernel(SampleArgs a) {
+  __shared__ float red_v[16];
+  __shared__ int red_i[16];
+  const int r = blockIdx.x;
+  if (a.temperature[r] > 0.f) return;
+  const int best = block_argmax(a.logits + (size_t)r * a.V, a.V, red_v, red_i);
+  if (threadIdx.x == 0) a.out[r] = best;
+}
+
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// The scratch memory ifx_sample needs besides the weights [R, V], in blocks of 256 bytes (0: a launch of the
+// one-workgroup form).
+static bool sliced_form(int R, int V, int any_filters) {
+  return V >= SLICED_MIN_V && R <= (any_filters ? SLICED_MAX_ROWS : SLICED_MAX_ROWS_PLAIN);
+}
+
+extern "C" int ifx_sample_scratch_blocks(int R, int V, int any_filters) {
+  if (R <= 0 || !sliced_form(R, V, any_filters)) return 0;
+  const size_t rows = (size_t)R;
+  return (int)((align256(rows * SAMPLE_SLICES * sizeof(float)) + align256(rows * HIST_BINS * sizeof(u64)) +
+                align256(rows * HIST_BINS * sizeof(unsigned)) + align256(rows * (size_t)V * sizeof(float)) +
+                align256(rows * sizeof(unsigned)) * 2 + align256(rows * SAMPLE_SEGMENTS * sizeof(float)) * 2) / 256);
+}
+
+// ``scratch``: ifx_sample_scratch_blocks(R, V, any_filters) blocks of 256 bytes, aligned to 256 (or null when that is 0).  ``any_greedy`` 0: the
+// caller knows that every row has a temperature above zero; ``any_filters`` 0: that no row has top-k or top-p (each
+// saves the sliced form launches that would find nothing to do).
 extern "C" int ifx_sample(const float* logits, float* weights, const float* temperature, const int* top_k,
                           const float* top_p, const float* min_p, const float* uniform, const unsigned* draws, int* out,
-                          int R, int V, void* stream) {
+                          int R, int V, void* scratch, int any_greedy, int any_filters, void* stream) {
   IFX_REQUIRE(R >= 0 && V > 0, "sample: bad sizes R=%d V=%d", R, V);
   IFX_REQUIRE((uniform != nullptr) != (draws != nullptr), "sample: either the uniform numbers or the seeds and counters of the draws");
   if (R == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
   SampleArgs a{logits, weights, temperature, top_k, top_p, min_p, uniform, draws, out, V};
-  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, a);
+  if (!sliced_form(R, V, any_filters)) {
+    hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, s, a);
+    IFX_LAUNCH_CHECK();
+  }
+  IFX_REQUIRE(scratch != nullptr && ((size_t)scratch & 255) == 0, "sample: needs ifx_sample_scratch_blocks() of scratch memory, aligned to 256");
+  IFX_REQUIRE(R <= 65535, "sample: %d rows in one launch (at most 65,535)", R);
+  unsigned char* at = (unsigned char*)scratch;
+  auto take = [&](size_t bytes) { unsigned char* p = at; at += align256(bytes); return p; };
+  const size_t rows = (size_t)R;
+  SlicedArgs g;
+  g.a = a;
+  g.slice_max = (float*)take(rows * SAMPLE_SLICES * sizeof(float));
+  g.hist_sum = (u64*)take(rows * HIST_BINS * sizeof(u64));
+  g.hist_count = (unsigned*)take(rows * HIST_BINS * sizeof(unsigned));
+  g.cand = (float*)take(rows * (size_t)V * sizeof(float));
+  g.n_cand = (unsigned*)take(rows * sizeof(unsigned));
+  g.thr_bits = (unsigned*)take(rows * sizeof(unsigned));
+  g.seg_sum = (float*)take(rows * SAMPLE_SEGMENTS * sizeof(float));
+  g.seg_last = (int*)take(rows * SAMPLE_SEGMENTS * sizeof(int));
+  g.seg = ((V + SAMPLE_SEGMENTS - 1) / SAMPLE_SEGMENTS + WAVE - 1) / WAVE * WAVE;
+  g.any_filters = any_filters;
+  const dim3 slices(SAMPLE_SLICES, R);
+  if (any_greedy) hipLaunchKernelGGL(greedy_rows_kernel, dim3(R), dim3(SAMPLE_THREADS), 0, s, a);
+  hipLaunchKernelGGL(sliced_max_kernel, slices, dim3(SAMPLE_THREADS), 0, s, g);
+  hipLaunchKernelGGL(sliced_weights_kernel, slices, dim3(SAMPLE_THREADS), 0, s, g);
+  if (any_filters) {
+    hipLaunchKernelGGL(sliced_gather_kernel, slices, dim3(SAMPLE_THREADS), 0, s, g);
+    hipLaunchKernelGGL(sliced_sums_kernel, slices, dim3(SAMPLE_THREADS), 0, s, g);
+  }
+  hipLaunchKernelGGL(sliced_pick_kernel, dim3(R), dim3(WAVE), 0, s, g);
   IFX_LAUNCH_CHECK();
 }
 

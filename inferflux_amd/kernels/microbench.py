@@ -158,10 +158,10 @@ def sampling(args) -> None:
     t08, t1, k0, k50, p1, p09, m0, m001 = (full(0.8), full(1.0), full(0, torch.int32), full(50, torch.int32), full(1.0), full(0.9),
                                            full(0.0), full(0.01))
     cases = [("argmax", lambda i: ops.argmax(logits)),
-             ("temperature 0.8", lambda i: ops.sample(logits, t08, k0, p1, m0, u)),
-             ("temperature 0.8, top-k 50, top-p 0.9", lambda i: ops.sample(logits, t08, k50, p09, m0, u)),
-             ("temperature 0.8, top-p 0.9", lambda i: ops.sample(logits, t08, k0, p09, m0, u)),
-             ("temperature 1, min-p 0.01", lambda i: ops.sample(logits, t1, k0, p1, m001, u)),
+             ("temperature 0.8", lambda i: ops.sample(logits, t08, k0, p1, m0, u, any_greedy=False, any_filters=False)),
+             ("temperature 0.8, top-k 50, top-p 0.9", lambda i: ops.sample(logits, t08, k50, p09, m0, u, any_greedy=False)),
+             ("temperature 0.8, top-p 0.9", lambda i: ops.sample(logits, t08, k0, p09, m0, u, any_greedy=False)),
+             ("temperature 1, min-p 0.01", lambda i: ops.sample(logits, t1, k0, p1, m001, u, any_greedy=False, any_filters=False)),
              ("log-probabilities, 5 alternatives", lambda i: ops.logprobs(logits, chosen, 5)),
              ("log-probability of the token alone", lambda i: ops.logprobs(logits, chosen, 0))]
     for name, fn in cases:

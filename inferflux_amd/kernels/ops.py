@@ -886,8 +886,11 @@ def add_logit_bias(logits: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, 
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           min_p: torch.Tensor, uniform: Optional[torch.Tensor] = None, draws: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One token per row of float32 ``logits`` [R, V]; rows with temperature <= 0 take the argmax.  The number in
+           min_p: torch.Tensor, uniform: Optional[torch.Tensor] = None, draws: Optional[torch.Tensor] = None,
+           any_greedy: bool = True, any_filters: bool = True) -> torch.Tensor:
+    """One token per row of float32 ``logits`` [R, V]; rows with temperature <= 0 take the argmax (``any_greedy``
+    False: the caller knows that there is no such row; ``any_filters`` False: that no row has top-k or top-p; both
+    save launches that would find nothing to do).  The number in
     [0, 1) that a row's draw uses is either given (``uniform`` [R]) or made by the kernel from ``draws`` (int32
     [R, 4]: the row's seed and the count of its draws so far, 64 bits each, low word first), as
     ``sampling.params.philox_uniform`` makes it."""
@@ -903,12 +906,17 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         _check(uniform, "uniform", (R,), torch.float32)
     else:
         _check(draws, "draws", (R, 4), torch.int32)
+    mod = load_module("sampling")
     weights = torch.empty_like(logits)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    _call(load_module("sampling"), "ifx_sample", (P, P, P, P, P, P, P, P, P, I, I, P),
+    # large vocabularies are drawn by several workgroups a row, which hand each other their results in scratch memory
+    n_scratch = mod.fn("ifx_sample_scratch_blocks", (I, I, I))(R, V, 1 if any_filters else 0)
+    scratch = torch.empty((n_scratch * 256,), dtype=torch.uint8, device=logits.device) if n_scratch else None
+    _call(mod, "ifx_sample", (P, P, P, P, P, P, P, P, P, I, I, P, I, I, P),
           logits.data_ptr(), weights.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
           min_p.data_ptr(), uniform.data_ptr() if uniform is not None else None,
-          draws.data_ptr() if draws is not None else None, out.data_ptr(), R, V, _stream())
+          draws.data_ptr() if draws is not None else None, out.data_ptr(), R, V, _ptr(scratch), 1 if any_greedy else 0,
+          1 if any_filters else 0, _stream())
     return out
 
 

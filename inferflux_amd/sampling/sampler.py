@@ -138,7 +138,9 @@ class Sampler:
                 np.asarray([s.params.top_k for s in states], np.int32),
                 np.asarray([s.params.top_p for s in states], np.float32),
                 np.asarray([s.params.min_p for s in states], np.float32), words)
-            chosen = ops.sample(logits, temperature, top_k, top_p, min_p, draws=draws.view(R, 4))
+            chosen = ops.sample(logits, temperature, top_k, top_p, min_p, draws=draws.view(R, 4),
+                                any_greedy=any(s.params.greedy for s in states),
+                                any_filters=any(s.params.top_k > 0 or s.params.top_p < 1.0 for s in states))
         top_n = max((s.params.logprobs for s in states if s.params.logprobs is not None), default=None)
         if top_n is not None:
             lp_dev = ops.logprobs(logits, chosen, top_n)

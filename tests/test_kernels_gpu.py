@@ -551,11 +551,20 @@ def test_sample_rows_of_every_shape(case):
     logits = torch.stack([build(g, V) for _ in range(R)])
     u = torch.tensor([0.0, 0.25, 0.5, 0.75, 0.999999])
     full = lambda v, dt: torch.full((R,), v, dtype=dt, device=DEV)
-    got = ops.sample(logits.to(DEV), full(temp, torch.float32), full(k, torch.int32), full(p, torch.float32),
-                     full(mp, torch.float32), u.to(DEV)).cpu().tolist()
+    args = (logits.to(DEV), full(temp, torch.float32), full(k, torch.int32), full(p, torch.float32), full(mp, torch.float32), u.to(DEV))
+    got = ops.sample(*args).cpu().tolist()
+    assert ops.sample(*args, any_greedy=False).cpu().tolist() == got        # (no row here has temperature 0)
+    # the same rows among twenty: large vocabularies are then drawn by one workgroup a row instead of sixteen
+    many = [torch.cat([t, t, t, t]) for t in args]
+    among = ops.sample(*many).cpu().tolist()
+    assert among[:R] == among[R:2 * R] == among[3 * R:]
     for r in range(R):
         w = pm.filtered_probs(logits[r], temp, k, p, mp)
-        assert w[got[r]] > 0, (name, r, "a filtered-out token was drawn")
+        assert w[got[r]] > 0 and w[among[r]] > 0, (name, r, "a filtered-out token was drawn")
+        if among[r] != got[r]:                   # only a draw on the edge between two kept tokens may differ between the forms
+            cum = torch.cumsum(w.double(), 0) / w.double().sum()
+            a, b = min(among[r], got[r]), max(among[r], got[r])
+            assert abs(float(cum[a]) - float(u[r])) < 1e-4 and float(w[a + 1:b].sum()) == 0.0, (name, r, among[r], got[r])
         cum = torch.cumsum(w.double(), 0) / w.double().sum()
         lo = float(cum[got[r] - 1]) if got[r] > 0 else 0.0
         assert lo - 1e-4 <= float(u[r]) <= float(cum[got[r]]) + 1e-4, (name, r, got[r], lo, float(u[r]), float(cum[got[r]]))
