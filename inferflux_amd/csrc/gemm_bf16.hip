@@ -20,6 +20,7 @@
 // The reference sends these products to cuBLAS (runtime/backends/cuda/native/cublas_gemm.cpp:
 // 99-117) and measured 30-44 % of its roofline there (docs/benchmarks.md:180-183).
 #include "common.h"
+#include "row_scale.h"
 
 IFX_DEFINE_LAST_ERROR()
 
@@ -35,16 +36,6 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-// A normalisation whose factor per row is applied to the product's results instead of to its input:
-// row m of x stands for x[m] * rsqrt(sum_j pieces[j][m] / width + eps).  ``pieces`` is [n][16]
-// (16 rows whatever M is), written by the EPI 2 epilogue below: piece j is the sum of squares of 16
-// consecutive elements of the row before it was weighted.
-struct RowScale {
-  const float* pieces;  // null: no factor
-  int n;
-  float width, eps;
-};
-
 // EPI 2: the product is added to the float stream [M, N] in place, and what the norm that follows needs is
 // written beside it: rows[m, n] = bf16(stream[m, n] * norm_w[n]) and pieces[n / 16][m] (see RowScale).
 struct StreamOut {
@@ -59,40 +50,6 @@ __device__ __forceinline__ float sum_over_groups(float v) {
   v += __shfl_xor(v, 16);
   v += __shfl_xor(v, 32);
   return v;
-}
-
-// The factor of row lane % 16, computed by one wave.  The pieces are read as float4s (rows 4 (c % 4) ... + 3 of
-// piece c / 4 in float4 number c), lane l taking numbers l, l + 64, ...: sixteen loads are in flight at a time
-// (one after the other they would cost a trip to the L2 each), a lane always meets the same four rows, and the
-// sums are added in a fixed order.
-__device__ __forceinline__ float row_factor(const RowScale& s, int lane) {
-  const int chunks = 4 * s.n;
-  floatx4 t{0.f, 0.f, 0.f, 0.f};
-  for (int base = lane; base < chunks; base += WAVE * 16) {
-    floatx4 v[16];
-#pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      const int c = base + WAVE * u;
-      v[u] = c < chunks ? *(const floatx4*)(s.pieces + (size_t)4 * c) : floatx4{0.f, 0.f, 0.f, 0.f};
-    }
-#pragma unroll
-    for (int u = 0; u < 16; ++u)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) t[r] += v[u][r];
-  }
-#pragma unroll
-  for (int off = 4; off < WAVE; off <<= 1)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) t[r] += __shfl_xor(t[r], off);
-  // every lane with lane % 4 == q now holds the sums of rows 4 q ... 4 q + 3
-  const int col = lane & 15;
-  float sum = 0.f;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float from = __shfl(t[r], col >> 2);
-    if ((col & 3) == r) sum = from;
-  }
-  return rsqrtf(sum / s.width + s.eps);
 }
 
 // The sums of one workgroup: acc[nt][mt] = W tile (first_tile + nt) times x rows 16 mt ..., K split over

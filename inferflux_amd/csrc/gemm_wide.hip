@@ -1,5 +1,6 @@
-// Weight-streaming matrix product for 17-128 rows:  out[M,N] = x[M,K] * W[N,K]^T from the tiled copy of W
-// (layout: gemm_bf16.hip), bf16 in, float accumulate on the matrix cores (16x16x32), out bf16 or float.
+// Weight-streaming matrix product for 17-128 rows (and for 9-16 rows of large tall weights):  out[M,N] = x[M,K] * W[N,K]^T
+// from the tiled copy of W (layout: gemm_bf16.hip), bf16 in, float accumulate on the matrix cores (16x16x32), out bf16 or
+// float; up to 16 rows may come with a norm's factor per row, applied to the sums (row_scale.h).
 //
 // At these sizes the product is still bound by reading W once, but every tile of W now meets two to eight
 // tiles of x, and a wave that fetched those from the L2 itself would move more bytes of x than of W.  A
@@ -30,6 +31,7 @@
 //
 // The reference sends these products to cuBLAS (runtime/backends/cuda/native/cublas_gemm.cpp:99-117).
 #include "common.h"
+#include "row_scale.h"
 
 IFX_DEFINE_LAST_ERROR()
 
@@ -69,17 +71,24 @@ __device__ __forceinline__ void store2(bf16_t* p, float a, float b) {
 // ``order``: tile t of the copy holds the weight's rows 16 order[t] ...; null: in order.
 // ``MINW``: the fewest waves a workgroup of this form may have (each thread then copies more pieces of x to LDS and
 // holds them in more registers, which a workgroup of at most 8 waves has).
+// ``scale`` (up to 16 rows): the sums of row m are multiplied by the row's factor (see RowScale).  Every thread asks for
+// its few of the pieces before the first rounds of W and x, so that they arrive first and cost no trip of their own; the
+// waves' shares of the rows' sums meet in LDS.
 template <int MT, typename TO, int EPI, int MINW>
 __global__ __launch_bounds__((16 * MT > MANY_ROWS || MINW < MIN_WAVES ? MIN_WAVES : MAX_WAVES) * WAVE) void wide_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wt,
                                                                      TO* __restrict__ out, float* __restrict__ part, int M,
                                                                      int N, int K, int k_tiles, int rounds_per_slice,
-                                                                     const int* __restrict__ order, int tile_rows) {
+                                                                     const int* __restrict__ order, int tile_rows, RowScale scale) {
   constexpr int R = MT * 16;                                  // rows of x in LDS
   constexpr int X_PIECES = R * WK_PIECES;                     // 16-byte pieces of a round's x
   constexpr int X_PER_THREAD = (X_PIECES + MINW * WAVE - 1) / (MINW * WAVE);
   __shared__ __attribute__((aligned(16))) bf16x8 xs[2][X_PIECES];
+  __shared__ __attribute__((aligned(16))) float row_sums[MAX_WAVES][16];
   const int tid = threadIdx.x, threads = blockDim.x, waves = threads / WAVE;
   const int wid = tid / WAVE, lane = tid % WAVE, col = lane & 15, g = lane >> 4;
+  const bool scaled = MT == 1 && scale.pieces != nullptr;
+  RowSumsEarly pieces_asked;
+  if (scaled) row_sums_ask(scale, tid, threads, pieces_asked);
   const int tile = blockIdx.x * waves + wid, n_tiles = (N + tile_rows - 1) / tile_rows;
   const int n_rounds = (K + WK - 1) / WK;
   const int r_begin = blockIdx.y * rounds_per_slice, n = min(n_rounds, r_begin + rounds_per_slice) - r_begin;
@@ -134,6 +143,10 @@ __global__ __launch_bounds__((16 * MT > MANY_ROWS || MINW < MIN_WAVES ? MIN_WAVE
     store_x(0, xreg[0]);
     if (DEPTH < n) load_x(r_begin + DEPTH, xreg[0]);
   }
+  if (scaled) {
+    const rs_floatx4 sums = row_sums_of_wave(row_sums_of_thread(scale, tid, threads, pieces_asked));
+    if (lane < 4) *(rs_floatx4*)&row_sums[wid][4 * lane] = sums;
+  }
   __syncthreads();
   for (int c0 = 0; c0 < n; c0 += 2 * DEPTH) {   // unrolled over the register sets and the two LDS buffers
 #pragma unroll
@@ -157,6 +170,13 @@ __global__ __launch_bounds__((16 * MT > MANY_ROWS || MINW < MIN_WAVES ? MIN_WAVE
   // multiples of four columns they go out as one store (16 bytes of float, 8 of bf16) instead of four: the head's
   // 39 MB of logits at 64 rows otherwise arrive as 4-byte pieces 600 KB apart.
   const bool whole = held == 4 && n0 + 3 < N && ((N | n0) & 3) == 0;
+  if (scaled) {   // (the shares were written before the first barrier above, which every wave has passed)
+    float sum = 0.f;
+    for (int w = 0; w < waves; ++w) sum += row_sums[w][col];
+    const float f = rsqrtf(sum / scale.width + scale.eps);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[0][r] *= f;
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + col;
@@ -219,7 +239,8 @@ extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S
 
 // Waves per workgroup and slices of K for a shape.  ``waves`` / ``slices`` 0: chosen here (about one workgroup
 // for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
-// several workgroups to a unit; 8 waves for more than 64 rows; then slices of at least two rounds, at most eight);
+// several workgroups to a unit (10 up to 16 rows, where the heads of the 3B and 72B shapes take 4-17 % less time so);
+// 8 waves for more than 64 rows; then slices of at least two rounds, at most eight);
 // the gate/up epilogue takes one slice.  Returns waves * 256 + slices.
 // Fewer than 8 waves are chosen for the gate/up epilogue at 33-64 rows only: there the tall weights of narrow models
 // (600-1,700 tiles) take 4-17 % less time with one workgroup of 4-7 waves on every unit than with 8 waves on two thirds
@@ -229,7 +250,7 @@ extern "C" int ifx_wide_gemm_plan(int rows, int N, int K, int waves, int slices,
   if (tile_rows < 8 || tile_rows > 16) tile_rows = 16;
   const int n_tiles = (N + tile_rows - 1) / tile_rows, n_rounds = (K + WK - 1) / WK;
   if (waves <= 0) {
-    waves = n_tiles > 256 * MAX_WAVES ? MIN_WAVES : (n_tiles + 255) / 256;
+    waves = n_tiles > 256 * MAX_WAVES ? (rows <= 16 ? 10 : MIN_WAVES) : (n_tiles + 255) / 256;
     if (waves < MIN_WAVES && (rows <= 32 || epi == 0)) waves = MIN_WAVES;   // (products that may be cut into slices of K fill the chip that way)
   }
   const int fewest = rows > MANY_ROWS ? MIN_WAVES : FEW_WAVES;
@@ -250,13 +271,13 @@ extern "C" int ifx_wide_gemm_plan(int rows, int N, int K, int waves, int slices,
 
 template <int MT>
 static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K, int waves,
-                       int slices, int rps, int epi, const int* order, bool add_slices, int tile_rows, hipStream_t s) {
+                       int slices, int rps, int epi, const int* order, bool add_slices, int tile_rows, RowScale scale, hipStream_t s) {
   const int n_tiles = (N + tile_rows - 1) / tile_rows;
   const dim3 grid((n_tiles + waves - 1) / waves, slices);
   const int k_tiles = (K + 63) / 64 * 2;
 #define GO(TO_, EPI_, MINW_)                                                                                       \
   hipLaunchKernelGGL((wide_gemm_kernel<MT, TO_, EPI_, MINW_>), grid, dim3(waves * WAVE), 0, s, (const bf16_t*)x,   \
-                     (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order, tile_rows)
+                     (const bf16_t*)Wt, (TO_*)out, part, M, N, K, k_tiles, rps, order, tile_rows, scale)
 #define GO_ALL(MINW_)                                    \
   if (out_dtype == DT_BF16 && epi == 0) GO(bf16_t, 0, MINW_); \
   else if (out_dtype == DT_BF16) GO(bf16_t, 1, MINW_);        \
@@ -285,8 +306,10 @@ static int launch_wide(const void* x, const void* Wt, void* out, int out_dtype, 
 // order: the row-tile order the copy was written with (or null); tile_rows: the rows to a tile it was written with.
 // ``out`` null with more than one slice: the partial sums are left in ``part`` for a kernel that adds them itself
 // (ifx_add_rmsnorm, ifx_rope_append).
+// scale_pieces [n_scale_pieces][16] (or null), scale_width, scale_eps: a factor per row of x (M <= 16), see RowScale.
 extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_dtype, float* part, int M, int N, int K,
-                             int waves, int slices, int epi, const int* order, int tile_rows, void* stream) {
+                             int waves, int slices, int epi, const int* order, int tile_rows, const float* scale_pieces,
+                             int n_scale_pieces, float scale_width, float scale_eps, void* stream) {
   IFX_REQUIRE(out || slices > 1, "wide_gemm: no output");
   IFX_REQUIRE(tile_rows >= 8 && tile_rows <= 16 && tile_rows % 2 == 0 && (tile_rows == 16 || !order),
               "wide_gemm: %d rows to a tile (8 to 16, even; a tile order goes with 16)", tile_rows);
@@ -300,18 +323,21 @@ extern "C" int ifx_wide_gemm(const void* x, const void* Wt, void* out, int out_d
               waves, FEW_WAVES, MAX_WAVES, slices, n_rounds);
   IFX_REQUIRE(M <= MANY_ROWS || waves == MIN_WAVES, "wide_gemm: %d rows take workgroups of %d waves, not %d", M, MIN_WAVES, waves);
   IFX_REQUIRE(slices == 1 || part, "wide_gemm: %d slices of K need a scratch buffer", slices);
+  IFX_REQUIRE(!scale_pieces || (M <= 16 && n_scale_pieces > 0 && scale_width > 0.f),
+              "wide_gemm: row factors take at most 16 rows (M=%d, %d pieces, width %g)", M, n_scale_pieces, (double)scale_width);
+  const RowScale scale{scale_pieces, n_scale_pieces, scale_width, scale_eps};
   if (M == 0) return 0;
   const int rps = (n_rounds + slices - 1) / slices;
   IFX_REQUIRE((n_rounds + rps - 1) / rps == slices, "wide_gemm: %d rounds do not cut into %d slices (ask ifx_wide_gemm_plan)", n_rounds, slices);
   hipStream_t s = (hipStream_t)stream;
   switch ((M + 15) / 16) {
-    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    case 4: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    case 5: return launch_wide<5>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    case 6: return launch_wide<6>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    case 7: return launch_wide<7>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
-    default: return launch_wide<8>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, s);
+    case 1: return launch_wide<1>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    case 2: return launch_wide<2>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    case 3: return launch_wide<3>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    case 4: return launch_wide<4>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    case 5: return launch_wide<5>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    case 6: return launch_wide<6>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    case 7: return launch_wide<7>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
+    default: return launch_wide<8>(x, Wt, out, out_dtype, part, M, N, K, waves, slices, rps, epi, order, out != nullptr, tile_rows, scale, s);
   }
 }

@@ -437,7 +437,7 @@ def takes_scaled_rows(n_rows: int, weight) -> bool:
         return False
     N, K = weight.rows.shape
     return (weight.rows.dtype == torch.bfloat16 and n_rows <= 16
-            and _small_m_kernel(n_rows, N, K, weight.tiled is not None) == "skinny")
+            and _small_m_kernel(n_rows, N, K, weight.tiled is not None) in ("skinny", "wide"))
 
 
 def adds_into_stream(n_rows: int, weight, norm_weight: torch.Tensor) -> bool:
@@ -544,13 +544,14 @@ def skinny_gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
-def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
+def wide_gemm(x, weight: LinearWeight, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0,
               slices: int = 0, swiglu_pairs: bool = False, keep_slices: bool = False):
     """bfloat16 x [M <= 128, K] times ``weight`` transposed from its tiled copy, x shared through LDS by the waves
-    of a workgroup: the product for 17-64 rows, and for 65-128 rows of weights with few rows.  ``waves`` (4-16 per
-    workgroup, 8 beyond 64 rows; one tile of weight rows each) and ``slices`` of K (added in a fixed order): 0 lets the
-    kernel choose.  With ``keep_slices`` a product of
-    several slices comes back as ``SliceSums``."""
+    of a workgroup: the product for 17-64 rows, for 65-128 rows of weights with few rows, and for 9-16 rows of large
+    tall weights.  ``waves`` (4-16 per workgroup, 8 beyond 64 rows; one tile of weight rows each) and ``slices`` of K
+    (added in a fixed order): 0 lets the kernel choose.  With ``keep_slices`` a product of several slices comes back as
+    ``SliceSums``.  ``x`` may be ``ScaledRows`` (up to 16 rows)."""
+    x, scale = _scale_args(x)
     _check(x, "x", (None, None), torch.bfloat16)
     M, K = x.shape
     N = weight.rows.shape[0]
@@ -568,9 +569,9 @@ def wide_gemm(x: torch.Tensor, weight: LinearWeight, out_dtype: torch.dtype = to
     part = torch.empty((n_slices, M, N), dtype=torch.float32, device=x.device) if n_slices > 1 else None
     keep = keep_slices and n_slices > 1
     out = None if keep else torch.empty((M, N // 2 if swiglu_pairs else N), dtype=out_dtype, device=x.device)
-    _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, I, P),
+    _call(mod, "ifx_wide_gemm", (P, P, P, I, P, I, I, I, I, I, I, P, I, P, I, F, F, P),
           x.data_ptr(), weight.tiled.data_ptr(), _ptr(out), _DT[out_dtype], _ptr(part), M, N, K, n_waves, n_slices,
-          1 if swiglu_pairs else 0, _ptr(weight.order), weight.tile_rows, _stream())
+          1 if swiglu_pairs else 0, _ptr(weight.order), weight.tile_rows, *scale, _stream())
     return SliceSums(part, out_dtype) if keep else out
 
 
@@ -658,10 +659,25 @@ def library_k_slices(M: int, N: int, K: int) -> int:
     return S
 
 
+WIDE_FEW_ROWS_MIN_N = 16384               # rows of a weight (tall enough to fill the chip without slices of K) and ...
+WIDE_FEW_ROWS_MIN_WEIGHT = 100_000_000    # ... its elements from which 9-16 rows take the product that shares x through LDS
+
+
+def _wide_for_few_rows(M: int, N: int, K: int) -> bool:
+    """Whether up to 16 rows go to the product that shares x through LDS instead of the one that splits K over a
+    workgroup's waves.  From 9 rows on the latter reads as much of x from the L2 as of W from memory; for large tall
+    weights, which fill the chip without slices of K, the former then wins (both with the norm's factor per row; gate/up
+    of the 7B shape at 9-16 rows 44.4 against 46.9 us, of the 14B shape 46 against 47-49, 32B 87 against 88-94 from 12
+    rows, 72B 145 against 157-164; the heads of the 7B, 3B and 72B shapes from 12 rows: 177 against 185, 99 against 105
+    and 385 against 414 at 16).  Smaller weights (gate/up of the 3B shape: 20 against 17 us) stay where they are."""
+    return N >= WIDE_FEW_ROWS_MIN_N and N * K >= WIDE_FEW_ROWS_MIN_WEIGHT and M >= (12 if N >= 65536 else 9)
+
+
 def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional[str]:
     """Which of the streaming kernels takes a bfloat16 product of this shape, or None for the library.
     Measured on the 7B shapes: up to 16 rows the product that splits K over the waves of a workgroup (with x
-    staged in LDS for very tall weights such as the head's when there is no tiled copy); from 17 to 64 rows
+    staged in LDS for very tall weights such as the head's when there is no tiled copy; 9-16 rows of large tall
+    weights as from 17 rows, see _wide_for_few_rows); from 17 to 64 rows
     the product that shares x through LDS, which needs the tiled copy (without it, the first kernel up to 32
     rows on narrow weights); from 65 to 128 rows the same product for weights of few rows, whose K it cuts into
     slices to fill the chip where the library has too few output tiles to (down, o and q/k/v of the 7B shape:
@@ -670,6 +686,8 @@ def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional
     if K % 8:
         return None
     if M <= 16:
+        if has_tiled and _wide_for_few_rows(M, N, K):
+            return "wide"
         return "staged" if N >= 65536 and not has_tiled else "skinny"
     if has_tiled and (M <= SKINNY_MAX_M or (M <= WIDE_MAX_M and N <= WIDE_MANY_ROWS_MAX_N)):
         return "wide"

@@ -503,6 +503,40 @@ def test_decode_rows_taken_whole_by_one_workgroup_in_the_engine(name, sharp_fold
         assert rel_err(torch.stack(rows), want) < tol("bfloat16", name), r
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_nine_to_sixteen_rows_through_the_product_that_shares_x(name, sharp_folders, monkeypatch):
+    """Steps of 9-16 rows in which gate/up and the head take the product that shares x through LDS, with the norm's
+    factor per row (large tall weights do by themselves; the tiny models' are made to by lowering the sizes from which
+    it applies to just above their hidden size, so that o and down keep adding into the stream): decode steps of 9-16
+    requests, eager and replayed, and prompt portions of 9-16 tokens, against the plain model."""
+    from inferflux_amd.kernels import ops
+    cfg = TINY[name]
+    folder, V = sharp_folders[name, "bfloat16"], cfg["vocab_size"]
+    assert min(2 * cfg["intermediate_size"], V) > cfg["hidden_size"]
+    monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_N", cfg["hidden_size"] + 1)
+    monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_WEIGHT", 1)
+    used = []
+    real = ops.wide_gemm
+    monkeypatch.setattr(ops, "wide_gemm", lambda x, *a, **k: (used.append((x.shape[0], isinstance(x, ops.ScaledRows))), real(x, *a, **k))[1])
+    runner = load_runner(folder, torch.bfloat16, num_pages=96, max_requests=16)
+    seqs = {f"r{i}": seeded_ids(640 + i, 40 + 5 * i, V) for i in range(16)}
+    heads = {r: 9 + (i % 8) for i, r in enumerate(seqs)}                  # prompts of 9-16 tokens, one step each
+    for rid, ids in seqs.items():
+        runner.add_request(rid)
+        first = runner.step([StepEntry(rid, ids[:heads[rid]], list(range(heads[rid])))]).float().cpu()
+        assert rel_err(first, plain_logits(folder, ids)[:heads[rid]]) < tol("bfloat16", name), rid
+    got = {r: [] for r in seqs}
+    for k in range(21):
+        live = [r for r in seqs if int(r[1:]) < 9 or k < 3 * (16 - int(r[1:]))]           # 16 requests, one fewer every three steps, 9 at the end
+        logits = runner.step([StepEntry(r, [seqs[r][heads[r] + k]], [0]) for r in live]).float().cpu()
+        for i, r in enumerate(live):
+            got[r].append(logits[i].clone())
+    assert any(9 <= m <= 16 and scaled for m, scaled in used) and runner.graph_replays > 5, used[-8:]
+    for r, rows in got.items():
+        want = plain_logits(folder, seqs[r])[heads[r]: heads[r] + len(rows)]
+        assert rel_err(torch.stack(rows), want) < tol("bfloat16", name), r
+
+
 def test_sixty_four_requests_decode_together(sharp_folders, monkeypatch):
     """Sixty-four requests of configuration C (3 kv heads: 192 (row, kv head) pairs, from which on a pair is taken
     whole by one workgroup) decode together after prompts of 3-60 tokens: every request's rows are the plain model's."""

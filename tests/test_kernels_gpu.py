@@ -1367,6 +1367,69 @@ def test_stream_add_and_row_factors_random_shapes(seed):
     assert torch.allclose(act, want_act, rtol=8e-3, atol=1e-3 * max(1.0, float(want_act.abs().max()))), (M, H, K, I, copy)
 
 
+@pytest.mark.parametrize("M", [1, 9, 16])
+@pytest.mark.parametrize("copy", [True, 14, 8])
+def test_row_factors_in_the_product_that_shares_x_through_lds(M, copy):
+    """The product that large tall weights take from 9 rows on applies the norm's factor per row like the other one:
+    every number of waves (the waves' shares of the sums of squares meet in LDS), both outputs, SwiGLU, a width whose
+    pieces do not fill a wave's loads and one that needs several rounds of them."""
+    for H, I, eps in ((200, 300, 1e-3), (4104, 72, 1e-6)):
+        x, w, stream, nw, lw = _stream_case(M, H, 136, 35, copy)
+        s = stream.to(DEV)
+        scaled = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), eps)
+        rows = scaled.rows.cpu().double()
+        factor = torch.rsqrt((s.cpu().double() ** 2).mean(-1, keepdim=True) + eps)
+        g = gen(36)
+        w2 = (torch.randn(I, H, generator=g) * 0.2).to(BF16)
+        lw2 = ops.LinearWeight(w2.to(DEV), ops.tile_weights(w2.to(DEV), tile_rows=lw.tile_rows), None, lw.tile_rows)
+        ref = (rows @ w2.double().t()) * factor
+        big = max(1.0, float(ref.abs().max()))
+        gt, up = ref[:, 0::2], ref[:, 1::2]
+        want_act = gt / (1 + torch.exp(-gt)) * up
+        for waves in (0, 4, 5, 8, 11, 16):
+            got32 = ops.wide_gemm(scaled, lw2, torch.float32, waves=waves, slices=1 if waves else 0).cpu().double()
+            assert torch.allclose(got32, ref, rtol=1e-4, atol=1e-4 * big), (H, waves, float((got32 - ref).abs().max()))
+            got = ops.wide_gemm(scaled, lw2, BF16, waves=waves, slices=1 if waves else 0).cpu().double()
+            assert torch.allclose(got, ref, rtol=8e-3, atol=8e-3 * big), (H, waves)
+            act = ops.wide_gemm(scaled, lw2, BF16, waves=waves, slices=1 if waves else 0, swiglu_pairs=True).cpu().double()
+            assert torch.allclose(act, want_act, rtol=8e-3, atol=1e-3 * max(1.0, float(want_act.abs().max()))), (H, waves)
+        sliced = ops.wide_gemm(scaled, lw2, torch.float32, waves=8, slices=2).cpu().double()      # the factor on partial sums
+        assert torch.allclose(sliced, ref, rtol=1e-4, atol=1e-4 * big)
+        other = ops.skinny_gemm(scaled, lw2.rows, torch.float32, tiled=lw2.tiled, tile_rows=lw2.tile_rows).cpu().double()
+        assert torch.allclose(other, got32, rtol=1e-4, atol=1e-4 * big)                              # the two kernels agree
+    with pytest.raises(ops.KernelError, match="at most 16"):
+        ops.wide_gemm(ops.ScaledRows(torch.zeros(17, H, dtype=BF16, device=DEV), scaled.pieces, H, 1e-3), lw2)
+
+
+def test_few_rows_of_large_tall_weights_take_the_product_that_shares_x(monkeypatch):
+    """The choice between the two products for up to 16 rows, and that ``linear`` / ``linear_swiglu`` follow it with
+    scaled rows (forced here for a small weight by lowering the size from which it applies)."""
+    assert ops._small_m_kernel(9, 37888, 3584, True) == "wide" and ops._small_m_kernel(8, 37888, 3584, True) == "skinny"
+    assert ops._small_m_kernel(16, 37888, 3584, False) == "skinny"                     # no tiled copy
+    assert ops._small_m_kernel(16, 22016, 2048, True) == "skinny"                      # a smaller weight
+    assert ops._small_m_kernel(11, 152064, 3584, True) == "skinny" and ops._small_m_kernel(12, 152064, 3584, True) == "wide"
+    assert ops._small_m_kernel(16, 3584, 18944, True) == "skinny"                      # few rows of W: K would need slices
+    M, H, eps = 12, 136, 1e-5
+    x, w, stream, nw, lw = _stream_case(M, H, 72, 37, True)
+    s = stream.to(DEV)
+    scaled = ops.linear_into_stream(x.to(DEV), lw, s, nw.to(DEV), eps)
+    w2 = (torch.randn(16400, H, generator=gen(38)) * 0.2).to(BF16)
+    lw2 = ops.prepare_linear(w2.to(DEV))
+    before = ops.linear(scaled, lw2, torch.float32)
+    calls = []
+    real = ops.wide_gemm
+    monkeypatch.setattr(ops, "wide_gemm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_WEIGHT", 1)
+    assert ops.takes_scaled_rows(M, lw2)
+    after = ops.linear(scaled, lw2, torch.float32)
+    act = ops.linear_swiglu(scaled, lw2)
+    assert len(calls) == 2
+    big = float(before.abs().max())
+    assert torch.allclose(after, before, rtol=1e-5, atol=1e-5 * big)
+    gt, up = before.double()[:, 0::2], before.double()[:, 1::2]
+    assert torch.allclose(act.double(), gt / (1 + torch.exp(-gt)) * up, rtol=8e-3, atol=1e-3 * big)
+
+
 def test_row_factors_in_the_fused_qkv_product():
     M, d, nH, nKV, K, P, eps = 6, 32, 3, 1, 96, 16, 1e-6
     g = gen(33)
