@@ -51,7 +51,9 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-__device__ __forceinline__ void store4(float* p, floatx4 v) { *(floatx4*)p = v; }
+// (float results are logits, 39 MB at 64 rows of a 152,064-token vocabulary, read again only by the sampler: written
+// with streaming stores they do not push the rows of x out of the L2: the 7B head at 64 rows 206 -> 189 us, 14B 288 -> 263)
+__device__ __forceinline__ void store4(float* p, floatx4 v) { __builtin_nontemporal_store(v, (floatx4*)p); }
 __device__ __forceinline__ void store4(bf16_t* p, floatx4 v) {
   typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
   bf16x4 w;
@@ -238,10 +240,14 @@ extern "C" int ifx_sum_slices(const float* part, void* out, int out_dtype, int S
 }
 
 // Waves per workgroup and slices of K for a shape.  ``waves`` / ``slices`` 0: chosen here (about one workgroup
-// for each of the 256 compute units: as many waves as that takes, or the fewest where even 16 waves leave
-// several workgroups to a unit (10 up to 16 rows, where the heads of the 3B and 72B shapes take 4-17 % less time so);
-// 8 waves for more than 64 rows; then slices of at least two rounds, at most eight);
-// the gate/up epilogue takes one slice.  Returns waves * 256 + slices.
+// for each of the 256 compute units: as many waves as that takes; 8 waves for more than 64 rows; then slices of at
+// least two rounds, at most eight); the gate/up epilogue takes one slice.  Returns waves * 256 + slices.
+// Where even 16 waves leave several workgroups to a unit (the head: 9,500 tiles), what counts is how many tiles the
+// fullest unit gets and how often x is staged: 8, 10 and 14 waves give the fullest unit 40, 40 and 42 tiles, the numbers
+// between 44-48.  Measured on the heads of the 0.5B-72B shapes: 10 waves up to 32 rows (7B 179 -> 172 us at 17 rows, 3B
+// 122 -> 99, 72B 399 -> 374; K below 2,048 gains nothing), 8 beyond, except for K a multiple of 2,048, where 8 waves
+// are markedly slower at every number of rows (3B at 64 rows 131 us with 8 waves, 116 with 14; the tiles a workgroup's
+// waves stream together then lie a power of two apart in memory, which may be why).
 // Fewer than 8 waves are chosen for the gate/up epilogue at 33-64 rows only: there the tall weights of narrow models
 // (600-1,700 tiles) take 4-17 % less time with one workgroup of 4-7 waves on every unit than with 8 waves on two thirds
 // of them; up to 32 rows the form for few waves is the slower one at every shape measured, and the other products
@@ -250,7 +256,8 @@ extern "C" int ifx_wide_gemm_plan(int rows, int N, int K, int waves, int slices,
   if (tile_rows < 8 || tile_rows > 16) tile_rows = 16;
   const int n_tiles = (N + tile_rows - 1) / tile_rows, n_rounds = (K + WK - 1) / WK;
   if (waves <= 0) {
-    waves = n_tiles > 256 * MAX_WAVES ? (rows <= 16 ? 10 : MIN_WAVES) : (n_tiles + 255) / 256;
+    if (n_tiles > 256 * MAX_WAVES) waves = rows <= 32 ? (K >= 2048 ? 10 : MIN_WAVES) : (K % 2048 == 0 ? 14 : MIN_WAVES);
+    else waves = (n_tiles + 255) / 256;
     if (waves < MIN_WAVES && (rows <= 32 || epi == 0)) waves = MIN_WAVES;   // (products that may be cut into slices of K fill the chip that way)
   }
   const int fewest = rows > MANY_ROWS ? MIN_WAVES : FEW_WAVES;
