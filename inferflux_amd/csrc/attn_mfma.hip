@@ -49,7 +49,9 @@ extern "C" int ifx_attn_head_dim() { return D; }
 //
 // STREAM: the keys and values are asked for with streaming loads.  A launch of many rows reads each of them once and
 // gains from it (64 rows over 3,072 keys: 82 -> 76 us); a single row is faster with plain loads (a decode step of one
-// request loses 1.6 % with streaming ones), so the launch chooses by its number of rows.
+// request loses 1.6 % with streaming ones), so the launch chooses by its number of rows.  Pages of more than 16 tokens
+// are read with plain loads always: a tile of 16 keys takes 32 bytes of each 2 P-byte row of V, and the lines must stay
+// in the L2 for the tiles that want the rest (64 rows over 3,100 keys in pages of 64: 141 us streaming, 108 plain).
 constexpr int ROW_STREAM_MIN_ROWS = 8;
 
 template <bool STREAM, typename T>
@@ -336,11 +338,12 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
             scale * 1.4426950408889634f, 0, waves, req_is_row};
   hipStream_t s = (hipStream_t)stream;
+  const bool streaming = n_rows >= ROW_STREAM_MIN_ROWS && page_size == 16;
   if (waves > 0) {
     const int nc = nH / nKV < 16 ? nH / nKV : 16;
     const size_t lds = (size_t)waves * nc * (OPAD + 2) * sizeof(float);
     IFX_REQUIRE(lds <= 65536, "attn_rows: %d waves of %d heads need %zu bytes of LDS", waves, nc, lds);
-    if (n_rows >= ROW_STREAM_MIN_ROWS)
+    if (streaming)
       hipLaunchKernelGGL(attn_rows_whole_kernel<true>, dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
     else
       hipLaunchKernelGGL(attn_rows_whole_kernel<false>, dim3(nKV, n_rows), dim3(WAVE * waves), lds, s, a);
@@ -348,7 +351,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   }
   IFX_REQUIRE(chunk > 0 && chunk % 32 == 0 && max_splits > 0 && max_splits <= 65535, "attn_rows: bad chunk %d / splits %d", chunk, max_splits);
   IFX_REQUIRE(part_o && part_ml, "attn_rows: splits need scratch for their partial results");
-  if (n_rows >= ROW_STREAM_MIN_ROWS) hipLaunchKernelGGL(attn_rows_kernel<true>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
+  if (streaming) hipLaunchKernelGGL(attn_rows_kernel<true>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
   else hipLaunchKernelGGL(attn_rows_kernel<false>, dim3(max_splits, nKV, n_rows), dim3(WAVE), 0, s, a);
   hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, a);
   IFX_LAUNCH_CHECK();
