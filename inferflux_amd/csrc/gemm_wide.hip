@@ -37,6 +37,7 @@ IFX_DEFINE_LAST_ERROR()
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
 
 constexpr int DEPTH = 3;                                           // rounds of W and x on their way
 constexpr int MIN_WAVES = 8, MAX_WAVES = 16;                     // of the kernel's usual form
@@ -187,6 +188,12 @@ __global__ __launch_bounds__((16 * MT > MANY_ROWS || MINW < MIN_WAVES ? MIN_WAVE
       float* dst = part + ((size_t)blockIdx.y * M + m) * N + n0;
       if (whole) {
         *(floatx4*)dst = acc[mt];
+      } else if (((N | n0) & 1) == 0) {   // (tiles of 10 or 14 rows start at even columns: pairs go out as 8 bytes; plain
+                                           //  stores: the kernel that adds the slices reads them next, and streaming ones
+                                           //  cost a decode step of 64 requests 2 %)
+#pragma unroll
+        for (int r = 0; r < 4; r += 2)
+          if (r < held && n0 + r < N) *(floatx2*)(dst + r) = floatx2{acc[mt][r], acc[mt][r + 1]};
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
