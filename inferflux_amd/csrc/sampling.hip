@@ -10,8 +10,9 @@
 // index only within one thread's stride (124-156); here the lowest index always wins a tie.
 //
 // The filters are expressed as thresholds on the unnormalised weight w_i = exp(l_i/T - max):
-// a filter keeps every token whose weight is >= its threshold, found by bisection over the
-// bit patterns of positive floats, so tokens of equal weight are kept or dropped together.
+// a filter keeps every token whose weight is >= its threshold, an exact selection on the bit
+// patterns of the weights (a histogram of their upper bits, then the threshold's bin by its
+// lower bits), so tokens of equal weight are kept or dropped together.
 #include "common.h"
 #include "sampling.h"
 
