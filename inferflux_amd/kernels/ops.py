@@ -663,14 +663,29 @@ WIDE_FEW_ROWS_MIN_N = 16384               # rows of a weight (tall enough to fil
 WIDE_FEW_ROWS_MIN_WEIGHT = 100_000_000    # ... its elements from which 9-16 rows take the product that shares x through LDS
 
 
+def _tile_pairs_fit(N: int) -> bool:
+    """Whether the product that splits K over a workgroup's waves takes the 16-row tiles of a weight of ``N`` rows in
+    pairs (the rule of ifx_skinny_gemm: pairs halve its reads of x, and it takes them where they do not give the fullest
+    of the 256 compute units more tiles than single tiles would)."""
+    n_tiles = -(-N // 16)
+    fullest = lambda nt: -(-(-(-n_tiles // nt)) // 256) * nt
+    return -(-n_tiles // 2) >= 128 and fullest(2) <= fullest(1)
+
+
 def _wide_for_few_rows(M: int, N: int, K: int) -> bool:
     """Whether up to 16 rows go to the product that shares x through LDS instead of the one that splits K over a
     workgroup's waves.  From 9 rows on the latter reads as much of x from the L2 as of W from memory; for large tall
     weights, which fill the chip without slices of K, the former then wins (both with the norm's factor per row; gate/up
     of the 7B shape at 9-16 rows 44.4 against 46.9 us, of the 14B shape 46 against 47-49, 32B 87 against 88-94 from 12
     rows, 72B 145 against 157-164; the heads of the 7B, 3B and 72B shapes from 12 rows: 177 against 185, 99 against 105
-    and 385 against 414 at 16).  Smaller weights (gate/up of the 3B shape: 20 against 17 us) stay where they are."""
-    return N >= WIDE_FEW_ROWS_MIN_N and N * K >= WIDE_FEW_ROWS_MIN_WEIGHT and M >= (12 if N >= 65536 else 9)
+    and 385 against 414 at 16).  Where the other product cannot take tiles in pairs (gate/up of the 14B and 72B shapes)
+    it reads x twice as often and loses from 6 rows on (14B 44.6 against 46.6-47.3 us at 6-8 rows, 72B 143-145 against
+    146-149).  Smaller weights (gate/up of the 3B shape: 20 against 17 us) stay where they are."""
+    if N < WIDE_FEW_ROWS_MIN_N or N * K < WIDE_FEW_ROWS_MIN_WEIGHT:
+        return False
+    if M >= (12 if N >= 65536 else 9):
+        return True
+    return M >= 6 and N < 65536 and not _tile_pairs_fit(N)
 
 
 def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional[str]:

@@ -1409,6 +1409,8 @@ def test_few_rows_of_large_tall_weights_take_the_product_that_shares_x(monkeypat
     assert ops._small_m_kernel(16, 22016, 2048, True) == "skinny"                      # a smaller weight
     assert ops._small_m_kernel(11, 152064, 3584, True) == "skinny" and ops._small_m_kernel(12, 152064, 3584, True) == "wide"
     assert ops._small_m_kernel(16, 3584, 18944, True) == "skinny"                      # few rows of W: K would need slices
+    assert not ops._tile_pairs_fit(27648) and ops._tile_pairs_fit(37888)              # 1,728 tiles: 7 to a unit one by one, 8 in pairs
+    assert ops._small_m_kernel(6, 27648, 5120, True) == "wide" and ops._small_m_kernel(5, 27648, 5120, True) == "skinny"
     M, H, eps = 12, 136, 1e-5
     x, w, stream, nw, lw = _stream_case(M, H, 72, 37, True)
     s = stream.to(DEV)
