@@ -681,11 +681,33 @@ def _wide_for_few_rows(M: int, N: int, K: int) -> bool:
     and 385 against 414 at 16).  Where the other product cannot take tiles in pairs (gate/up of the 14B and 72B shapes)
     it reads x twice as often and loses from 6 rows on (14B 44.6 against 46.6-47.3 us at 6-8 rows, 72B 143-145 against
     146-149).  Smaller weights (gate/up of the 3B shape: 20 against 17 us) stay where they are."""
-    if N < WIDE_FEW_ROWS_MIN_N or N * K < WIDE_FEW_ROWS_MIN_WEIGHT:
+    if N < WIDE_FEW_ROWS_MIN_N:
+        return _few_rows_in_slices(M, N, K)
+    if N * K < WIDE_FEW_ROWS_MIN_WEIGHT:
         return False
     if M >= (12 if N >= 65536 else 9):
         return True
     return M >= 6 and N < 65536 and not _tile_pairs_fit(N)
+
+
+UNEVEN_TILES_MIN_WEIGHT = 64_000_000      # elements from which a weight whose tiles lie unevenly on the chip is cut into slices of K
+
+
+def _few_rows_in_slices(M: int, N: int, K: int) -> bool:
+    """Whether 8-16 rows times a large weight of few rows go to the product that shares x through LDS and cuts K into slices
+    (their sum left to the norm's kernel) instead of the one that adds into the stream itself.  The latter gives a
+    workgroup whole row tiles: 5,120 rows are 320 tiles, two for 64 of the 256 compute units and one for the others,
+    and the product takes as long as one of 8,192 rows (lower tiles do not help it: measured).  Slices of K fill the
+    chip evenly whatever the number of tiles, at the price of the kernel that adds them (5.6 us).  down of the 32B shape
+    (5,120 x 27,648) at 8 / 12 / 16 rows: 55 / 61 / 67 us against 43 + 5.6; of the 14B shape (5,120 x 13,824) 29 / 33 / 36
+    against 24 + 5.6; its o (5,120 x 5,120: 14-17 against 11 + 5.6) is too small to gain, and weights whose tiles lie
+    evenly (3,584 rows in tiles of 14, 8,192 rows) lose.  Decode steps: 8 requests at the 32B shape 13.4 -> 12.9 ms, 16 at
+    the 14B shape 11.5 -> 11.3."""
+    if M < (8 if N * K >= 2 * UNEVEN_TILES_MIN_WEIGHT else 9) or N * K < UNEVEN_TILES_MIN_WEIGHT:   # (8 rows: the smaller weight ties)
+        return False
+    tile_rows = choose_tile_rows(N)
+    n_tiles = -(-N // tile_rows)
+    return N < 0.7 * (-(-n_tiles // COMPUTE_UNITS) * COMPUTE_UNITS * tile_rows)
 
 
 def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional[str]:

@@ -503,18 +503,26 @@ def test_decode_rows_taken_whole_by_one_workgroup_in_the_engine(name, sharp_fold
         assert rel_err(torch.stack(rows), want) < tol("bfloat16", name), r
 
 
+@pytest.mark.parametrize("which", ["tall", "narrow"])
 @pytest.mark.parametrize("name", ["A", "B"])
-def test_nine_to_sixteen_rows_through_the_product_that_shares_x(name, sharp_folders, monkeypatch):
-    """Steps of 9-16 rows in which gate/up and the head take the product that shares x through LDS, with the norm's
-    factor per row (large tall weights do by themselves; the tiny models' are made to by lowering the sizes from which
-    it applies to just above their hidden size, so that o and down keep adding into the stream): decode steps of 9-16
-    requests, eager and replayed, and prompt portions of 9-16 tokens, against the plain model."""
+def test_nine_to_sixteen_rows_through_the_product_that_shares_x(name, which, sharp_folders, monkeypatch):
+    """Steps of 9-16 rows in which products take the kernel that shares x through LDS, against the plain model: decode
+    steps of 9-16 requests, eager and replayed, and prompt portions of 9-16 tokens.  "tall": gate/up and the head, with
+    the norm's factor per row (large tall weights do by themselves; the tiny models' are made to by lowering the sizes
+    from which it applies to just above their hidden size, so that o and down keep adding into the stream).  "narrow":
+    o, down and q/k/v, which then leave the stream add to the norm's kernel (large weights whose tiles lie unevenly on
+    the chip do by themselves; here every weight is made to)."""
     from inferflux_amd.kernels import ops
     cfg = TINY[name]
     folder, V = sharp_folders[name, "bfloat16"], cfg["vocab_size"]
     assert min(2 * cfg["intermediate_size"], V) > cfg["hidden_size"]
-    monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_N", cfg["hidden_size"] + 1)
-    monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_WEIGHT", 1)
+    if which == "tall":
+        monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_N", cfg["hidden_size"] + 1)
+        monkeypatch.setattr(ops, "WIDE_FEW_ROWS_MIN_WEIGHT", 1)
+    else:
+        monkeypatch.setattr(ops, "UNEVEN_TILES_MIN_WEIGHT", 1)
+        lw = ops.prepare_linear(torch.zeros(cfg["hidden_size"], cfg["intermediate_size"], dtype=torch.bfloat16, device="cuda"))
+        assert not ops.adds_into_stream(9, lw, torch.zeros(cfg["hidden_size"], dtype=torch.bfloat16, device="cuda"))
     used = []
     real = ops.wide_gemm
     monkeypatch.setattr(ops, "wide_gemm", lambda x, *a, **k: (used.append((x.shape[0], isinstance(x, ops.ScaledRows))), real(x, *a, **k))[1])
@@ -531,7 +539,7 @@ def test_nine_to_sixteen_rows_through_the_product_that_shares_x(name, sharp_fold
         logits = runner.step([StepEntry(r, [seqs[r][heads[r] + k]], [0]) for r in live]).float().cpu()
         for i, r in enumerate(live):
             got[r].append(logits[i].clone())
-    assert any(9 <= m <= 16 and scaled for m, scaled in used) and runner.graph_replays > 5, used[-8:]
+    assert any(9 <= m <= 16 and (scaled or which == "narrow") for m, scaled in used) and runner.graph_replays > 5, used[-8:]
     for r, rows in got.items():
         want = plain_logits(folder, seqs[r])[heads[r]: heads[r] + len(rows)]
         assert rel_err(torch.stack(rows), want) < tol("bfloat16", name), r

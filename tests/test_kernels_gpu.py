@@ -1411,6 +1411,13 @@ def test_few_rows_of_large_tall_weights_take_the_product_that_shares_x(monkeypat
     assert ops._small_m_kernel(16, 3584, 18944, True) == "skinny"                      # few rows of W: K would need slices
     assert not ops._tile_pairs_fit(27648) and ops._tile_pairs_fit(37888)              # 1,728 tiles: 7 to a unit one by one, 8 in pairs
     assert ops._small_m_kernel(6, 27648, 5120, True) == "wide" and ops._small_m_kernel(5, 27648, 5120, True) == "skinny"
+    # large weights of few rows whose 16-row tiles lie unevenly on the 256 units (5,120 rows: 320 tiles) are cut into slices of K
+    assert ops._small_m_kernel(8, 5120, 27648, True) == "wide" and ops._small_m_kernel(7, 5120, 27648, True) == "skinny"
+    assert ops._small_m_kernel(9, 5120, 13824, True) == "wide" and ops._small_m_kernel(8, 5120, 13824, True) == "skinny"
+    assert ops._small_m_kernel(16, 5120, 5120, True) == "skinny" and ops._small_m_kernel(16, 8192, 29568, True) == "skinny"
+    lw = ops.LinearWeight(torch.empty(5120, 27648, dtype=BF16, device="meta"), torch.empty(1, device="meta"), None, 16)
+    nw = torch.empty(5120, dtype=BF16, device="meta")
+    assert ops.adds_into_stream(7, lw, nw) and not ops.adds_into_stream(8, lw, nw)
     M, H, eps = 12, 136, 1e-5
     x, w, stream, nw, lw = _stream_case(M, H, 72, 37, True)
     s = stream.to(DEV)
