@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restri
   float x[NV][4];
   float ss = 0.f;
   // Every load that does not depend on another goes out before the first is used: the row and the delta (or
-  // its first slice) for all of the thread's elements, then the further slices four at a time for all elements.
+  // its first slice) for all of the thread's elements, then the further slices, up to seven at a time, for all elements.
   // With the elements outermost a row of 8 slices cost a dozen trips to the L2 one after the other.
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
@@ -220,10 +220,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restri
       if (i < H) load4<TD>(dl + i, d4[v]);
       else d4[v][0] = d4[v][1] = d4[v][2] = d4[v][3] = 0.f;
     }
-    for (int s0 = 1; s0 < n_slices; s0 += 4) {   // partial sums, added in slice order
-      float p4[4][NV][4];
+    constexpr int AT_ONCE = NV <= 4 ? 7 : 4;   // (the products cut K into at most eight slices: one trip for all of them)
+    for (int s0 = 1; s0 < n_slices; s0 += AT_ONCE) {   // partial sums, added in slice order
+      float p4[AT_ONCE][NV][4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < AT_ONCE; ++u)
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
           const int i = 4 * (threadIdx.x + 256 * v);
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_slices_kernel(float* __restri
           else p4[u][v][0] = p4[u][v][1] = p4[u][v][2] = p4[u][v][3] = 0.f;
         }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < AT_ONCE; ++u)
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
